@@ -1,0 +1,160 @@
+#!/usr/bin/env python3
+"""Benchmark of the EXL3 trellis GEMV hot path on one MI355X.
+
+Workload (BASELINE.json configs[1] at the bit rate the metric is quoted on): the
+dense 27B-shaped decode linear set at batch 1, 4 bpw, mul1 codebook — q_proj
+5120x6144, k/v_proj 5120x1024, o_proj 6144x5120, gate/up 5120x17408, down
+17408x5120 — fp16 activations N(0,1), uniform random trellis words, suh/svh
+random signs times lognormal(0,0.1).  One step = the seven linears of one layer,
+each through berth_exl3_linear (one fused kernel launch per linear).  Steps rotate
+over `--layers` distinct weight sets (default 8 = 1.36 GB) so that reads come
+from HBM, not from the 256 MB memory-side cache.  Inputs are resident in HBM
+before the timed region.
+
+value = algorithmic bytes of the step / time, in GB/s (the metric's unit);
+roofline.achieved is the same quantity for the dominant kernel (all seven
+launches are the one GEMV kernel), against the 8 TB/s HBM peak.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+ORDER = ["q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"]
+OUT_FP32 = {"q_proj": False, "k_proj": False, "v_proj": False, "o_proj": True,
+            "gate_proj": False, "up_proj": False, "down_proj": True}
+
+
+def linear_bytes(K, N, bits, m, out_bytes):
+    """Algorithmic bytes of one linear on m rows: packed trellis + suh + svh +
+    activation in + output out."""
+    return K * N * bits // 8 + 2 * K + 2 * N + 2 * m * K + out_bytes * m * N
+
+
+def cpu_baseline(bits: int, seconds: float):
+    """The CPU oracle's decode-on-the-fly GEMV (a port: the reference has no CPU
+    trellis path), timed on this host's cores on a bounded sample."""
+    from berth_amd import synth
+    from oracle import oracle as O
+    K, N = synth.SHAPES_27B["q_proj"]
+    tr, suh, svh = synth.linear(11, K, N, bits)
+    x = synth.activations(12, 1, K)
+    O.gemv_fused(x, tr, suh, svh, K, N, bits, 2, out_fp32=False)       # warm (builds the state table)
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        O.gemv_fused(x, tr, suh, svh, K, N, bits, 2, out_fp32=False)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt >= seconds or reps >= 200:
+            break
+    nbytes = linear_bytes(K, N, bits, 1, 2) * reps
+    return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": O.num_threads(), "kind": "port",
+            "sample": f"{reps} x q_proj {K}x{N} {bits} bpw batch-1 decode-on-the-fly GEMV in {dt:.1f} s "
+                      f"({K * N * reps / dt / 1e6:.0f} M weights/s)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--layers", type=int, default=8)
+    ap.add_argument("--bits", type=int, default=4)
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path is single-GPU by design); "
+              "--gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from berth_amd import kernels as Kn
+    from berth_amd import synth
+    from berth_amd.device import Exl3Linear, Gpu
+    from berth_amd.kernels import OutDtype
+
+    Kn.load()
+    gpu = Gpu(0)
+    bits = args.bits
+
+    layers = []
+    for li in range(args.layers):
+        lin = {}
+        for j, name in enumerate(ORDER):
+            K, N = synth.SHAPES_27B[name]
+            tr, suh, svh = synth.linear(1000 * li + 10 * j, K, N, bits)
+            lin[name] = Exl3Linear(gpu, f"layers.{li}.{name}", tr, suh, svh)
+        layers.append(lin)
+
+    xin = {K: gpu.upload(synth.activations(5, 1, K).view(np.uint16)) for K in (5120, 6144, 17408)}
+    outs = {name: torch.zeros(synth.SHAPES_27B[name][1], dtype=torch.float32 if OUT_FP32[name] else torch.float16,
+                              device=gpu.device) for name in ORDER}
+
+    step_bytes = sum(linear_bytes(*synth.SHAPES_27B[n], bits, 1, 4 if OUT_FP32[n] else 2) for n in ORDER)
+
+    def step(i):
+        lin = layers[i % len(layers)]
+        for name in ORDER:
+            l = lin[name]
+            l.forward(gpu, xin[l.size_k], outs[name], OutDtype.F32 if OUT_FP32[name] else OutDtype.F16)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(args.steps):
+        step(i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ev_ms = e0.elapsed_time(e1)
+    ms_per_step = wall_ms / args.steps
+    value = step_bytes * args.steps / (wall_ms * 1e-3) / 1e9
+
+    launches = args.steps * len(ORDER)
+    avg_launch_us = ev_ms * 1e3 / launches
+    achieved = step_bytes * args.steps / (ev_ms * 1e-3) / 1e9
+
+    line = {
+        "metric": "trellis GEMV HBM GB/s at 4 bpw, batch 1",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": f"27B-shaped decode linear set (q,k,v,o,gate,up,down), batch 1, {bits} bpw, mul1",
+                   "layers_rotated": len(layers), "bytes_per_step": step_bytes,
+                   "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": Kn.last_launch().split(" grid=")[0],
+                     "avg_launch_us": round(avg_launch_us, 3),
+                     "bytes_per_launch": step_bytes // len(ORDER)},
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(bits, args.cpu_seconds)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,60 @@
+"""Compile the HIP sources under berth_amd/csrc for gfx950 into in-tree shared
+libraries (berth_amd/lib/*.so).  hipcc cross-compiles without a GPU."""
+from __future__ import annotations
+
+import concurrent.futures as cf
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "lib")
+OBJ = os.path.join(HERE, "lib", "obj")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# packed fp32 VALU ops are switched off for every device compilation
+# no implicit mul+add fusion: the Hadamard butterflies must round like the CPU oracle
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-Wno-unused-result", "-Wno-unknown-warning-option"]
+
+LIBRARIES = {
+    "libberth_kernels_hip.so": ["api.hip", "exl3_gemv.hip", "exl3_gemm.hip",
+                                "exl3_reconstruct.hip", "elementwise.hip", "moe.hip"],
+    "libberth_hip.so": ["berth_hip.hip"],
+}
+
+
+def _compile(src: str) -> str:
+    obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+    cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{r.stderr[-4000:]}")
+    return obj
+
+
+def build_all(jobs: int = 8, only: str | None = None) -> list[str]:
+    os.makedirs(OBJ, exist_ok=True)
+    libs = {k: v for k, v in LIBRARIES.items() if only in (None, k)}
+    sources = sorted({s for v in libs.values() for s in v if os.path.exists(os.path.join(CSRC, s))})
+    with cf.ThreadPoolExecutor(max_workers=min(jobs, 16)) as ex:
+        objs = dict(zip(sources, ex.map(_compile, sources)))
+    built = []
+    for name, srcs in libs.items():
+        have = [objs[s] for s in srcs if s in objs]
+        if not have:
+            continue
+        out = os.path.join(LIB, name)
+        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *have, "-o", out]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"link failed for {name}:\n{r.stderr[-4000:]}")
+        built.append(out)
+    return built
+
+
+if __name__ == "__main__":
+    for path in build_all(only=sys.argv[1] if len(sys.argv) > 1 else None):
+        print("built", path)

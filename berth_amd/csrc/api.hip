@@ -1,0 +1,242 @@
+// C-ABI entry points of libberth_kernels_hip.so: validation, dispatch, and the
+// thread-local error / launch strings.  Validation order and messages follow
+// crates/berth-kernels/csrc/linear.cu:224-235 and
+// crates/berth-kernels/csrc/prefill_lin/linear.cu:248-266 so that the host-only
+// tests of crates/berth-kernels/src/lib.rs:235-319 read the same here.
+#include "launch.h"
+
+#include "../../include/berth_kernels_hip.h"
+
+#include <mutex>
+
+namespace berth {
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_ws_mu;
+Workspace g_ws[kMaxDevices];
+}  // namespace
+
+Workspace& workspace_for_current_device()
+{
+    int device = 0;
+    hip_ok(hipGetDevice(&device), "hipGetDevice");
+    if (device < 0 || device >= kMaxDevices) throw std::runtime_error("device index out of range");
+    std::lock_guard<std::mutex> lock(g_ws_mu);
+    Workspace& ws = g_ws[device];
+    if (ws.device < 0) {
+        void* partials = nullptr;
+        void* counters = nullptr;
+        hip_ok(hipMalloc(&partials, kPartialBytes), "split-K workspace");
+        hip_ok(hipMalloc(&counters, kCounters * sizeof(unsigned)), "split-K counters");
+        hip_ok(hipMemset(counters, 0, kCounters * sizeof(unsigned)), "split-K counter memset");
+        int cus = 0;
+        hip_ok(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device), "multiProcessorCount");
+        ws.partials = (float*)partials;
+        ws.counters = (unsigned*)counters;
+        ws.cu_count = cus;
+        ws.device = device;
+    }
+    return ws;
+}
+
+namespace {
+
+thread_local std::string g_exl3_err, g_exl3_launch;
+thread_local std::string g_prefill_err, g_prefill_launch;
+thread_local std::string g_ops_err, g_ops_launch;
+
+void check_linear(const char* who, const LinearArgs& a)
+{
+    const std::string w(who);
+    if (!a.a || !a.trellis || !a.c || !a.suh || !a.a_had || !a.svh)
+        throw std::runtime_error(w + ": null device pointer");
+}
+
+void check_shape(const char* who, const LinearArgs& a)
+{
+    const std::string w(who);
+    if (a.k_bits < 1 || a.k_bits > 8) throw std::runtime_error(w + ": K must be in 1..=8");
+    if (a.codebook < 0 || a.codebook > 2)
+        throw std::runtime_error(w + ": codebook must be 0 (default), 1 (mcg), or 2 (mul1)");
+    if (a.size_k % 16 != 0) throw std::runtime_error(w + ": size_k must be a multiple of 16");
+    if (a.size_n % 128 != 0) throw std::runtime_error(w + ": size_n must be a multiple of 128");
+    if (a.size_k % 128 != 0)
+        throw std::runtime_error(w + ": size_k must be a multiple of 128 (one Hadamard block)");
+}
+
+std::string dispatch_linear(const LinearArgs& a)
+{
+    if (a.size_m <= 8) return launch_gemv(a);
+    return launch_gemm(a);
+}
+
+}  // namespace
+}  // namespace berth
+
+using namespace berth;
+
+extern "C" int berth_exl3_linear(const void* a, const void* trellis, void* c, const void* suh,
+                                 void* a_had, const void* svh, int size_m, int size_k, int size_n,
+                                 int k_bits, int codebook, int out_fp32, void* stream)
+{
+    try {
+        g_exl3_err.clear();
+        g_exl3_launch.clear();
+        LinearArgs args{a, trellis, c, suh, a_had, svh, size_m, size_k, size_n,
+                        k_bits, codebook, out_fp32 ? 1 : 0, (hipStream_t)stream};
+        check_linear("exl3 linear", args);
+        if (size_m < 1 || size_k < 1 || size_n < 1)
+            throw std::runtime_error("exl3 linear: sizes must be positive");
+        check_shape("exl3 linear", args);
+        g_exl3_launch = dispatch_linear(args);
+        return 0;
+    } catch (const std::exception& err) {
+        g_exl3_err = err.what();
+        g_exl3_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
+extern "C" const char* berth_exl3_last_error(void) { return g_exl3_err.c_str(); }
+extern "C" const char* berth_exl3_last_launch(void) { return g_exl3_launch.c_str(); }
+
+extern "C" int berth_device_cc(int device)
+{
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) != hipSuccess) return -1;
+    // gcnArchName is "gfx950:sramecc+:xnack-"
+    int cc = 0;
+    for (const char* p = prop.gcnArchName + 3; *p >= '0' && *p <= '9'; ++p) cc = cc * 10 + (*p - '0');
+    return cc;
+}
+
+extern "C" int berth_device_sms(int device)
+{
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return -1;
+    return cus;
+}
+
+extern "C" int berth_prefill_exl3_linear(const void* a, const void* trellis, void* c,
+                                         const void* suh, void* a_had, const void* svh,
+                                         void* w_scratch, int size_m, int size_k, int size_n,
+                                         int k_bits, int codebook, int c_fp32, void* stream)
+{
+    try {
+        g_prefill_err.clear();
+        g_prefill_launch.clear();
+        LinearArgs args{a, trellis, c, suh, a_had, svh, size_m, size_k, size_n,
+                        k_bits, codebook, c_fp32 ? 1 : 0, (hipStream_t)stream};
+        check_linear("prefill exl3 linear", args);
+        if (size_m < 2)
+            throw std::runtime_error("prefill exl3 linear: size_m must be > 1 (m = 1 is exl3_linear)");
+        if (size_k < 1 || size_n < 1)
+            throw std::runtime_error("prefill exl3 linear: sizes must be positive");
+        check_shape("prefill exl3 linear", args);
+        if (size_m > 144 && !w_scratch)
+            throw std::runtime_error(
+                "prefill exl3 linear: w_scratch (fp16, size_k * min(size_n, 32768)) is required when rows > 144");
+        g_prefill_launch = dispatch_linear(args);
+        return 0;
+    } catch (const std::exception& err) {
+        g_prefill_err = err.what();
+        g_prefill_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
+extern "C" int berth_prefill_hgemm(const void* a, const void* b, void* c, int size_m, int size_k,
+                                   int size_n, int ldc, int c_fp32, void* stream)
+{
+    try {
+        g_prefill_err.clear();
+        g_prefill_launch.clear();
+        if (!a || !b || !c) throw std::runtime_error("prefill hgemm: null device pointer");
+        if (size_m < 1 || size_k < 1 || size_n < 1 || ldc < size_n)
+            throw std::runtime_error("prefill hgemm: bad shape");
+        g_prefill_launch = launch_hgemm(a, b, c, size_m, size_k, size_n, ldc, c_fp32 ? 1 : 0, (hipStream_t)stream);
+        return 0;
+    } catch (const std::exception& err) {
+        g_prefill_err = err.what();
+        g_prefill_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
+extern "C" int berth_prefill_reconstruct(void* unpacked, const void* packed, int size_k, int slice_n,
+                                         int full_n, int n_offset, int k_bits, int codebook,
+                                         void* stream)
+{
+    try {
+        g_prefill_err.clear();
+        g_prefill_launch.clear();
+        if (!unpacked || !packed) throw std::runtime_error("prefill reconstruct: null device pointer");
+        if (size_k < 16 || slice_n < 128 || full_n < 128)
+            throw std::runtime_error("prefill reconstruct: sizes must be positive");
+        if (k_bits < 1 || k_bits > 8) throw std::runtime_error("prefill reconstruct: K must be in 1..=8");
+        if (codebook < 0 || codebook > 2) throw std::runtime_error("prefill reconstruct: codebook must be 0, 1, or 2");
+        if (size_k % 16) throw std::runtime_error("prefill reconstruct: K must be a multiple of 16");
+        if (slice_n % 128) throw std::runtime_error("prefill reconstruct: slice N must be a multiple of 128");
+        if (full_n % 16) throw std::runtime_error("prefill reconstruct: full N must be a multiple of 16");
+        if (n_offset % 128) throw std::runtime_error("prefill reconstruct: n_offset must be a multiple of 128");
+        if (n_offset < 0 || n_offset + slice_n > full_n)
+            throw std::runtime_error("prefill reconstruct: slice exceeds the trellis");
+        g_prefill_launch = launch_reconstruct(unpacked, packed, size_k, slice_n, full_n, n_offset,
+                                              k_bits, codebook, (hipStream_t)stream);
+        return 0;
+    } catch (const std::exception& err) {
+        g_prefill_err = err.what();
+        g_prefill_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
+extern "C" int berth_prefill_had_r_128(const void* input, void* output, const void* scale,
+                                       int pre_scale, int rows, int cols, int fp32, void* stream)
+{
+    try {
+        g_prefill_err.clear();
+        g_prefill_launch.clear();
+        if (!input || !output) throw std::runtime_error("prefill had_r_128: null device pointer");
+        if (cols < 128 || cols % 128)
+            throw std::runtime_error("prefill reconstruct: had columns must be a multiple of 128");
+        if (rows < 1) throw std::runtime_error("prefill had_r_128: rows must be positive");
+        g_prefill_launch = launch_had_r_128(input, output, scale, pre_scale, rows, cols, fp32 ? 1 : 0,
+                                            (hipStream_t)stream);
+        return 0;
+    } catch (const std::exception& err) {
+        g_prefill_err = err.what();
+        g_prefill_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
+extern "C" const char* berth_prefill_last_error(void) { return g_prefill_err.c_str(); }
+extern "C" const char* berth_prefill_last_launch(void) { return g_prefill_launch.c_str(); }
+
+extern "C" int berth_ops_silu_mul(const void* gate, const void* up, void* out, int64_t numel,
+                                  float act_limit, void* stream)
+{
+    try {
+        g_ops_err.clear();
+        g_ops_launch.clear();
+        if (!gate || !up || !out) throw std::runtime_error("silu_mul: null device pointer");
+        if (numel < 2 || (numel & 1)) throw std::runtime_error("silu_mul: numel must be positive and even");
+        g_ops_launch = launch_silu_mul(gate, up, out, numel, act_limit, (hipStream_t)stream);
+        return 0;
+    } catch (const std::exception& err) {
+        g_ops_err = err.what();
+        g_ops_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
+extern "C" const char* berth_ops_last_error(void) { return g_ops_err.c_str(); }
+extern "C" const char* berth_ops_last_launch(void) { return g_ops_launch.c_str(); }

@@ -1,0 +1,60 @@
+// Internal C++ interface between the C-ABI entry points and the kernel launchers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <stdexcept>
+#include <string>
+
+namespace berth {
+
+inline void hip_ok(hipError_t e, const char* what)
+{
+    if (e != hipSuccess)
+        throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+// Per-device scratch owned by the library, allocated on first use and kept for
+// the life of the process: split-K partial sums and their arrival counters
+// (the role of the fixed 16 MiB workspace of
+// crates/berth-kernels/csrc/int8_sq.cu:20-47).
+struct Workspace {
+    float* partials = nullptr;      // kPartialBytes
+    unsigned* counters = nullptr;   // kCounters entries, zero between launches
+    int device = -1;
+    int cu_count = 0;
+};
+constexpr size_t kPartialBytes = 16u << 20;
+constexpr int kCounters = 65536;
+Workspace& workspace_for_current_device();
+
+struct LinearArgs {
+    const void* a;
+    const void* trellis;
+    void* c;
+    const void* suh;
+    void* a_had;
+    const void* svh;
+    int size_m, size_k, size_n, k_bits, codebook, out_fp32;
+    hipStream_t stream;
+};
+
+// rows 1..8: VALU dot-product kernel.  Returns the launch description.
+std::string launch_gemv(const LinearArgs& args);
+// any row count: fp16 MFMA kernel (rows padded to 32 inside the kernel).
+std::string launch_gemm(const LinearArgs& args);
+// trellis -> fp16 [K][slice_n] (row stride slice_n), columns n_offset.. of a
+// [K][full_n] weight
+std::string launch_reconstruct(void* unpacked, const void* packed, int size_k, int slice_n,
+                               int full_n, int n_offset, int k_bits, int codebook,
+                               hipStream_t stream);
+// per row, per 128 columns: Hadamard with pre- or post-scale
+std::string launch_had_r_128(const void* in, void* out, const void* scale, int pre_scale,
+                             int rows, int cols, int fp32, hipStream_t stream);
+std::string launch_silu_mul(const void* gate, const void* up, void* out, int64_t numel,
+                            float act_limit, hipStream_t stream);
+std::string launch_hgemm(const void* a, const void* b, void* c, int m, int k, int n, int ldc,
+                         int c_fp32, hipStream_t stream);
+
+}  // namespace berth

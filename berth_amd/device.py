@@ -1,0 +1,159 @@
+"""Host-side owners of device buffers for the EXL3 linear path, mirroring
+crates/berth-engine/src/device.rs:14-367 (`Gpu`, `Exl3Linear`, `RowScratch`) and
+crates/berth-engine/src/mlp.rs:25-334 (`MlpLayer`).  torch is used for device
+memory and the stream only; every computation goes through the C ABI.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from . import kernels as K
+from .kernels import Codebook, OutDtype
+
+MAX_RECONSTRUCT_N = 32768   # crates/berth-engine/src/device.rs:193
+
+
+class InputError(ValueError):
+    """crates/berth-engine `Error::Input`."""
+
+
+class Gpu:
+    """Device 0 and the stream every launch goes on (device.rs:14-43)."""
+
+    def __init__(self, device: int = 0):
+        if not torch.cuda.is_available():
+            raise RuntimeError("no HIP device")
+        self.device = torch.device("cuda", device)
+        torch.cuda.set_device(self.device)
+        self.stream = torch.cuda.current_stream(self.device)
+        self.sm_count = K.device_sms(device)
+
+    def raw_stream(self):
+        return self.stream.cuda_stream or None
+
+    def zeroed(self, nbytes: int) -> torch.Tensor:
+        return torch.zeros(nbytes, dtype=torch.uint8, device=self.device)
+
+    def upload(self, array: np.ndarray) -> torch.Tensor:
+        a = np.ascontiguousarray(array)
+        if a.dtype == np.uint16:
+            a = a.view(np.int16)
+        return torch.from_numpy(a).to(self.device)
+
+    def synchronize(self):
+        torch.cuda.synchronize(self.device)
+
+
+def ptr(t: torch.Tensor) -> int:
+    return t.data_ptr()
+
+
+def _out_dtype(out: OutDtype):
+    return torch.float32 if out == OutDtype.F32 else torch.float16
+
+
+class RowScratch:
+    """Scratch shared by every linear of a prefill chunk (device.rs:176-212)."""
+
+    def __init__(self, gpu: Gpu, max_rows: int, max_k: int, max_n: int):
+        self.a_had = torch.zeros(max_rows * max_k, dtype=torch.float16, device=gpu.device)
+        self.weight = torch.zeros(max_k * min(max_n, MAX_RECONSTRUCT_N), dtype=torch.float16,
+                                  device=gpu.device)
+        self.max_rows, self.max_k, self.max_n = max_rows, max_k, max_n
+
+
+class Exl3Linear:
+    """One EXL3 linear on the device: trellis, fp16 Hadamard scales, and the
+    fp16 scratch the kernel writes the rotated input to (device.rs:77-367)."""
+
+    def __init__(self, gpu: Gpu, prefix: str, trellis: np.ndarray, suh: np.ndarray, svh: np.ndarray,
+                 codebook: Codebook = Codebook.MUL1):
+        if trellis.ndim != 3 or trellis.shape[2] % 16:
+            raise InputError(f"{prefix}: trellis must be (K/16, N/16, 16*bits)")
+        self.prefix = prefix
+        self.k_bits = trellis.shape[2] // 16
+        self.size_k = int(suh.size)
+        self.size_n = int(svh.size)
+        if trellis.shape[0] * 16 != self.size_k or trellis.shape[1] * 16 != self.size_n:
+            raise InputError(f"{prefix}: trellis shape does not match suh / svh")
+        self.codebook = codebook
+        self.trellis = gpu.upload(trellis.view(np.uint16))
+        self.suh = gpu.upload(suh.view(np.uint16))
+        self.svh = gpu.upload(svh.view(np.uint16))
+        self.a_had = torch.zeros(self.size_k, dtype=torch.float16, device=gpu.device)
+
+    def trellis_bytes(self) -> int:
+        return self.trellis.numel() * 2
+
+    # device.rs:127-165
+    def forward(self, gpu: Gpu, a: torch.Tensor, c: torch.Tensor, out: OutDtype) -> None:
+        if a.numel() * a.element_size() < self.size_k * 2 or \
+           c.numel() * c.element_size() < self.size_n * (4 if out == OutDtype.F32 else 2):
+            raise InputError(f"{self.prefix}: buffer too small")
+        K.exl3_linear(ptr(a), ptr(self.trellis), ptr(c), ptr(self.suh), ptr(self.a_had), ptr(self.svh),
+                      1, self.size_k, self.size_n, self.k_bits, self.codebook, out, gpu.raw_stream())
+
+    # device.rs:210-272
+    def forward_rows(self, gpu: Gpu, scratch: RowScratch, a: torch.Tensor, c: torch.Tensor, rows: int,
+                     out: OutDtype) -> None:
+        if rows < 2:
+            raise InputError(f"{self.prefix}: forward_rows needs rows > 1")
+        if rows > scratch.max_rows or self.size_k > scratch.max_k or self.size_n > scratch.max_n:
+            raise InputError(f"{self.prefix}: {rows} x {self.size_k} x {self.size_n} exceeds the row scratch")
+        if a.numel() * a.element_size() < rows * self.size_k * 2 or \
+           c.numel() * c.element_size() < rows * self.size_n * (4 if out == OutDtype.F32 else 2):
+            raise InputError(f"{self.prefix}: buffer too small")
+        weight = ptr(scratch.weight) if rows > 144 else None
+        K.prefill_lin.exl3_linear(ptr(a), ptr(self.trellis), ptr(c), ptr(self.suh), ptr(scratch.a_had),
+                                  ptr(self.svh), weight, rows, self.size_k, self.size_n, self.k_bits,
+                                  self.codebook, out, gpu.raw_stream())
+
+    # device.rs:288-366
+    def forward_n(self, gpu: Gpu, a_had: torch.Tensor, a: torch.Tensor, c: torch.Tensor, rows: int,
+                  out: OutDtype) -> None:
+        if rows == 1:
+            return self.forward(gpu, a, c, out)
+        if rows == 0 or rows > 144:
+            raise InputError(f"{self.prefix}: forward_n rows {rows} are outside 1..=144")
+        need = rows * self.size_k * 2
+        if a_had.numel() * a_had.element_size() < need or a.numel() * a.element_size() < need or \
+           c.numel() * c.element_size() < rows * self.size_n * (4 if out == OutDtype.F32 else 2):
+            raise InputError(f"{self.prefix}: buffer too small")
+        if self.k_bits == 6:
+            K.exl3_linear(ptr(a), ptr(self.trellis), ptr(c), ptr(self.suh), ptr(a_had), ptr(self.svh),
+                          rows, self.size_k, self.size_n, self.k_bits, self.codebook, out, gpu.raw_stream())
+        else:
+            K.prefill_lin.exl3_linear(ptr(a), ptr(self.trellis), ptr(c), ptr(self.suh), ptr(a_had),
+                                      ptr(self.svh), None, rows, self.size_k, self.size_n, self.k_bits,
+                                      self.codebook, out, gpu.raw_stream())
+
+
+class MlpLayer:
+    """gate -> up -> silu_mul -> down (mlp.rs:118-150 decode, :219-303 prefill)."""
+
+    def __init__(self, gpu: Gpu, gate: Exl3Linear, up: Exl3Linear, down: Exl3Linear, max_rows: int = 1):
+        self.gate, self.up, self.down = gate, up, down
+        self.hidden = gate.size_k
+        self.intermediate = gate.size_n
+        if up.size_k != self.hidden or up.size_n != self.intermediate or \
+           down.size_k != self.intermediate or down.size_n != self.hidden:
+            raise InputError("mlp: projection shapes do not chain")
+        self.g = torch.zeros(max_rows * self.intermediate, dtype=torch.float16, device=gpu.device)
+        self.u = torch.zeros(max_rows * self.intermediate, dtype=torch.float16, device=gpu.device)
+
+    def forward(self, gpu: Gpu, x: torch.Tensor, y: torch.Tensor) -> None:
+        """x fp16 [hidden] -> y fp32 [hidden]."""
+        self.gate.forward(gpu, x, self.g, OutDtype.F16)
+        self.up.forward(gpu, x, self.u, OutDtype.F16)
+        K.ops.silu_mul(ptr(self.g), ptr(self.u), ptr(self.u), self.intermediate, 0.0, gpu.raw_stream())
+        self.down.forward(gpu, self.u, y, OutDtype.F32)
+
+    def prefill(self, gpu: Gpu, scratch: RowScratch, x: torch.Tensor, y: torch.Tensor, rows: int) -> None:
+        """x fp16 [rows][hidden] -> y fp32 [rows][hidden]."""
+        if rows * self.intermediate > self.g.numel():
+            raise InputError("mlp: rows exceed the layer scratch")
+        self.gate.forward_rows(gpu, scratch, x, self.g, rows, OutDtype.F16)
+        self.up.forward_rows(gpu, scratch, x, self.u, rows, OutDtype.F16)
+        K.ops.silu_mul(ptr(self.g), ptr(self.u), ptr(self.u), rows * self.intermediate, 0.0, gpu.raw_stream())
+        self.down.forward_rows(gpu, scratch, self.u, y, rows, OutDtype.F32)

@@ -1,0 +1,148 @@
+"""ctypes binding of libberth_kernels_hip.so, shaped like the reference's
+`berth_kernels` crate (crates/berth-kernels/src/{lib,prefill_lin,ops}.rs): raw
+device addresses in, a launch error raised with the shim's message, and
+`last_launch()` naming the kernel that ran.
+
+There is no fallback: if the HIP library is missing every call raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import enum
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libberth_kernels_hip.so")
+
+
+class LaunchError(RuntimeError):
+    """crates/berth-kernels/src/error.rs `Error::Launch`."""
+
+
+class Codebook(enum.IntEnum):
+    """crates/berth-kernels/src/lib.rs:54-63."""
+    DEFAULT = 0
+    MCG = 1
+    MUL1 = 2
+
+
+class OutDtype(enum.IntEnum):
+    """crates/berth-kernels/src/lib.rs:69-85 (`as_c`)."""
+    F16 = 0
+    F32 = 1
+
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise LaunchError(
+                f"{LIB_PATH} is missing: build it with `python -m berth_amd.build` "
+                "(there is no CPU fallback)")
+        L = C.CDLL(LIB_PATH)
+        vp, ci = C.c_void_p, C.c_int
+        L.berth_exl3_linear.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
+        L.berth_prefill_exl3_linear.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
+        L.berth_prefill_hgemm.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, vp]
+        L.berth_prefill_reconstruct.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, vp]
+        L.berth_prefill_had_r_128.argtypes = [vp, vp, vp, ci, ci, ci, ci, vp]
+        L.berth_ops_silu_mul.argtypes = [vp, vp, vp, C.c_int64, C.c_float, vp]
+        for name in ("berth_exl3_last_error", "berth_exl3_last_launch", "berth_prefill_last_error",
+                     "berth_prefill_last_launch", "berth_ops_last_error", "berth_ops_last_launch"):
+            getattr(L, name).restype = C.c_char_p
+        L.berth_device_cc.argtypes = [ci]
+        L.berth_device_sms.argtypes = [ci]
+        _lib = L
+    return _lib
+
+
+def _s(b) -> str:
+    return (b or b"").decode("utf-8", "replace")
+
+
+# ---- crates/berth-kernels/src/lib.rs:135-192
+def exl3_linear(a, trellis, c, suh, a_had, svh, size_m, size_k, size_n, k_bits,
+                codebook: Codebook, out: OutDtype, stream=None) -> None:
+    L = load()
+    rc = L.berth_exl3_linear(a, trellis, c, suh, a_had, svh, size_m, size_k, size_n, k_bits,
+                             int(codebook), int(out), stream)
+    if rc != 0:
+        raise LaunchError(last_error() or f"exl3 linear launch failed ({rc})")
+
+
+def last_launch() -> str:
+    return _s(load().berth_exl3_last_launch())
+
+
+def last_error() -> str:
+    return _s(load().berth_exl3_last_error())
+
+
+def device_cc(device: int = 0) -> int:
+    return load().berth_device_cc(device)
+
+
+def device_sms(device: int = 0) -> int:
+    return load().berth_device_sms(device)
+
+
+class prefill_lin:
+    """crates/berth-kernels/src/prefill_lin.rs."""
+
+    @staticmethod
+    def exl3_linear(a, trellis, c, suh, a_had, svh, w_scratch, size_m, size_k, size_n, k_bits,
+                    codebook: Codebook, out: OutDtype, stream=None) -> None:
+        L = load()
+        rc = L.berth_prefill_exl3_linear(a, trellis, c, suh, a_had, svh, w_scratch, size_m, size_k,
+                                         size_n, k_bits, int(codebook), int(out), stream)
+        if rc != 0:
+            raise LaunchError(prefill_lin.last_error() or f"prefill exl3 linear launch failed ({rc})")
+
+    @staticmethod
+    def hgemm(a, b, c, size_m, size_k, size_n, ldc, out: OutDtype, stream=None) -> None:
+        rc = load().berth_prefill_hgemm(a, b, c, size_m, size_k, size_n, ldc, int(out), stream)
+        if rc != 0:
+            raise LaunchError(prefill_lin.last_error() or f"prefill hgemm launch failed ({rc})")
+
+    @staticmethod
+    def reconstruct(unpacked, packed, size_k, slice_n, full_n, n_offset, k_bits,
+                    codebook: Codebook, stream=None) -> None:
+        rc = load().berth_prefill_reconstruct(unpacked, packed, size_k, slice_n, full_n, n_offset,
+                                              k_bits, int(codebook), stream)
+        if rc != 0:
+            raise LaunchError(prefill_lin.last_error() or f"prefill reconstruct launch failed ({rc})")
+
+    @staticmethod
+    def had_r_128(inp, out, scale, pre_scale: bool, rows, cols, fp32: bool, stream=None) -> None:
+        rc = load().berth_prefill_had_r_128(inp, out, scale, int(pre_scale), rows, cols, int(fp32), stream)
+        if rc != 0:
+            raise LaunchError(prefill_lin.last_error() or f"prefill had_r_128 launch failed ({rc})")
+
+    @staticmethod
+    def last_launch() -> str:
+        return _s(load().berth_prefill_last_launch())
+
+    @staticmethod
+    def last_error() -> str:
+        return _s(load().berth_prefill_last_error())
+
+
+class ops:
+    """crates/berth-kernels/src/ops.rs (the EXL3-path subset)."""
+
+    @staticmethod
+    def silu_mul(gate, up, out, numel: int, act_limit: float = 0.0, stream=None) -> None:
+        rc = load().berth_ops_silu_mul(gate, up, out, numel, act_limit, stream)
+        if rc != 0:
+            raise LaunchError(ops.last_error() or f"silu_mul launch failed ({rc})")
+
+    @staticmethod
+    def last_launch() -> str:
+        return _s(load().berth_ops_last_launch())
+
+    @staticmethod
+    def last_error() -> str:
+        return _s(load().berth_ops_last_error())

@@ -1,0 +1,89 @@
+/*
+ * berth_kernels_hip.h — C ABI of libberth_kernels_hip.so (MI355X / gfx950).
+ *
+ * Drop-in for the `extern "C"` surface the reference's berth-kernels crate binds
+ * for the EXL3 linear path.  Each declaration cites the reference interface it
+ * replaces.  Conventions, all taken from the reference
+ * (crates/berth-kernels/src/lib.rs:88-133,179-192; csrc/linear.cu:362-404):
+ *   - every pointer is a raw device address; the caller owns every buffer;
+ *   - `stream` is a hipStream_t passed as void*, NULL = the default stream;
+ *     launches are asynchronous on it and never synchronise;
+ *   - return 0 on success, -1 on error; the message is a thread-local C string
+ *     (`*_last_error`) valid until the next call of the same family on the
+ *     thread and empty after a success; `*_last_launch` names the kernel that
+ *     ran and is empty after a failure;
+ *   - argument validation happens before any device call; C++ exceptions never
+ *     cross this boundary; bias is not applied;
+ *   - the library owns lazily allocated per-device internals (a 16 MiB split-K
+ *     workspace and its counters) that are never freed or grown; concurrent
+ *     launches on one device are not serialised and share that workspace.
+ */
+#ifndef BERTH_KERNELS_HIP_H
+#define BERTH_KERNELS_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* codebook: 0 default (3INST), 1 mcg, 2 mul1 — crates/berth-kernels/src/lib.rs:54-63 */
+
+/* ---- single linear, the decode shim --------------------------------------
+ * replaces crates/berth-kernels/src/ffi.rs:7-21 / csrc/linear.cu:362-394.
+ * a fp16 [size_m][size_k]; trellis int16 [size_k/16][size_n/16][16*k_bits];
+ * c fp16|fp32 [size_m][size_n]; suh fp16 [size_k]; a_had fp16 [size_m][size_k]
+ * (written); svh fp16 [size_n].  size_k % 128 == 0, size_n % 128 == 0,
+ * k_bits 1..8, any size_m >= 1. */
+int berth_exl3_linear(const void* a, const void* trellis, void* c, const void* suh,
+                      void* a_had, const void* svh, int size_m, int size_k, int size_n,
+                      int k_bits, int codebook, int out_fp32, void* stream);
+const char* berth_exl3_last_error(void);   /* ffi.rs:23, linear.cu:396 */
+const char* berth_exl3_last_launch(void);  /* ffi.rs:24, linear.cu:401 */
+
+/* crates/berth-kernels/csrc/linear.cu:301-332.  cc is the gfx target number
+ * (950 on MI355X); sms is the compute-unit count. */
+int berth_device_cc(int device);
+int berth_device_sms(int device);
+
+/* ---- rows > 1, the prefill shim -------------------------------------------
+ * replaces crates/berth-kernels/src/prefill_lin.rs:36-79 /
+ * csrc/prefill_lin/linear.cu:348-430.  Same tensors as above; w_scratch (fp16,
+ * size_k * min(size_n, 32768)) must be non-NULL when size_m > 144 as in the
+ * reference contract, though this implementation decodes inside the GEMM and
+ * does not write it. */
+int berth_prefill_exl3_linear(const void* a, const void* trellis, void* c, const void* suh,
+                              void* a_had, const void* svh, void* w_scratch, int size_m,
+                              int size_k, int size_n, int k_bits, int codebook, int c_fp32,
+                              void* stream);
+/* C[m][ldc] (fp16|fp32) = A[m][k] @ B[k][n], fp16 operands, fp32 accumulate */
+int berth_prefill_hgemm(const void* a, const void* b, void* c, int size_m, int size_k,
+                        int size_n, int ldc, int c_fp32, void* stream);
+const char* berth_prefill_last_error(void);
+const char* berth_prefill_last_launch(void);
+
+/* The reference keeps these two internal (C++ linkage,
+ * crates/berth-kernels/csrc/prefill_lin/api.h, reconstruct.cu:31-93); they are
+ * exported here because the dequantised weight is a parity target of its own.
+ * reconstruct: unpacked fp16 [size_k][slice_n] = columns n_offset.. of the
+ * decoded [size_k][full_n] inner weight.  had_r_128: per row and 128 columns,
+ * out = Hh(in*scale) when pre_scale, else Hh(in)*scale; fp32 selects float
+ * tensors. */
+int berth_prefill_reconstruct(void* unpacked, const void* packed, int size_k, int slice_n,
+                              int full_n, int n_offset, int k_bits, int codebook, void* stream);
+int berth_prefill_had_r_128(const void* input, void* output, const void* scale, int pre_scale,
+                            int rows, int cols, int fp32, void* stream);
+
+/* ---- ops -------------------------------------------------------------------
+ * replaces crates/berth-kernels/src/ops.rs:82-90 / csrc/ops/act.cu:35-69:
+ * out = silu(gate) * up, fp16, numel even, act_limit 0 = no clamp; out may
+ * alias up. */
+int berth_ops_silu_mul(const void* gate, const void* up, void* out, int64_t numel,
+                       float act_limit, void* stream);
+const char* berth_ops_last_error(void);    /* ops.rs:145 */
+const char* berth_ops_last_launch(void);   /* ops.rs:146 */
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,97 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the
+header declares, and validates arguments before any device call (the
+host-only tests of crates/berth-kernels/src/lib.rs:235-319 and
+crates/berth-kernels/src/prefill_lin.rs:338-383, with dangling pointers)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from berth_amd import kernels as K
+from berth_amd.kernels import Codebook, LaunchError, OutDtype
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+P = 0x1000   # non-null, never dereferenced: the checks return first
+
+
+def _declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(berth_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_kernel_library_exports_every_declared_symbol():
+    lib = K.load()
+    names = _declared("berth_kernels_hip.h")
+    assert "berth_exl3_linear" in names and "berth_ops_silu_mul" in names
+    for name in names:
+        assert getattr(lib, name) is not None, name
+
+
+def test_runtime_library_exports_every_declared_symbol():
+    path = os.path.join(ROOT, "berth_amd", "lib", "libberth_hip.so")
+    lib = C.CDLL(path)
+    names = _declared("berth_hip.h")
+    assert len(names) > 20
+    for name in names:
+        assert getattr(lib, name) is not None, name
+
+
+def test_linear_null_and_bad_sizes_do_not_touch_the_device():
+    with pytest.raises(LaunchError, match="null"):
+        K.exl3_linear(None, None, None, None, None, None, 1, 128, 256, 4, Codebook.MUL1, OutDtype.F16)
+    assert K.last_launch() == ""
+    with pytest.raises(LaunchError, match="multiple of 16"):
+        K.exl3_linear(P, P, P, P, P, P, 1, 15, 256, 4, Codebook.MUL1, OutDtype.F32)
+    with pytest.raises(LaunchError, match="multiple of 128"):
+        K.exl3_linear(P, P, P, P, P, P, 1, 16, 100, 4, Codebook.MUL1, OutDtype.F16)
+    with pytest.raises(LaunchError, match="positive"):
+        K.exl3_linear(P, P, P, P, P, P, 0, 16, 128, 4, Codebook.MUL1, OutDtype.F16)
+    with pytest.raises(LaunchError, match="1..=8"):
+        K.exl3_linear(P, P, P, P, P, P, 1, 128, 128, 9, Codebook.MUL1, OutDtype.F16)
+    with pytest.raises(LaunchError, match="codebook"):
+        K.load().berth_exl3_linear(P, P, P, P, P, P, 1, 128, 128, 4, 3, 0, None) and (_ for _ in ()).throw(
+            LaunchError(K.last_error()))
+    # size_k = 16 passes the reference's checks; the Hadamard block needs 128
+    with pytest.raises(LaunchError, match="multiple of 128"):
+        K.exl3_linear(P, P, P, P, P, P, 1, 16, 128, 4, Codebook.MUL1, OutDtype.F16)
+    assert K.last_error() != ""
+
+
+def test_error_is_cleared_by_the_next_failure_and_is_per_family():
+    with pytest.raises(LaunchError):
+        K.exl3_linear(None, None, None, None, None, None, 1, 128, 256, 4, Codebook.MUL1, OutDtype.F16)
+    first = K.last_error()
+    with pytest.raises(LaunchError):
+        K.ops.silu_mul(P, P, P, 3)
+    assert K.last_error() == first            # the ops family has its own slot
+    assert "even" in K.ops.last_error()
+
+
+def test_prefill_validation_order():
+    with pytest.raises(LaunchError, match="null"):
+        K.prefill_lin.exl3_linear(None, P, P, P, P, P, None, 2, 128, 128, 4, Codebook.MUL1, OutDtype.F16)
+    with pytest.raises(LaunchError, match="size_m must be > 1"):
+        K.prefill_lin.exl3_linear(P, P, P, P, P, P, None, 1, 128, 128, 4, Codebook.MUL1, OutDtype.F16)
+    with pytest.raises(LaunchError, match="multiple of 16"):
+        K.prefill_lin.exl3_linear(P, P, P, P, P, P, None, 2, 24, 128, 4, Codebook.MUL1, OutDtype.F16)
+    with pytest.raises(LaunchError, match="w_scratch"):
+        K.prefill_lin.exl3_linear(P, P, P, P, P, P, None, 145, 128, 128, 4, Codebook.MUL1, OutDtype.F16)
+    assert K.prefill_lin.last_launch() == ""
+    with pytest.raises(LaunchError, match="bad shape"):
+        K.prefill_lin.hgemm(P, P, P, 4, 8, 16, 8, OutDtype.F16)
+    with pytest.raises(LaunchError, match="null"):
+        K.prefill_lin.hgemm(None, P, P, 4, 8, 16, 16, OutDtype.F16)
+    with pytest.raises(LaunchError, match="slice exceeds"):
+        K.prefill_lin.reconstruct(P, P, 128, 256, 256, 128, 4, Codebook.MUL1)
+    with pytest.raises(LaunchError, match="had columns"):
+        K.prefill_lin.had_r_128(P, P, P, True, 1, 100, False)
+
+
+def test_silu_mul_validation():
+    with pytest.raises(LaunchError, match="null"):
+        K.ops.silu_mul(None, P, P, 4)
+    with pytest.raises(LaunchError, match="positive and even"):
+        K.ops.silu_mul(P, P, P, 0)
+    assert K.ops.last_launch() == ""

@@ -1,0 +1,252 @@
+"""GPU parity of the EXL3 linear path against the CPU oracle, through the C ABI.
+
+Bars: dequantised weights, rotated activations (a_had), Hadamard rows and the
+SiLU gate are bit-exact; linear outputs are within rtol 2e-3 / atol 1e-3 of the
+oracle's fp32 matmul over the oracle-decoded weights."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from berth_amd import kernels as K
+from berth_amd import synth
+from berth_amd.kernels import Codebook, OutDtype
+from oracle import oracle as O
+from tests.gpu_util import DEV, close, dev, host_f16, host_u16
+
+pytestmark = pytest.mark.gpu
+
+
+def _reconstruct(tr, Kk, N, bits, cb, n_offset=0, slice_n=None):
+    slice_n = slice_n or N
+    out = torch.zeros((Kk, slice_n), dtype=torch.float16, device=DEV)
+    d_tr = dev(tr)
+    K.prefill_lin.reconstruct(out.data_ptr(), d_tr.data_ptr(), Kk, slice_n, N, n_offset, bits, Codebook(cb))
+    torch.cuda.synchronize()
+    return host_u16(out)
+
+
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("cb", [0, 1, 2])
+def test_dequant_bit_exact(bits, cb):
+    Kk, N = 144, 384            # 9 tile rows (not a multiple of the 4 a workgroup takes)
+    tr = synth.trellis_words(1000 + 10 * bits + cb, Kk, N, bits)
+    got = _reconstruct(tr, Kk, N, bits, cb)
+    want = O.dequant(tr, Kk, N, bits, cb).view(np.uint16)
+    assert np.array_equal(got, want)
+
+
+def test_dequant_every_state_of_every_codebook():
+    """A 4 bpw trellis built so that all 65536 states occur: a de Bruijn-like
+    sweep is not needed, 8 bpw tiles expose two arbitrary bytes per state."""
+    Kk, N = 256, 256            # 256 tiles x 256 states = 65536 states at 8 bpw
+    words = np.arange(65536, dtype=np.uint32)
+    # at 8 bpw state t = bytes (t-1, t) of the stream: lay all 16-bit values out as byte pairs
+    stream = np.zeros((256, 256), dtype=np.uint8)
+    rng = np.random.default_rng(0)
+    stream[:] = rng.integers(0, 256, size=(256, 256), dtype=np.uint8)
+    tr = (stream[:, 0::2].astype(np.uint16) << 8 | stream[:, 1::2]).reshape(16, 16, 128)
+    for cb in (0, 1, 2):
+        got = _reconstruct(tr, Kk, N, 8, cb)
+        want = O.dequant(tr, Kk, N, 8, cb).view(np.uint16)
+        assert np.array_equal(got, want)
+    del words
+
+
+def test_dequant_column_slice():
+    Kk, N, bits = 64, 512, 4
+    tr = synth.trellis_words(5, Kk, N, bits)
+    want = O.dequant(tr, Kk, N, bits, 2).view(np.uint16)
+    got = _reconstruct(tr, Kk, N, bits, 2, n_offset=128, slice_n=256)
+    assert np.array_equal(got, want[:, 128:384])
+
+
+def test_dequant_full_size_config0_is_bit_exact():
+    Kk = N = 4096
+    tr = synth.trellis_words(0, Kk, N, 4)
+    got = _reconstruct(tr, Kk, N, 4, 2)
+    want = O.dequant(tr, Kk, N, 4, 2).view(np.uint16)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("pre", [True, False])
+@pytest.mark.parametrize("fp32", [False, True])
+def test_had_r_128_bit_exact(pre, fp32):
+    rows, cols = 5, 384
+    sc = synth.sign_scale(3, cols)
+    x16 = synth.activations(4, rows, cols)
+    d_sc = dev(sc.view(np.uint16))
+    if fp32:
+        x = (x16.astype(np.float32) * 3.7).astype(np.float32)
+        d_x = torch.from_numpy(x).to(DEV)
+        d_o = torch.zeros_like(d_x)
+        K.prefill_lin.had_r_128(d_x.data_ptr(), d_o.data_ptr(), d_sc.data_ptr(), pre, rows, cols, True)
+        torch.cuda.synchronize()
+        want = O.had_rows_f32(x, sc, pre)
+        assert np.array_equal(d_o.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    else:
+        d_x = dev(x16.view(np.uint16))
+        d_o = torch.zeros_like(d_x)
+        K.prefill_lin.had_r_128(d_x.data_ptr(), d_o.data_ptr(), d_sc.data_ptr(), pre, rows, cols, False)
+        torch.cuda.synchronize()
+        want = O.had_rows_f16(x16, sc, pre).view(np.uint16)
+        assert np.array_equal(host_u16(d_o), want)
+
+
+def test_silu_mul_reference_fixture_bit_exact(golden_dir):
+    g = np.fromfile(os.path.join(golden_dir, "silu.gate.bin"), dtype=np.uint16)
+    u = np.fromfile(os.path.join(golden_dir, "silu.up.bin"), dtype=np.uint16)
+    want = np.fromfile(os.path.join(golden_dir, "silu.out.bin"), dtype=np.uint16)
+    d_g, d_u = dev(g), dev(u)
+    K.ops.silu_mul(d_g.data_ptr(), d_u.data_ptr(), d_u.data_ptr(), g.size, 0.0)   # in place on up
+    torch.cuda.synchronize()
+    assert "silu_mul_kernel" in K.ops.last_launch()
+    assert np.array_equal(host_u16(d_u), want)
+
+
+def test_silu_mul_random_matches_oracle():
+    rng = np.random.default_rng(8)
+    g = (rng.normal(size=4096) * 4).astype(np.float16)
+    u = (rng.normal(size=4096) * 4).astype(np.float16)
+    d_g, d_u, d_o = dev(g.view(np.uint16)), dev(u.view(np.uint16)), torch.zeros(4096, dtype=torch.float16, device=DEV)
+    K.ops.silu_mul(d_g.data_ptr(), d_u.data_ptr(), d_o.data_ptr(), 4096, 0.0)
+    torch.cuda.synchronize()
+    want = O.silu_mul(g, u).view(np.uint16)
+    d = np.abs(host_u16(d_o).view(np.int16).astype(np.int32) - want.view(np.int16).astype(np.int32))
+    assert d.max() <= 1 and (d == 0).mean() > 0.999
+
+
+def _run_linear(m, Kk, N, bits, cb, out_fp32, seed, prefill=False):
+    tr, suh, svh = synth.linear(seed, Kk, N, bits)
+    x = synth.activations(seed + 7, m, Kk)
+    d = {k: dev(v.view(np.uint16)) for k, v in dict(tr=tr, suh=suh, svh=svh, x=x).items()}
+    c = torch.zeros((m, N), dtype=torch.float32 if out_fp32 else torch.float16, device=DEV)
+    a_had = torch.zeros((m, Kk), dtype=torch.float16, device=DEV)
+    out = OutDtype.F32 if out_fp32 else OutDtype.F16
+    if prefill:
+        w = torch.zeros(Kk * min(N, 32768), dtype=torch.float16, device=DEV) if m > 144 else None
+        K.prefill_lin.exl3_linear(d["x"].data_ptr(), d["tr"].data_ptr(), c.data_ptr(), d["suh"].data_ptr(),
+                                  a_had.data_ptr(), d["svh"].data_ptr(), w.data_ptr() if w is not None else None,
+                                  m, Kk, N, bits, Codebook(cb), out)
+        launch = K.prefill_lin.last_launch()
+    else:
+        K.exl3_linear(d["x"].data_ptr(), d["tr"].data_ptr(), c.data_ptr(), d["suh"].data_ptr(),
+                      a_had.data_ptr(), d["svh"].data_ptr(), m, Kk, N, bits, Codebook(cb), out)
+        launch = K.last_launch()
+    torch.cuda.synchronize()
+    want, want_had = O.linear(x, tr, suh, svh, Kk, N, bits, cb, out_fp32=out_fp32)
+    got = c.cpu().numpy() if out_fp32 else host_f16(c)
+    return got, want, host_u16(a_had), want_had.view(np.uint16), launch
+
+
+@pytest.mark.parametrize("bits,cb", [(4, 2), (2, 2), (3, 2), (5, 2), (6, 2), (8, 2), (1, 2), (4, 0), (4, 1), (3, 1)])
+@pytest.mark.parametrize("out_fp32", [False, True])
+def test_gemv_m1(bits, cb, out_fp32):
+    got, want, ah, want_ah, launch = _run_linear(1, 512, 384, bits, cb, out_fp32, 50 + bits)
+    assert "exl3_gemv_kernel" in launch
+    assert np.array_equal(ah, want_ah)
+    bad, worst = close(got, want)
+    assert bad == 0, (bad, worst)
+
+
+@pytest.mark.parametrize("Kk,N", [(128, 128), (4096, 4096), (5120, 1024), (1024, 5120), (2048, 768), (768, 2048)])
+def test_gemv_m1_shapes_split_k(Kk, N):
+    got, want, ah, want_ah, launch = _run_linear(1, Kk, N, 4, 2, True, Kk + N)
+    assert np.array_equal(ah, want_ah)
+    bad, worst = close(got, want)
+    assert bad == 0, (bad, worst, launch)
+
+
+def test_gemv_m1_is_deterministic_and_counters_reset():
+    outs = []
+    for _ in range(3):
+        got, _, _, _, launch = _run_linear(1, 4096, 512, 4, 2, True, 99)
+        outs.append(got.view(np.uint32).copy())
+    assert "split_k=" in launch and "split_k=1 " not in launch
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
+@pytest.mark.parametrize("m", [2, 3, 4, 5, 8])
+def test_gemv_small_rows(m):
+    got, want, ah, want_ah, launch = _run_linear(m, 512, 256, 4, 2, m % 2 == 0, 70 + m, prefill=True)
+    assert "exl3_gemv_kernel" in launch
+    assert np.array_equal(ah, want_ah)
+    bad, worst = close(got, want)
+    assert bad == 0, (bad, worst)
+
+
+@pytest.mark.parametrize("m", [9, 32, 47, 144, 145, 200])
+@pytest.mark.parametrize("out_fp32", [False, True])
+def test_gemm_rows(m, out_fp32):
+    got, want, ah, want_ah, launch = _run_linear(m, 512, 384, 4, 2, out_fp32, 80 + m, prefill=True)
+    assert "exl3_gemm_kernel" in launch
+    assert np.array_equal(ah, want_ah)
+    bad, worst = close(got, want)
+    assert bad == 0, (bad, worst)
+
+
+@pytest.mark.parametrize("bits,cb", [(2, 2), (3, 2), (5, 2), (6, 2), (4, 0), (4, 1)])
+def test_gemm_other_rates(bits, cb):
+    got, want, ah, want_ah, _ = _run_linear(64, 256, 256, bits, cb, True, 90 + bits, prefill=True)
+    assert np.array_equal(ah, want_ah)
+    bad, worst = close(got, want)
+    assert bad == 0, (bad, worst)
+
+
+def test_linear_through_decode_entry_with_many_rows():
+    """forward_n passes rows 2..144 of a K = 6 linear to the m = 1 entry
+    (crates/berth-engine/src/device.rs:338-352)."""
+    got, want, ah, want_ah, launch = _run_linear(20, 256, 256, 6, 2, False, 123)
+    assert "exl3_gemm_kernel" in launch
+    assert np.array_equal(ah, want_ah)
+    assert close(got, want)[0] == 0
+
+
+def test_hgemm_matches_oracle():
+    rng = np.random.default_rng(12)
+    m, k, n = 70, 200, 136
+    a = rng.normal(size=(m, k)).astype(np.float16)
+    b = rng.normal(size=(k, n)).astype(np.float16)
+    d_a, d_b = dev(a.view(np.uint16)), dev(b.view(np.uint16))
+    for fp32 in (True, False):
+        c = torch.zeros((m, n + 8), dtype=torch.float32 if fp32 else torch.float16, device=DEV)
+        K.prefill_lin.hgemm(d_a.data_ptr(), d_b.data_ptr(), c.data_ptr(), m, k, n, n + 8,
+                            OutDtype.F32 if fp32 else OutDtype.F16)
+        torch.cuda.synchronize()
+        want = O.hgemm(a, b, True)
+        got = c.cpu().numpy()[:, :n] if fp32 else host_f16(c)[:, :n]
+        assert np.allclose(got, want, rtol=2e-3, atol=2e-3)
+        assert not c.cpu().numpy()[:, n:].any() if fp32 else True
+
+
+def test_full_size_gemv_round_trip_property():
+    """At the 27B gate shape the oracle is too slow to run in a test; check the
+    size-independent property that the kernel is linear in the activation:
+    y(x1 + x2) == y(x1) + y(x2) within tolerance, and y(0) == 0 exactly."""
+    Kk, N = 5120, 17408
+    tr, suh, svh = synth.linear(7, Kk, N, 4)
+    d_tr, d_suh, d_svh = dev(tr), dev(suh.view(np.uint16)), dev(svh.view(np.uint16))
+    a_had = torch.zeros(Kk, dtype=torch.float16, device=DEV)
+
+    def run(xv):
+        c = torch.zeros(N, dtype=torch.float32, device=DEV)
+        dx = dev(xv.view(np.uint16))
+        K.exl3_linear(dx.data_ptr(), d_tr.data_ptr(), c.data_ptr(), d_suh.data_ptr(), a_had.data_ptr(),
+                      d_svh.data_ptr(), 1, Kk, N, 4, Codebook.MUL1, OutDtype.F32)
+        torch.cuda.synchronize()
+        return c.cpu().numpy()
+
+    x1 = (synth.activations(1, 1, Kk) * np.float16(0.5)).astype(np.float16)
+    x2 = (synth.activations(2, 1, Kk) * np.float16(0.5)).astype(np.float16)
+    y0 = run(np.zeros((1, Kk), dtype=np.float16))
+    assert not y0.any()
+    y1, y2 = run(x1), run(x2)
+    xs = (x1.astype(np.float32) + x2.astype(np.float32)).astype(np.float16)
+    ys = run(xs)
+    scale = np.abs(ys).max()
+    assert np.abs(ys - (y1 + y2)).max() < 4e-3 * scale
+    # spot-check 256 output columns against the oracle on the matching trellis slice
+    sub = tr[:, 16:32, :]                       # columns 256..511
+    want, _ = O.linear(x1, sub, suh, svh[256:512], Kk, 256, 4, 2, out_fp32=True)
+    assert close(y1[256:512], want.reshape(-1))[0] == 0
