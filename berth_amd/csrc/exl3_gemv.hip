@@ -19,6 +19,8 @@
 #include "hadamard.cuh"
 #include "launch.h"
 
+#include <cstdlib>
+
 namespace berth {
 
 struct GemvParams {
@@ -147,24 +149,40 @@ __global__ __launch_bounds__(256) void exl3_gemv_kernel(GemvParams p)
             for (int m = 0; m < MMAX; ++m)
                 __hip_atomic_store(mine + m * 128 + t, z[m], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        __threadfence();
+        // The partial sums travel as agent-scope atomic stores and loads, which go
+        // straight to the level of the memory hierarchy all compute dies share, so
+        // no cache-wide write-back or invalidate is needed: it is enough that this
+        // wave's stores have completed (the workgroup-scope release waits for them)
+        // before the arrival counter is bumped.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (t == 0) {
-            unsigned old = __hip_atomic_fetch_add(p.counters + nb, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+            unsigned old = __hip_atomic_fetch_add(p.counters + nb, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             s_last = (old == (unsigned)(p.S - 1)) ? 1u : 0u;
         }
         __syncthreads();
         if (!s_last) return;
-        __threadfence();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         if (t < 128) {
             const float* all = p.partials + ((size_t)(nb * p.S) * MMAX) * 128;
 #pragma unroll
             for (int m = 0; m < MMAX; ++m) z[m] = 0.0f;
-            for (int ss = 0; ss < p.S; ++ss) {
+            // loads in flight eight splits at a time; the adds stay in split order
+            for (int s0 = 0; s0 < p.S; s0 += 8) {
+                float part[8][MMAX];
 #pragma unroll
-                for (int m = 0; m < MMAX; ++m)
-                    z[m] += __hip_atomic_load(all + ((size_t)ss * MMAX + m) * 128 + t, __ATOMIC_RELAXED,
-                                              __HIP_MEMORY_SCOPE_AGENT);
+                for (int j = 0; j < 8; ++j)
+#pragma unroll
+                    for (int m = 0; m < MMAX; ++m)
+                        part[j][m] = (s0 + j < p.S)
+                            ? __hip_atomic_load(all + ((size_t)(s0 + j) * MMAX + m) * 128 + t, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT)
+                            : 0.0f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+#pragma unroll
+                    for (int m = 0; m < MMAX; ++m)
+                        if (s0 + j < p.S) z[m] += part[j][m];
             }
         }
         if (t == 0) __hip_atomic_store(p.counters + nb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -241,7 +259,12 @@ std::string launch_gemv(const LinearArgs& a)
 
     // waves per column block: enough workgroups to cover the chip several times,
     // at most one k-block per wave
-    const long target_wg = (long)ws.cu_count * 6;
+    static const int wg_per_cu = [] {
+        const char* e = std::getenv("BERTH_GEMV_WG_PER_CU");
+        int v = e ? std::atoi(e) : 0;
+        return v > 0 ? v : 6;
+    }();
+    const long target_wg = (long)ws.cu_count * wg_per_cu;
     int S = (int)((target_wg + p.NB - 1) / p.NB);
     const int s_max = (p.KB + 3) / 4;
     if (S > s_max) S = s_max;
