@@ -18,18 +18,22 @@
 // lane/32) + 8h + i], one 16-byte LDS read.  Column slots map to columns
 // 16*(slot/8) + slot%8 + 8f; the epilogue undoes that when it stages the fp32
 // tile in LDS for the output Hadamard.
-#include "exl3_decode.cuh"
-#include "hadamard.cuh"
+#include "exl3_gemv_kernel.cuh"
 #include "launch.h"
 
 namespace berth {
 
 struct GemmParams {
-    const _Float16* a_had;      // [M][K], already rotated
-    const uint32_t* trellis;
-    void* c;
-    const _Float16* svh;
+    const _Float16* a_had[2];   // [rows][K], already rotated (one per linear of the launch)
+    ExpertLin lin;              // dense mode
+    void* c[2];
     int M, K, N, out_fp32;
+    // grouped mode (problems != nullptr): blockIdx.y = problem (<= BM rows),
+    // blockIdx.z = which of the launch's linears
+    const ExpertLin* experts;
+    const GroupProblem* problems;
+    const int* num_problems;
+    int lins_per_expert, lin_base;
 };
 
 constexpr int kAStride = 128 + 8;   // halves per LDS row of the A tile (272 B: conflict-free b128 reads)
@@ -48,7 +52,19 @@ __global__ __launch_bounds__(256) void exl3_gemm_kernel(GemmParams p)
     const int half_id = lane >> 5;                      // which of the two tile rows
     const int slot = lane & 31;                         // MFMA row / column slot
     const int n0 = blockIdx.x * 256;
-    const int m0 = blockIdx.y * BM;
+    const int which = blockIdx.z;
+    int m0 = blockIdx.y * BM;
+    int m_end = p.M;
+    ExpertLin lin = p.lin;
+    if (p.problems) {
+        if ((int)blockIdx.y >= *p.num_problems) return;
+        const GroupProblem gp = p.problems[blockIdx.y];
+        lin = p.experts[gp.expert * p.lins_per_expert + p.lin_base + which];
+        m0 = gp.row0;
+        m_end = gp.row0 + gp.nrows;
+    }
+    const _Float16* a_had = p.a_had[which];
+    void* cout = p.c[which];
     const int nw = n0 + wave * 64;                      // first column of this wave
     const bool active = nw < p.N;
     const int tn = p.N >> 4;
@@ -66,7 +82,7 @@ __global__ __launch_bounds__(256) void exl3_gemm_kernel(GemmParams p)
             for (int r = 0; r < 16; ++r) acc[mb][f][r] = 0.0f;
 
     // lane's trellis position inside a k-block: tile row 2*step + half_id, tile (nw/16 + slot/8)
-    const uint32_t* tbase = p.trellis + (size_t)half_id * row_dw +
+    const uint32_t* tbase = lin.trellis + (size_t)half_id * row_dw +
                             (size_t)((nw >> 4) + (slot >> 3)) * tile_dw + (slot & 7) * BITS;
 
     uint32_t nxt[4][BITS];
@@ -89,8 +105,8 @@ __global__ __launch_bounds__(256) void exl3_gemm_kernel(GemmParams p)
         for (int idx = threadIdx.x; idx < BM * 8; idx += 256) {
             const int r = idx >> 3, ch = idx & 7;
             uint4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
-            if (m0 + r < p.M) {
-                const uint4* src = (const uint4*)(p.a_had + (size_t)(m0 + r) * p.K + kb * 128 + ch * 16);
+            if (m0 + r < m_end) {
+                const uint4* src = (const uint4*)(a_had + (size_t)(m0 + r) * p.K + kb * 128 + ch * 16);
                 v0 = src[0];
                 v1 = src[1];
             }
@@ -156,34 +172,34 @@ __global__ __launch_bounds__(256) void exl3_gemm_kernel(GemmParams p)
             const int row = task >> 1, blk = task & 1;
             const int gm = m0 + mb * 32 + row;
             const int gn = n0 + blk * 128;
-            if (gm >= p.M || gn >= p.N) continue;
+            if (gm >= m_end || gn >= p.N) continue;
             float v0 = z_tile[row * kZStride + blk * 128 + 2 * lane];
             float v1 = z_tile[row * kZStride + blk * 128 + 2 * lane + 1];
             had128_wave(v0, v1, lane);
-            const half2_t sv = ((const half2_t*)(p.svh + gn))[lane];
+            const half2_t sv = ((const half2_t*)(lin.svh + gn))[lane];
             v0 = (v0 * kRsqrt128) * (float)sv.x;
             v1 = (v1 * kRsqrt128) * (float)sv.y;
             const size_t at = (size_t)gm * p.N + gn + 2 * lane;
             if (p.out_fp32) {
                 float2_t o = {v0, v1};
-                *(float2_t*)((float*)p.c + at) = o;
+                *(float2_t*)((float*)cout + at) = o;
             } else {
                 half2_t o = {(_Float16)v0, (_Float16)v1};
-                *(half2_t*)((_Float16*)p.c + at) = o;
+                *(half2_t*)((_Float16*)cout + at) = o;
             }
         }
     }
 }
 
 template <int BITS, int CB>
-static void gemm_launch(const GemmParams& p, hipStream_t stream, std::string& desc)
+static void gemm_launch(const GemmParams& p, hipStream_t stream, std::string& desc, int grid_y = 0, int grid_z = 1)
 {
     constexpr int MB = 4;
     constexpr int BM = MB * 32;
     const size_t smem_a = (size_t)BM * kAStride * sizeof(_Float16);
     const size_t smem_z = (size_t)32 * (256 + 4) * sizeof(float);
     const size_t smem = smem_a > smem_z ? smem_a : smem_z;
-    dim3 grid((p.N + 255) / 256, (p.M + BM - 1) / BM);
+    dim3 grid((p.N + 255) / 256, grid_y ? grid_y : (p.M + BM - 1) / BM, grid_z);
     hipLaunchKernelGGL((exl3_gemm_kernel<BITS, CB, MB>), grid, dim3(256), smem, stream, p);
     desc = "exl3_gemm_kernel<" + std::to_string(BITS) + "," + std::to_string(CB) + "," + std::to_string(BM) +
            "x256> grid=" + std::to_string(grid.x) + "x" + std::to_string(grid.y) + " block=256 smem=" +
@@ -191,12 +207,26 @@ static void gemm_launch(const GemmParams& p, hipStream_t stream, std::string& de
 }
 
 template <int BITS>
-static void gemm_cb(const GemmParams& p, int cb, hipStream_t stream, std::string& desc)
+static void gemm_cb(const GemmParams& p, int cb, hipStream_t stream, std::string& desc, int gy = 0, int gz = 1)
 {
     switch (cb) {
-    case 0: gemm_launch<BITS, 0>(p, stream, desc); break;
-    case 1: gemm_launch<BITS, 1>(p, stream, desc); break;
-    default: gemm_launch<BITS, 2>(p, stream, desc); break;
+    case 0: gemm_launch<BITS, 0>(p, stream, desc, gy, gz); break;
+    case 1: gemm_launch<BITS, 1>(p, stream, desc, gy, gz); break;
+    default: gemm_launch<BITS, 2>(p, stream, desc, gy, gz); break;
+    }
+}
+
+static void gemm_bits(const GemmParams& p, int bits, int cb, hipStream_t stream, std::string& desc, int gy = 0, int gz = 1)
+{
+    switch (bits) {
+    case 1: gemm_cb<1>(p, cb, stream, desc, gy, gz); break;
+    case 2: gemm_cb<2>(p, cb, stream, desc, gy, gz); break;
+    case 3: gemm_cb<3>(p, cb, stream, desc, gy, gz); break;
+    case 4: gemm_cb<4>(p, cb, stream, desc, gy, gz); break;
+    case 5: gemm_cb<5>(p, cb, stream, desc, gy, gz); break;
+    case 6: gemm_cb<6>(p, cb, stream, desc, gy, gz); break;
+    case 7: gemm_cb<7>(p, cb, stream, desc, gy, gz); break;
+    default: gemm_cb<8>(p, cb, stream, desc, gy, gz); break;
     }
 }
 
@@ -204,28 +234,44 @@ std::string launch_gemm(const LinearArgs& a)
 {
     if (a.size_k % 128 != 0) throw std::runtime_error("exl3 linear: size_k must be a multiple of 128");
     std::string d0 = launch_had_r_128(a.a, a.a_had, a.suh, 1, a.size_m, a.size_k, 0, a.stream);
-    GemmParams p;
-    p.a_had = (const _Float16*)a.a_had;
-    p.trellis = (const uint32_t*)a.trellis;
-    p.c = a.c;
-    p.svh = (const _Float16*)a.svh;
+    GemmParams p{};
+    p.a_had[0] = (const _Float16*)a.a_had;
+    p.lin.trellis = (const uint32_t*)a.trellis;
+    p.lin.svh = (const _Float16*)a.svh;
+    p.c[0] = a.c;
     p.M = a.size_m;
     p.K = a.size_k;
     p.N = a.size_n;
     p.out_fp32 = a.out_fp32;
     std::string desc;
-    switch (a.k_bits) {
-    case 1: gemm_cb<1>(p, a.codebook, a.stream, desc); break;
-    case 2: gemm_cb<2>(p, a.codebook, a.stream, desc); break;
-    case 3: gemm_cb<3>(p, a.codebook, a.stream, desc); break;
-    case 4: gemm_cb<4>(p, a.codebook, a.stream, desc); break;
-    case 5: gemm_cb<5>(p, a.codebook, a.stream, desc); break;
-    case 6: gemm_cb<6>(p, a.codebook, a.stream, desc); break;
-    case 7: gemm_cb<7>(p, a.codebook, a.stream, desc); break;
-    default: gemm_cb<8>(p, a.codebook, a.stream, desc); break;
-    }
+    gemm_bits(p, a.k_bits, a.codebook, a.stream, desc);
     hip_ok(hipGetLastError(), "exl3_gemm_kernel launch");
     return d0 + " + " + desc + (a.out_fp32 ? " out=f32" : " out=f16");
+}
+
+// grouped: problems of at most 128 rows each; a_had rows are in problem order
+std::string launch_gemm_grouped(const GroupedArgs& g)
+{
+    if (g.size_k % 128 != 0 || g.size_n % 128 != 0)
+        throw std::runtime_error("moe grouped linear: sizes must be multiples of 128");
+    GemmParams p{};
+    p.a_had[0] = (const _Float16*)g.a_had;
+    p.a_had[1] = (const _Float16*)g.a_had2;
+    p.c[0] = g.c0;
+    p.c[1] = g.c1;
+    p.M = 0;
+    p.K = g.size_k;
+    p.N = g.size_n;
+    p.out_fp32 = g.out_fp32;
+    p.experts = (const ExpertLin*)g.experts;
+    p.problems = (const GroupProblem*)g.problems;
+    p.num_problems = g.num_problems;
+    p.lins_per_expert = g.lins_per_expert;
+    p.lin_base = g.lin_base;
+    std::string desc;
+    gemm_bits(p, g.k_bits, g.codebook, g.stream, desc, g.max_problems, g.num_lins);
+    hip_ok(hipGetLastError(), "exl3_gemm_kernel grouped launch");
+    return desc + " grouped";
 }
 
 // ---- plain fp16 GEMM (crates/berth-kernels/csrc/prefill_lin/linear.cu:387-418):

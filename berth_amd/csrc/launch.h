@@ -17,7 +17,7 @@ inline void hip_ok(hipError_t e, const char* what)
 
 // Per-device scratch owned by the library, allocated on first use and kept for
 // the life of the process: split-K partial sums and their arrival counters
-// (the role of the fixed 16 MiB workspace of
+// (the role of the fixed workspace of
 // crates/berth-kernels/csrc/int8_sq.cu:20-47).
 struct Workspace {
     float* partials = nullptr;      // kPartialBytes
@@ -25,7 +25,7 @@ struct Workspace {
     int device = -1;
     int cu_count = 0;
 };
-constexpr size_t kPartialBytes = 16u << 20;
+constexpr size_t kPartialBytes = 32u << 20;
 constexpr int kCounters = 65536;
 Workspace& workspace_for_current_device();
 
@@ -39,6 +39,27 @@ struct LinearArgs {
     int size_m, size_k, size_n, k_bits, codebook, out_fp32;
     hipStream_t stream;
 };
+
+// grouped (MoE) launches: problems, experts and num_problems are device memory
+struct GroupedArgs {
+    const void* a;              // input rows (fp16); with a_up the input is silu(a) * a_up
+    const void* a_up;
+    const int32_t* gather;      // optional: source row = gather[r] / gather_div
+    int gather_div;
+    const void* experts;        // ExpertLin[num_experts * lins_per_expert]
+    const void* problems;       // GroupProblem[max_problems]
+    const int* num_problems;
+    int max_problems;
+    int lins_per_expert, lin_base, num_lins;   // num_lins 1 or 2 consecutive linears per launch
+    void* c0;
+    void* c1;
+    const void* a_had;          // MFMA path: rotated input rows [rows][K] of the first linear
+    const void* a_had2;         // ... and of the second linear of the launch
+    int size_k, size_n, k_bits, codebook, out_fp32;
+    hipStream_t stream;
+};
+std::string launch_gemv_grouped(const GroupedArgs& args);
+std::string launch_gemm_grouped(const GroupedArgs& args);
 
 // rows 1..8: VALU dot-product kernel.  Returns the launch description.
 std::string launch_gemv(const LinearArgs& args);

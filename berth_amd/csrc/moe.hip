@@ -1,0 +1,600 @@
+// MoE layer on top of the EXL3 linears: route -> permute -> grouped expert FFNs
+// -> weighted combine.  The reference has no MoE implementation (its engine
+// rejects such layers, crates/berth-engine/src/model.rs:404-409); what it fixes is
+// the shape of the problem — MoeDims / Ffn::Moe{router, shared, experts}
+// (crates/berth-plan/src/shape.rs:64-69, plan.rs:24-59), "an expert is three EXL3
+// linears" (docs/exl3.md:39) and the expert-selection arguments of its multi-
+// linear kernel (crates/berth-kernels/csrc/ops/mgemm.cu:194-228).  The arithmetic
+// contract implemented here:
+//   logits[t][e] = sum over 64-row segments of (sum_h x[t][h] * wr[h][e], fp32 fma in
+//                  row order), segments added in order, then + bias[e];
+//   top-k on the logits, largest first, ties to the lowest expert index;
+//   weights = exp(logit - max) normalised over the selected k (renorm) or over
+//   all experts; pairs (token, slot) stable-sorted by expert;
+//   out[t] = shared(x[t]) + sum_j w[t][j] * FFN_{idx[t][j]}(x[t]) in slot order (fp32 fma).
+#include "exl3_gemv_kernel.cuh"
+#include "launch.h"
+
+#include "../../include/berth_kernels_hip.h"
+
+namespace berth {
+
+constexpr int kRouteSeg = 64;       // rows of the router weight per partial sum
+constexpr int kRouteTT = 4;         // tokens per route workgroup
+constexpr int kMaxExperts = 1024;
+constexpr int kMaxTopK = 32;
+constexpr int kValuRows = 8;        // experts with at most this many rows take the VALU kernel
+constexpr int kGemmRows = 128;      // rows per MFMA problem
+
+// ------------------------------------------------------------------ route
+
+struct RouteParams {
+    const _Float16* x;      // [T][H]
+    const _Float16* wr;     // [H][E]
+    const float* bias;      // [E] or null
+    float* parts;           // [T][nseg][E]
+    unsigned* counters;     // [ceil(T / kRouteTT)]
+    int32_t* idx;           // [T][k]
+    float* w;               // [T][k]
+    float* logits;          // [T][E] or null
+    int T, H, E, k, nseg, renorm;
+};
+
+__global__ __launch_bounds__(256) void moe_route_kernel(RouteParams p)
+{
+    __shared__ float xs[kRouteTT][kRouteSeg];
+    __shared__ unsigned s_last;
+    const int seg = blockIdx.x, grp = blockIdx.y;
+    const int t0 = grp * kRouteTT;
+    const int h0 = seg * kRouteSeg;
+    const int hn = min(kRouteSeg, p.H - h0);
+    const int tid = threadIdx.x;
+
+    for (int i = tid; i < kRouteTT * kRouteSeg; i += 256) {
+        const int tt = i / kRouteSeg, h = i % kRouteSeg;
+        float v = 0.0f;
+        if (t0 + tt < p.T && h < hn) v = (float)p.x[(size_t)(t0 + tt) * p.H + h0 + h];
+        xs[tt][h] = v;
+    }
+    __syncthreads();
+
+    for (int e = tid; e < p.E; e += 256) {
+        float part[kRouteTT];
+#pragma unroll
+        for (int tt = 0; tt < kRouteTT; ++tt) part[tt] = 0.0f;
+        for (int h = 0; h < hn; ++h) {
+            const float wv = (float)p.wr[(size_t)(h0 + h) * p.E + e];
+#pragma unroll
+            for (int tt = 0; tt < kRouteTT; ++tt) part[tt] = __builtin_fmaf(xs[tt][h], wv, part[tt]);
+        }
+#pragma unroll
+        for (int tt = 0; tt < kRouteTT; ++tt)
+            if (t0 + tt < p.T)
+                __hip_atomic_store(p.parts + ((size_t)(t0 + tt) * p.nseg + seg) * p.E + e, part[tt],
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (tid == 0) {
+        unsigned old = __hip_atomic_fetch_add(p.counters + grp, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (old == (unsigned)(p.nseg - 1)) ? 1u : 0u;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    if (tid == 0) __hip_atomic_store(p.counters + grp, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+    // ---- last workgroup of the token group: wave tt finishes token t0 + tt
+    const int lane = tid & 63, tt = tid >> 6;
+    const int t = t0 + tt;
+    if (t >= p.T) return;
+    constexpr int PER = kMaxExperts / 64;
+    float lg[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int e = lane + 64 * i;
+        float v = -INFINITY;
+        if (e < p.E) {
+            v = 0.0f;
+            const float* src = p.parts + (size_t)t * p.nseg * p.E + e;
+            for (int sg = 0; sg < p.nseg; ++sg)
+                v += __hip_atomic_load(src + (size_t)sg * p.E, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (p.bias) v += p.bias[e];
+            if (p.logits) p.logits[(size_t)t * p.E + e] = v;
+        }
+        lg[i] = v;
+    }
+    unsigned taken = 0;
+    float sel_logit = 0.0f;         // lane j keeps the logit of slot j
+    int sel_idx = 0;
+    for (int j = 0; j < p.k; ++j) {
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int e = lane + 64 * i;
+            if (e < p.E && !((taken >> i) & 1u) && (bi == 0x7fffffff || lg[i] > bv)) { bv = lg[i]; bi = e; }
+        }
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const float ov = __shfl_xor(bv, d, 64);
+            const int oi = __shfl_xor(bi, d, 64);
+            const bool take = (oi != 0x7fffffff) && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi));
+            if (take) { bv = ov; bi = oi; }
+        }
+        if ((bi & 63) == lane) taken |= 1u << (bi >> 6);
+        if (lane == j) { sel_logit = bv; sel_idx = bi; }
+    }
+    const float mx = __shfl(sel_logit, 0, 64);
+    float ev = (lane < p.k) ? expf(sel_logit - mx) : 0.0f;
+    float denom = 0.0f;
+    if (p.renorm) {
+        for (int j = 0; j < p.k; ++j) denom += __shfl(ev, j, 64);       // slot order
+    } else {
+        float loc = 0.0f;
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+            if (lane + 64 * i < p.E) loc += expf(lg[i] - mx);
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) loc += __shfl_xor(loc, d, 64);
+        denom = loc;
+    }
+    if (lane < p.k) {
+        p.idx[(size_t)t * p.k + lane] = sel_idx;
+        p.w[(size_t)t * p.k + lane] = ev / denom;
+    }
+}
+
+// ---------------------------------------------------------------- permute
+
+struct PermuteParams {
+    const int32_t* idx;     // [P] expert of each (token, slot) pair, P = T * k
+    int32_t* offsets;       // [E + 1]
+    int32_t* perm;          // [P] sorted position -> pair
+    int32_t* inv;           // [P] pair -> sorted position
+    int32_t* row_rows;      // [P] sorted position -> number of rows of its expert
+    int32_t* row_expert;    // [P] sorted position -> expert
+    int32_t* counts;        // [2] number of VALU problems, number of MFMA problems
+    GroupProblem* vprob;
+    GroupProblem* mprob;
+    int P, E;
+};
+
+// One workgroup.  Thread e scans the pairs in order and places those of expert
+// e: a stable counting sort whose result does not depend on scheduling.
+__global__ __launch_bounds__(1024) void moe_permute_kernel(PermuteParams p)
+{
+    __shared__ int cnt[kMaxExperts + 1];
+    __shared__ int off[kMaxExperts + 1];
+    const int tid = threadIdx.x;
+    for (int e = tid; e <= p.E; e += 1024) cnt[e] = 0;
+    __syncthreads();
+    for (int e = tid; e < p.E; e += 1024) {
+        int c = 0;
+        for (int q = 0; q < p.P; ++q) c += (p.idx[q] == e);
+        cnt[e] = c;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0, nv = 0, nm = 0;
+        for (int e = 0; e < p.E; ++e) {
+            off[e] = run;
+            const int m = cnt[e];
+            if (m > 0 && m <= kValuRows) {
+                p.vprob[nv++] = GroupProblem{e, run, m, 0};
+            } else if (m > kValuRows) {
+                for (int r = 0; r < m; r += kGemmRows)
+                    p.mprob[nm++] = GroupProblem{e, run + r, min(kGemmRows, m - r), 0};
+            }
+            run += m;
+        }
+        off[p.E] = run;
+        p.counts[0] = nv;
+        p.counts[1] = nm;
+    }
+    __syncthreads();
+    for (int e = tid; e <= p.E; e += 1024) p.offsets[e] = off[e];
+    for (int e = tid; e < p.E; e += 1024) {
+        int at = off[e];
+        const int m = cnt[e];
+        if (!m) continue;
+        for (int q = 0; q < p.P; ++q) {
+            if (p.idx[q] == e) {
+                p.perm[at] = q;
+                p.inv[q] = at;
+                p.row_rows[at] = m;
+                p.row_expert[at] = e;
+                ++at;
+            }
+        }
+    }
+}
+
+// ------------------------------------- rotated inputs for the MFMA problems
+
+struct HadRowsParams {
+    const _Float16* a;          // input rows
+    const _Float16* a_up;       // with a_up: input = silu(a[r]) * a_up[r]
+    const int32_t* gather;      // source row = gather[r] / gather_div, or r
+    int gather_div;
+    const int32_t* row_rows;
+    const int32_t* row_expert;
+    const ExpertLin* experts;
+    int lins_per_expert, lin_base;
+    _Float16* out[2];           // per blockIdx.z
+    int P, K;
+};
+
+__global__ __launch_bounds__(256) void moe_had_rows_kernel(HadRowsParams p)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = blockIdx.y;
+    if (p.row_rows[r] <= kValuRows) return;            // that expert takes the VALU kernel
+    const int kb = blockIdx.x * 4 + wave;
+    if (kb * 128 >= p.K) return;
+    const int which = blockIdx.z;
+    const ExpertLin lin = p.experts[p.row_expert[r] * p.lins_per_expert + p.lin_base + which];
+    const int src = p.gather ? p.gather[r] / p.gather_div : r;
+    half2_t x = ((const half2_t*)(p.a + (size_t)src * p.K + kb * 128))[lane];
+    if (p.a_up) {
+        const half2_t u = ((const half2_t*)(p.a_up + (size_t)src * p.K + kb * 128))[lane];
+        x.x = silu_mul_h(x.x, u.x);
+        x.y = silu_mul_h(x.y, u.y);
+    }
+    const half2_t sc = ((const half2_t*)(lin.suh + kb * 128))[lane];
+    float v0 = (float)x.x * (float)sc.x;
+    float v1 = (float)x.y * (float)sc.y;
+    had128_wave(v0, v1, lane);
+    half2_t o;
+    o.x = (_Float16)(v0 * kRsqrt128);
+    o.y = (_Float16)(v1 * kRsqrt128);
+    ((half2_t*)(p.out[which] + (size_t)r * p.K + kb * 128))[lane] = o;
+}
+
+// ---------------------------------------------------------------- combine
+
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ slot_out,
+                                                          const float* __restrict__ shared_out,
+                                                          const float* __restrict__ w,
+                                                          const int32_t* __restrict__ inv,
+                                                          float* __restrict__ out, int T, int H, int k)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)T * H) return;
+    const int t = (int)(i / H), h = (int)(i % H);
+    float acc = shared_out ? shared_out[i] : 0.0f;
+    for (int j = 0; j < k; ++j) {
+        const int pos = inv[t * k + j];
+        acc = __builtin_fmaf(w[t * k + j], slot_out[(size_t)pos * H + h], acc);
+    }
+    out[i] = acc;
+}
+
+// ------------------------------------------------------------ host side
+
+namespace {
+
+thread_local std::string g_moe_err, g_moe_launch;
+
+size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct MoeLayout {
+    size_t idx, w, parts, offsets, perm, inv, row_rows, row_expert, counts, vprob, mprob;
+    size_t ah0, ah1, g, u, ahd, slot_out, sg, su, s_ahad, shared_out, total;
+    int max_v, max_m, nseg;
+};
+
+MoeLayout moe_layout(int T, int H, int E, int k, int I, int shared_I)
+{
+    MoeLayout L{};
+    const size_t P = (size_t)T * k;
+    L.nseg = (H + kRouteSeg - 1) / kRouteSeg;
+    L.max_v = (int)std::min<size_t>((size_t)E, P);
+    L.max_m = P > (size_t)kValuRows ? (int)(P / (kValuRows + 1) + P / kGemmRows + 1) : 0;
+    size_t at = 0;
+    auto take = [&](size_t bytes) { size_t r = at; at = align_up(at + bytes); return r; };
+    L.idx = take(P * 4);
+    L.w = take(P * 4);
+    L.parts = take((size_t)T * L.nseg * E * 4);
+    L.offsets = take((size_t)(E + 1) * 4);
+    L.perm = take(P * 4);
+    L.inv = take(P * 4);
+    L.row_rows = take(P * 4);
+    L.row_expert = take(P * 4);
+    L.counts = take(16);
+    L.vprob = take((size_t)L.max_v * sizeof(GroupProblem));
+    L.mprob = take((size_t)std::max(L.max_m, 1) * sizeof(GroupProblem));
+    L.ah0 = take(L.max_m ? P * H * 2 : 0);
+    L.ah1 = take(L.max_m ? P * H * 2 : 0);
+    L.g = take(P * I * 2);
+    L.u = take(P * I * 2);
+    L.ahd = take(L.max_m ? P * I * 2 : 0);
+    L.slot_out = take(P * H * 4);
+    L.sg = take((size_t)T * shared_I * 2);
+    L.su = take((size_t)T * shared_I * 2);
+    L.s_ahad = take((size_t)T * std::max(H, shared_I) * 2);
+    L.shared_out = take(shared_I ? (size_t)T * H * 4 : 0);
+    L.total = at;
+    return L;
+}
+
+void check_route_shape(int T, int H, int E, int k)
+{
+    if (T < 1 || H < 1 || E < 1 || k < 1) throw std::runtime_error("moe: sizes must be positive");
+    if (k > E) throw std::runtime_error("moe: top-k exceeds the number of experts");
+    if (E > kMaxExperts) throw std::runtime_error("moe: at most 1024 experts");
+    if (k > kMaxTopK) throw std::runtime_error("moe: top-k must be at most 32");
+}
+
+std::string run_route(const void* x, const void* wr, const float* bias, int32_t* idx, float* w,
+                      float* logits, float* parts, int T, int H, int E, int k, int renorm,
+                      hipStream_t stream)
+{
+    Workspace& ws = workspace_for_current_device();
+    RouteParams p{};
+    p.x = (const _Float16*)x;
+    p.wr = (const _Float16*)wr;
+    p.bias = bias;
+    p.parts = parts;
+    p.counters = ws.counters;
+    p.idx = idx;
+    p.w = w;
+    p.logits = logits;
+    p.T = T; p.H = H; p.E = E; p.k = k; p.renorm = renorm;
+    p.nseg = (H + kRouteSeg - 1) / kRouteSeg;
+    const int groups = (T + kRouteTT - 1) / kRouteTT;
+    if (groups > kCounters) throw std::runtime_error("moe route: too many tokens for the counter table");
+    dim3 grid(p.nseg, groups);
+    hipLaunchKernelGGL(moe_route_kernel, grid, dim3(256), 0, stream, p);
+    hip_ok(hipGetLastError(), "moe_route_kernel launch");
+    return "moe_route_kernel grid=" + std::to_string(grid.x) + "x" + std::to_string(grid.y);
+}
+
+std::string run_permute(const int32_t* idx, unsigned char* wsb, const MoeLayout& L, int P, int E,
+                        hipStream_t stream)
+{
+    PermuteParams p{};
+    p.idx = idx;
+    p.offsets = (int32_t*)(wsb + L.offsets);
+    p.perm = (int32_t*)(wsb + L.perm);
+    p.inv = (int32_t*)(wsb + L.inv);
+    p.row_rows = (int32_t*)(wsb + L.row_rows);
+    p.row_expert = (int32_t*)(wsb + L.row_expert);
+    p.counts = (int32_t*)(wsb + L.counts);
+    p.vprob = (GroupProblem*)(wsb + L.vprob);
+    p.mprob = (GroupProblem*)(wsb + L.mprob);
+    p.P = P;
+    p.E = E;
+    hipLaunchKernelGGL(moe_permute_kernel, dim3(1), dim3(1024), 0, stream, p);
+    hip_ok(hipGetLastError(), "moe_permute_kernel launch");
+    return "moe_permute_kernel";
+}
+
+}  // namespace
+}  // namespace berth
+
+using namespace berth;
+
+extern "C" const char* berth_moe_last_error(void) { return g_moe_err.c_str(); }
+extern "C" const char* berth_moe_last_launch(void) { return g_moe_launch.c_str(); }
+
+#define MOE_TRY_BEGIN try { g_moe_err.clear(); g_moe_launch.clear();
+#define MOE_TRY_END return 0; } catch (const std::exception& err) { g_moe_err = err.what(); g_moe_launch.clear(); (void)hipGetLastError(); return -1; }
+
+extern "C" size_t berth_moe_workspace_bytes(int T, int H, int E, int k, int I, int shared_I)
+{
+    if (T < 1 || H < 1 || E < 1 || k < 1 || I < 1 || shared_I < 0) return 0;
+    return moe_layout(T, H, E, k, I, shared_I).total;
+}
+
+// byte offsets, inside a workspace of berth_moe_workspace_bytes, of the buffers a
+// caller may want to inspect after berth_moe_layer: {idx, w, offsets, perm, inv,
+// gate_out, up_out, slot_out, shared_out}
+extern "C" int berth_moe_workspace_offsets(int T, int H, int E, int k, int I, int shared_I, size_t out[9])
+{
+    if (T < 1 || H < 1 || E < 1 || k < 1 || I < 1 || shared_I < 0 || !out) return -1;
+    const MoeLayout L = moe_layout(T, H, E, k, I, shared_I);
+    const size_t v[9] = {L.idx, L.w, L.offsets, L.perm, L.inv, L.g, L.u, L.slot_out, L.shared_out};
+    for (int i = 0; i < 9; ++i) out[i] = v[i];
+    return 0;
+}
+
+extern "C" int berth_moe_route(const void* x, const void* wr, const float* bias, int32_t* idx, float* w,
+                               float* logits, void* parts_scratch, int T, int H, int E, int k,
+                               int renorm, void* stream)
+{
+    MOE_TRY_BEGIN
+    if (!x || !wr || !idx || !w || !parts_scratch) throw std::runtime_error("moe route: null device pointer");
+    check_route_shape(T, H, E, k);
+    g_moe_launch = run_route(x, wr, bias, idx, w, logits, (float*)parts_scratch, T, H, E, k, renorm,
+                             (hipStream_t)stream);
+    MOE_TRY_END
+}
+
+extern "C" int berth_moe_permute(const int32_t* idx, int32_t* offsets, int32_t* perm, int32_t* inv,
+                                 void* scratch, int T, int k, int E, void* stream)
+{
+    MOE_TRY_BEGIN
+    if (!idx || !offsets || !perm || !inv || !scratch) throw std::runtime_error("moe permute: null device pointer");
+    if (T < 1 || k < 1 || E < 1) throw std::runtime_error("moe: sizes must be positive");
+    if (E > kMaxExperts) throw std::runtime_error("moe: at most 1024 experts");
+    // scratch holds the row maps, the counts and the problem lists
+    const size_t P = (size_t)T * k;
+    unsigned char* sb = (unsigned char*)scratch;
+    PermuteParams p{};
+    p.idx = idx;
+    p.offsets = offsets;
+    p.perm = perm;
+    p.inv = inv;
+    size_t at = 0;
+    p.row_rows = (int32_t*)(sb + at); at = align_up(at + P * 4);
+    p.row_expert = (int32_t*)(sb + at); at = align_up(at + P * 4);
+    p.counts = (int32_t*)(sb + at); at = align_up(at + 16);
+    p.vprob = (GroupProblem*)(sb + at); at = align_up(at + (std::min<size_t>(E, P)) * sizeof(GroupProblem));
+    p.mprob = (GroupProblem*)(sb + at);
+    p.P = (int)P;
+    p.E = E;
+    hipLaunchKernelGGL(moe_permute_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, p);
+    hip_ok(hipGetLastError(), "moe_permute_kernel launch");
+    g_moe_launch = "moe_permute_kernel";
+    MOE_TRY_END
+}
+
+extern "C" size_t berth_moe_permute_scratch_bytes(int T, int k, int E)
+{
+    if (T < 1 || k < 1 || E < 1) return 0;
+    const size_t P = (size_t)T * k;
+    size_t at = 0;
+    at = align_up(at + P * 4);
+    at = align_up(at + P * 4);
+    at = align_up(at + 16);
+    at = align_up(at + std::min<size_t>(E, P) * sizeof(GroupProblem));
+    at = align_up(at + (P / (kValuRows + 1) + P / kGemmRows + 2) * sizeof(GroupProblem));
+    return at;
+}
+
+extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias, const void* experts,
+                               const berth_exl3_lin* shared, void* out, int32_t* idx_out, float* w_out,
+                               void* workspace, size_t workspace_bytes, int T, int H, int E, int k,
+                               int I, int shared_I, int k_bits, int codebook, int renorm, void* stream_)
+{
+    MOE_TRY_BEGIN
+    hipStream_t stream = (hipStream_t)stream_;
+    if (!x || !wr || !experts || !out || !workspace) throw std::runtime_error("moe layer: null device pointer");
+    check_route_shape(T, H, E, k);
+    if (I < 1) throw std::runtime_error("moe: sizes must be positive");
+    if ((long)T * k > 65535) throw std::runtime_error("moe layer: at most 65535 (token, slot) pairs per call");
+    if (k_bits < 1 || k_bits > 8) throw std::runtime_error("moe layer: K must be in 1..=8");
+    if (codebook < 0 || codebook > 2) throw std::runtime_error("moe layer: codebook must be 0, 1, or 2");
+    if (H % 128 || I % 128) throw std::runtime_error("moe layer: hidden and intermediate sizes must be multiples of 128");
+    if (shared && (shared_I < 128 || shared_I % 128))
+        throw std::runtime_error("moe layer: shared intermediate size must be a multiple of 128");
+    if (!shared) shared_I = 0;
+    const MoeLayout L = moe_layout(T, H, E, k, I, shared_I);
+    if (workspace_bytes < L.total)
+        throw std::runtime_error("moe layer: workspace too small (" + std::to_string(workspace_bytes) + " < " +
+                                 std::to_string(L.total) + ")");
+    unsigned char* wsb = (unsigned char*)workspace;
+    const int P = T * k;
+    int32_t* idx = (int32_t*)(wsb + L.idx);
+    float* w = (float*)(wsb + L.w);
+    std::string desc;
+
+    desc += run_route(x, wr, bias, idx, w, nullptr, (float*)(wsb + L.parts), T, H, E, k, renorm, stream);
+    desc += " + " + run_permute(idx, wsb, L, P, E, stream);
+
+    GroupedArgs g{};
+    g.experts = experts;
+    g.lins_per_expert = 3;
+    g.k_bits = k_bits;
+    g.codebook = codebook;
+    g.stream = stream;
+
+    // gate and up: input rows gathered from x, fp16 out in sorted order
+    g.a = x;
+    g.a_up = nullptr;
+    g.gather = (const int32_t*)(wsb + L.perm);
+    g.gather_div = k;
+    g.lin_base = 0;
+    g.num_lins = 2;
+    g.c0 = wsb + L.g;
+    g.c1 = wsb + L.u;
+    g.size_k = H;
+    g.size_n = I;
+    g.out_fp32 = 0;
+    g.problems = wsb + L.vprob;
+    g.num_problems = (const int*)(wsb + L.counts);
+    g.max_problems = L.max_v;
+    desc += " + " + launch_gemv_grouped(g);
+    if (L.max_m > 0) {
+        HadRowsParams h{};
+        h.a = (const _Float16*)x;
+        h.gather = (const int32_t*)(wsb + L.perm);
+        h.gather_div = k;
+        h.row_rows = (const int32_t*)(wsb + L.row_rows);
+        h.row_expert = (const int32_t*)(wsb + L.row_expert);
+        h.experts = (const ExpertLin*)experts;
+        h.lins_per_expert = 3;
+        h.lin_base = 0;
+        h.out[0] = (_Float16*)(wsb + L.ah0);
+        h.out[1] = (_Float16*)(wsb + L.ah1);
+        h.P = P;
+        h.K = H;
+        hipLaunchKernelGGL(moe_had_rows_kernel, dim3((H / 128 + 3) / 4, P, 2), dim3(256), 0, stream, h);
+        hip_ok(hipGetLastError(), "moe_had_rows_kernel launch");
+        g.problems = wsb + L.mprob;
+        g.num_problems = (const int*)(wsb + L.counts) + 1;
+        g.max_problems = L.max_m;
+        g.a_had = wsb + L.ah0;
+        g.a_had2 = wsb + L.ah1;
+        desc += " + moe_had_rows_kernel + " + launch_gemm_grouped(g);
+    }
+
+    // down: input silu(g) * u evaluated while the activation is rotated, fp32 out
+    g.a = wsb + L.g;
+    g.a_up = wsb + L.u;
+    g.gather = nullptr;
+    g.gather_div = 1;
+    g.lin_base = 2;
+    g.num_lins = 1;
+    g.c0 = wsb + L.slot_out;
+    g.c1 = nullptr;
+    g.size_k = I;
+    g.size_n = H;
+    g.out_fp32 = 1;
+    g.problems = wsb + L.vprob;
+    g.num_problems = (const int*)(wsb + L.counts);
+    g.max_problems = L.max_v;
+    desc += " + " + launch_gemv_grouped(g);
+    if (L.max_m > 0) {
+        HadRowsParams h{};
+        h.a = (const _Float16*)(wsb + L.g);
+        h.a_up = (const _Float16*)(wsb + L.u);
+        h.gather_div = 1;
+        h.row_rows = (const int32_t*)(wsb + L.row_rows);
+        h.row_expert = (const int32_t*)(wsb + L.row_expert);
+        h.experts = (const ExpertLin*)experts;
+        h.lins_per_expert = 3;
+        h.lin_base = 2;
+        h.out[0] = (_Float16*)(wsb + L.ahd);
+        h.P = P;
+        h.K = I;
+        hipLaunchKernelGGL(moe_had_rows_kernel, dim3((I / 128 + 3) / 4, P, 1), dim3(256), 0, stream, h);
+        hip_ok(hipGetLastError(), "moe_had_rows_kernel launch");
+        g.problems = wsb + L.mprob;
+        g.num_problems = (const int*)(wsb + L.counts) + 1;
+        g.max_problems = L.max_m;
+        g.a_had = wsb + L.ahd;
+        g.a_had2 = nullptr;
+        desc += " + moe_had_rows_kernel + " + launch_gemm_grouped(g);
+    }
+
+    // shared expert: three dense linears on every token
+    const float* shared_out = nullptr;
+    if (shared) {
+        for (int i = 0; i < 3; ++i)
+            if (!shared[i].trellis || !shared[i].suh || !shared[i].svh)
+                throw std::runtime_error("moe layer: null shared-expert pointer");
+        auto dense = [&](const void* a, const berth_exl3_lin& lin, void* c, int kk, int nn, int fp32) {
+            LinearArgs la{a, lin.trellis, c, lin.suh, wsb + L.s_ahad, lin.svh, T, kk, nn, k_bits, codebook, fp32, stream};
+            return T <= 8 ? launch_gemv(la) : launch_gemm(la);
+        };
+        dense(x, shared[0], wsb + L.sg, H, shared_I, 0);
+        dense(x, shared[1], wsb + L.su, H, shared_I, 0);
+        launch_silu_mul(wsb + L.sg, wsb + L.su, wsb + L.su, (int64_t)T * shared_I, 0.0f, stream);
+        dense(wsb + L.su, shared[2], wsb + L.shared_out, shared_I, H, 1);
+        shared_out = (const float*)(wsb + L.shared_out);
+        desc += " + shared expert";
+    }
+
+    const size_t total = (size_t)T * H;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                       (const float*)(wsb + L.slot_out), shared_out, (const float*)w,
+                       (const int32_t*)(wsb + L.inv), (float*)out, T, H, k);
+    hip_ok(hipGetLastError(), "moe_combine_kernel launch");
+    desc += " + moe_combine_kernel";
+    if (idx_out) hip_ok(hipMemcpyAsync(idx_out, idx, (size_t)P * 4, hipMemcpyDeviceToDevice, stream), "idx copy");
+    if (w_out) hip_ok(hipMemcpyAsync(w_out, w, (size_t)P * 4, hipMemcpyDeviceToDevice, stream), "w copy");
+    g_moe_launch = desc;
+    MOE_TRY_END
+}

@@ -53,6 +53,17 @@ def load() -> C.CDLL:
         for name in ("berth_exl3_last_error", "berth_exl3_last_launch", "berth_prefill_last_error",
                      "berth_prefill_last_launch", "berth_ops_last_error", "berth_ops_last_launch"):
             getattr(L, name).restype = C.c_char_p
+        L.berth_moe_route.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
+        L.berth_moe_permute.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, vp]
+        L.berth_moe_permute_scratch_bytes.argtypes = [ci, ci, ci]
+        L.berth_moe_permute_scratch_bytes.restype = C.c_size_t
+        L.berth_moe_layer.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t,
+                                      ci, ci, ci, ci, ci, ci, ci, ci, ci, vp]
+        L.berth_moe_workspace_bytes.argtypes = [ci] * 6
+        L.berth_moe_workspace_bytes.restype = C.c_size_t
+        L.berth_moe_workspace_offsets.argtypes = [ci] * 6 + [C.POINTER(C.c_size_t)]
+        L.berth_moe_last_error.restype = C.c_char_p
+        L.berth_moe_last_launch.restype = C.c_char_p
         L.berth_device_cc.argtypes = [ci]
         L.berth_device_sms.argtypes = [ci]
         _lib = L
@@ -146,3 +157,57 @@ class ops:
     @staticmethod
     def last_error() -> str:
         return _s(load().berth_ops_last_error())
+
+
+class ExpertLinStruct(C.Structure):
+    """`berth_exl3_lin`: device pointers of one EXL3 linear."""
+    _fields_ = [("trellis", C.c_void_p), ("suh", C.c_void_p), ("svh", C.c_void_p)]
+
+
+class moe:
+    """The MoE entry points (no counterpart in the reference's crate)."""
+
+    @staticmethod
+    def route(x, wr, bias, idx, w, logits, parts_scratch, T, H, E, k, renorm=True, stream=None) -> None:
+        rc = load().berth_moe_route(x, wr, bias, idx, w, logits, parts_scratch, T, H, E, k, int(renorm), stream)
+        if rc != 0:
+            raise LaunchError(moe.last_error() or f"moe route launch failed ({rc})")
+
+    @staticmethod
+    def permute(idx, offsets, perm, inv, scratch, T, k, E, stream=None) -> None:
+        rc = load().berth_moe_permute(idx, offsets, perm, inv, scratch, T, k, E, stream)
+        if rc != 0:
+            raise LaunchError(moe.last_error() or f"moe permute launch failed ({rc})")
+
+    @staticmethod
+    def permute_scratch_bytes(T, k, E) -> int:
+        return int(load().berth_moe_permute_scratch_bytes(T, k, E))
+
+    @staticmethod
+    def workspace_bytes(T, H, E, k, I, shared_I=0) -> int:
+        return int(load().berth_moe_workspace_bytes(T, H, E, k, I, shared_I))
+
+    @staticmethod
+    def workspace_offsets(T, H, E, k, I, shared_I=0) -> dict:
+        out = (C.c_size_t * 9)()
+        if load().berth_moe_workspace_offsets(T, H, E, k, I, shared_I, out) != 0:
+            raise LaunchError("moe: sizes must be positive")
+        names = ("idx", "w", "offsets", "perm", "inv", "gate_out", "up_out", "slot_out", "shared_out")
+        return dict(zip(names, (int(v) for v in out)))
+
+    @staticmethod
+    def layer(x, wr, bias, experts_dev, shared_host, out, idx_out, w_out, workspace, workspace_bytes,
+              T, H, E, k, I, shared_I, k_bits, codebook: Codebook, renorm=True, stream=None) -> None:
+        rc = load().berth_moe_layer(x, wr, bias, experts_dev, shared_host, out, idx_out, w_out, workspace,
+                                    workspace_bytes, T, H, E, k, I, shared_I, k_bits, int(codebook),
+                                    int(renorm), stream)
+        if rc != 0:
+            raise LaunchError(moe.last_error() or f"moe layer launch failed ({rc})")
+
+    @staticmethod
+    def last_launch() -> str:
+        return _s(load().berth_moe_last_launch())
+
+    @staticmethod
+    def last_error() -> str:
+        return _s(load().berth_moe_last_error())

@@ -14,13 +14,14 @@
  *     ran and is empty after a failure;
  *   - argument validation happens before any device call; C++ exceptions never
  *     cross this boundary; bias is not applied;
- *   - the library owns lazily allocated per-device internals (a 16 MiB split-K
+ *   - the library owns lazily allocated per-device internals (a 32 MiB split-K
  *     workspace and its counters) that are never freed or grown; concurrent
  *     launches on one device are not serialised and share that workspace.
  */
 #ifndef BERTH_KERNELS_HIP_H
 #define BERTH_KERNELS_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -82,6 +83,54 @@ int berth_ops_silu_mul(const void* gate, const void* up, void* out, int64_t nume
                        float act_limit, void* stream);
 const char* berth_ops_last_error(void);    /* ops.rs:145 */
 const char* berth_ops_last_launch(void);   /* ops.rs:146 */
+
+/* ---- MoE layer ---------------------------------------------------------------
+ * No counterpart in the reference, whose engine rejects MoE layers
+ * (crates/berth-engine/src/model.rs:404-409).  The shapes follow its plan schema
+ * (MoeDims / Ffn::Moe, crates/berth-plan/src/shape.rs:64-69, plan.rs:24-59: router,
+ * optional shared expert, E routed experts of three EXL3 linears each) and the
+ * expert-selection arguments of its multi-linear kernel
+ * (crates/berth-kernels/csrc/ops/mgemm.cu:194-228).  Same conventions as above;
+ * the message slots are berth_moe_last_error / berth_moe_last_launch.
+ *
+ * Arithmetic: logits = x @ wr in fp32 (64-row partial sums in row order, added in
+ * order) + bias; top-k on the logits, ties to the lowest index; weights =
+ * softmax over the selected k (renorm != 0) or over all experts; (token, slot)
+ * pairs stable-sorted by expert; expert FFN = down(silu(gate(x)) * up(x)) with
+ * fp16 gate/up outputs and fp32 down output; out = shared(x) + sum_j w_j *
+ * FFN_j(x) in slot order. */
+typedef struct {
+    const void* trellis;    /* int16 [K/16][N/16][16*k_bits] */
+    const void* suh;        /* fp16 [K] */
+    const void* svh;        /* fp16 [N] */
+} berth_exl3_lin;
+
+/* x fp16 [T][H]; wr fp16 [H][E] (the unquantised router, mlp.gate.weight laid out
+ * input-major); bias fp32 [E] or NULL; idx int32 [T][k]; w fp32 [T][k]; logits fp32
+ * [T][E] or NULL; parts_scratch fp32 [T][ceil(H/64)][E]. */
+int berth_moe_route(const void* x, const void* wr, const float* bias, int32_t* idx, float* w,
+                    float* logits, void* parts_scratch, int T, int H, int E, int k, int renorm,
+                    void* stream);
+/* offsets int32 [E+1]; perm int32 [T*k] (sorted position -> t*k + j); inv its
+ * inverse; scratch of berth_moe_permute_scratch_bytes bytes. */
+int berth_moe_permute(const int32_t* idx, int32_t* offsets, int32_t* perm, int32_t* inv,
+                      void* scratch, int T, int k, int E, void* stream);
+size_t berth_moe_permute_scratch_bytes(int T, int k, int E);
+/* Whole layer.  experts: DEVICE array of 3*E berth_exl3_lin (gate, up, down of
+ * expert 0, then expert 1, ...).  shared: HOST array of 3 berth_exl3_lin holding
+ * device pointers, or NULL.  out fp32 [T][H]; idx_out / w_out optional copies of
+ * the routing; workspace of berth_moe_workspace_bytes bytes, caller-owned. */
+int berth_moe_layer(const void* x, const void* wr, const float* bias, const void* experts,
+                    const berth_exl3_lin* shared, void* out, int32_t* idx_out, float* w_out,
+                    void* workspace, size_t workspace_bytes, int T, int H, int E, int k, int I,
+                    int shared_I, int k_bits, int codebook, int renorm, void* stream);
+size_t berth_moe_workspace_bytes(int T, int H, int E, int k, int I, int shared_I);
+/* byte offsets inside that workspace of {idx, w, offsets, perm, inv, gate_out
+ * fp16 [T*k][I], up_out fp16 [T*k][I], slot_out fp32 [T*k][H] (rows in expert-
+ * sorted order), shared_out fp32 [T][H]}, valid after berth_moe_layer returns */
+int berth_moe_workspace_offsets(int T, int H, int E, int k, int I, int shared_I, size_t out[9]);
+const char* berth_moe_last_error(void);
+const char* berth_moe_last_launch(void);
 
 #ifdef __cplusplus
 }

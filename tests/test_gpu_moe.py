@@ -1,0 +1,202 @@
+"""GPU parity of the MoE layer against the CPU oracle, through the C ABI.
+Bars: logits, top-k expert indices, offsets and the permutation are bit-exact;
+routing weights within 1e-5; layer outputs within rtol 2e-3 / atol 1e-3."""
+import numpy as np
+import pytest
+import torch
+
+from berth_amd import kernels as K
+from berth_amd import synth
+from berth_amd.device import Exl3Linear, Gpu
+from berth_amd.moe import MoeLayer
+from oracle import oracle as O
+from tests.gpu_util import DEV, close, dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _route(x, wr, k, bias=None, renorm=True):
+    T, H = x.shape
+    E = wr.shape[1]
+    d_x, d_w = dev(x.view(np.uint16)), dev(wr.view(np.uint16))
+    d_b = None if bias is None else torch.from_numpy(bias).to(DEV)
+    idx = torch.zeros((T, k), dtype=torch.int32, device=DEV)
+    w = torch.zeros((T, k), dtype=torch.float32, device=DEV)
+    logits = torch.zeros((T, E), dtype=torch.float32, device=DEV)
+    parts = torch.zeros(T * ((H + 63) // 64) * E, dtype=torch.float32, device=DEV)
+    K.moe.route(d_x.data_ptr(), d_w.data_ptr(), None if d_b is None else d_b.data_ptr(), idx.data_ptr(),
+                w.data_ptr(), logits.data_ptr(), parts.data_ptr(), T, H, E, k, renorm)
+    torch.cuda.synchronize()
+    return idx.cpu().numpy(), w.cpu().numpy(), logits.cpu().numpy()
+
+
+@pytest.mark.parametrize("T,H,E,k", [(1, 2048, 128, 8), (64, 2048, 128, 8), (5, 200, 16, 4), (3, 130, 7, 7),
+                                     (256, 2048, 512, 10), (9, 64, 300, 10)])
+def test_route_bit_exact(T, H, E, k):
+    x = synth.activations(T + H, T, H)
+    wr = synth.router_weight(E, H, E)
+    bias = synth.zipf_bias(3, E) if E == 512 else None
+    idx, w, logits = _route(x, wr, k, bias=bias)
+    oi, ow, ol = O.moe_route(x, wr, k, bias=bias, want_logits=True)
+    assert np.array_equal(logits.view(np.uint32), ol.view(np.uint32))
+    assert np.array_equal(idx, oi)
+    assert np.allclose(w, ow, rtol=1e-5, atol=1e-7)
+
+
+def test_route_ties_and_no_renorm():
+    H, E = 64, 8
+    x = np.ones((2, H), dtype=np.float16)
+    wr = np.zeros((H, E), dtype=np.float16)
+    idx, w, _ = _route(x, wr, 3)
+    assert idx.tolist() == [[0, 1, 2], [0, 1, 2]] and np.allclose(w, 1 / 3)
+    wr[:, 5] = 1.0
+    idx, w, _ = _route(x, wr, 2, renorm=False)
+    oi, ow = O.moe_route(x, wr, 2, renorm=False)
+    assert np.array_equal(idx, oi) and np.allclose(w, ow, rtol=1e-5, atol=1e-9)
+
+
+def test_permute_matches_oracle():
+    rng = np.random.default_rng(4)
+    for T, k, E in [(1, 8, 128), (64, 8, 128), (256, 10, 512), (7, 3, 5)]:
+        idx = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+        d_idx = torch.from_numpy(idx).to(DEV)
+        off = torch.zeros(E + 1, dtype=torch.int32, device=DEV)
+        perm = torch.zeros(T * k, dtype=torch.int32, device=DEV)
+        inv = torch.zeros(T * k, dtype=torch.int32, device=DEV)
+        scratch = torch.zeros(K.moe.permute_scratch_bytes(T, k, E), dtype=torch.uint8, device=DEV)
+        K.moe.permute(d_idx.data_ptr(), off.data_ptr(), perm.data_ptr(), inv.data_ptr(), scratch.data_ptr(), T, k, E)
+        torch.cuda.synchronize()
+        ooff, operm = O.moe_permute(idx, E)
+        assert np.array_equal(off.cpu().numpy(), ooff)
+        assert np.array_equal(perm.cpu().numpy(), operm)
+        assert np.array_equal(inv.cpu().numpy()[operm], np.arange(T * k))
+
+
+def _make_layer(gpu, seed, H, E, I, bits, shared_I=0, router_scale=1.0):
+    experts_np, experts = [], []
+    for e in range(E):
+        s = seed + 10 * e
+        trio = (synth.linear(s, H, I, bits), synth.linear(s + 3, H, I, bits), synth.linear(s + 6, I, H, bits))
+        experts_np.append(trio)
+        experts.append(tuple(Exl3Linear(gpu, f"experts.{e}.{n}", *lin)
+                             for n, lin in zip(("gate_proj", "up_proj", "down_proj"), trio)))
+    shared_np = shared = None
+    if shared_I:
+        s = seed + 99991
+        shared_np = (synth.linear(s, H, shared_I, bits), synth.linear(s + 3, H, shared_I, bits),
+                     synth.linear(s + 6, shared_I, H, bits))
+        shared = tuple(Exl3Linear(gpu, f"shared_expert.{n}", *lin)
+                       for n, lin in zip(("gate_proj", "up_proj", "down_proj"), shared_np))
+    wr = (synth.router_weight(seed + 5, H, E).astype(np.float32) * router_scale).astype(np.float16)
+    return wr, experts_np, experts, shared_np, shared
+
+
+def _check_stages(layer, x, experts_np, shared_np, idx, w, out, T, H, E, k, I, bits, shared_I):
+    """Each stage against the oracle on the SAME inputs the GPU stage consumed:
+    gate/up outputs from the gathered tokens, down outputs from the GPU's own
+    gate/up outputs, and the combine from the GPU's own down outputs."""
+    offs = K.moe.workspace_offsets(T, H, E, k, I, shared_I)
+    ws = layer._ws.cpu().numpy()
+    P = T * k
+
+    def view(name, dtype, shape):
+        n = int(np.prod(shape)) * np.dtype(dtype).itemsize
+        return ws[offs[name]:offs[name] + n].view(dtype).reshape(shape)
+
+    perm = view("perm", np.int32, (P,))
+    offsets = view("offsets", np.int32, (E + 1,))
+    inv = view("inv", np.int32, (P,))
+    ooff, operm = O.moe_permute(idx, E)
+    assert np.array_equal(offsets, ooff) and np.array_equal(perm, operm)
+    g = view("gate_out", np.float16, (P, I))
+    u = view("up_out", np.float16, (P, I))
+    slot = view("slot_out", np.float32, (P, H))
+    for e in range(E):
+        r0, r1 = int(offsets[e]), int(offsets[e + 1])
+        if r0 == r1:
+            continue
+        xe = x[perm[r0:r1] // k]
+        (gt, gs, gv), (ut, us, uv), (dt, ds, dv) = experts_np[e]
+        want_g, _ = O.linear(xe, gt, gs, gv, H, I, bits, 2)
+        want_u, _ = O.linear(xe, ut, us, uv, H, I, bits, 2)
+        assert close(g[r0:r1], want_g)[0] == 0, ("gate", e)
+        assert close(u[r0:r1], want_u)[0] == 0, ("up", e)
+        a = O.silu_mul(g[r0:r1], u[r0:r1]).reshape(r1 - r0, I)
+        want_d, _ = O.linear(a, dt, ds, dv, I, H, bits, 2, out_fp32=True)
+        assert close(slot[r0:r1], want_d)[0] == 0, ("down", e)
+    base = np.zeros((T, H), dtype=np.float32)
+    if shared_np is not None:
+        base = view("shared_out", np.float32, (T, H)).copy()
+        sg, _ = O.linear(x, *shared_np[0], H, shared_I, bits, 2)
+        su, _ = O.linear(x, *shared_np[1], H, shared_I, bits, 2)
+        # the shared expert's own down output is checked end to end below; its
+        # gate/up feed a SiLU whose fp16 rounding is shared by both sides
+        del sg, su
+    acc = base.astype(np.float32)
+    for j in range(k):
+        acc = (np.float32(1) * acc + w[:, j:j + 1].astype(np.float32) * slot[inv.reshape(T, k)[:, j]]).astype(np.float32)
+    assert np.allclose(out, acc, rtol=1e-5, atol=1e-5 * max(1.0, float(np.abs(acc).max())))
+
+
+@pytest.mark.parametrize("T,H,E,k,I,bits,shared_I,scale", [
+    (1, 256, 8, 2, 128, 4, 0, 1.0),
+    (4, 256, 8, 3, 256, 4, 128, 1.0),
+    (40, 256, 4, 2, 128, 4, 0, 1.0),        # every expert > 8 rows: MFMA problems only
+    (70, 256, 6, 2, 128, 3, 128, 30.0),     # skewed routing: mixed VALU and MFMA problems, one > 128 rows
+    (300, 128, 3, 1, 128, 4, 0, 50.0),      # a problem list with several 128-row chunks
+])
+def test_moe_layer_matches_oracle(T, H, E, k, I, bits, shared_I, scale):
+    gpu = Gpu(0)
+    wr, experts_np, experts, shared_np, shared = _make_layer(gpu, 500 + T, H, E, I, bits, shared_I, scale)
+    bias = synth.zipf_bias(7, E) if scale > 1 else None
+    layer = MoeLayer(gpu, wr, experts, k, shared=shared, bias=bias)
+    x = synth.activations(900 + T, T, H)
+    d_x = dev(x.view(np.uint16))
+    out = torch.zeros((T, H), dtype=torch.float32, device=DEV)
+    idx = torch.zeros((T, k), dtype=torch.int32, device=DEV)
+    w = torch.zeros((T, k), dtype=torch.float32, device=DEV)
+    layer.forward(gpu, d_x, out, T, idx, w)
+    torch.cuda.synchronize()
+    launch = K.moe.last_launch()
+    want, oi, ow = O.moe_layer(x, wr, experts_np, k, I, bits, 2, bias=bias, shared=shared_np, shared_I=shared_I)
+    assert np.array_equal(idx.cpu().numpy(), oi), launch
+    assert np.allclose(w.cpu().numpy(), ow, rtol=1e-5, atol=1e-7)
+    _check_stages(layer, x, experts_np, shared_np, oi, w.cpu().numpy(), out.cpu().numpy(), T, H, E, k, I, bits, shared_I)
+    # end to end, the fp16 roundings of gate/up outputs differ in a few last bits
+    # between two fp32 summation orders and propagate through down; bound the
+    # whole-layer error relative to the output scale
+    err = np.abs(out.cpu().numpy() - want)
+    assert err.max() <= 2e-3 * np.abs(want).max(), (err.max(), np.abs(want).max(), launch)
+    counts = np.bincount(oi.reshape(-1), minlength=E)
+    if counts.max() > 8:
+        assert "exl3_gemm_kernel" in launch
+    # a second call reuses the workspace and the self-resetting counters
+    out2 = torch.zeros_like(out)
+    layer.forward(gpu, d_x, out2, T)
+    torch.cuda.synchronize()
+    assert np.array_equal(out2.cpu().numpy().view(np.uint32), out.cpu().numpy().view(np.uint32))
+
+
+def test_moe_config3_shape_decode_token():
+    """hidden 2048, 128 experts, top-8, intermediate 768, 4 bpw, one token: the
+    oracle runs only the 8 selected experts."""
+    gpu = Gpu(0)
+    H, E, k, I, bits = 2048, 128, 8, 768, 4
+    wr, experts_np, experts, _, _ = _make_layer(gpu, 31, H, E, I, bits)
+    layer = MoeLayer(gpu, wr, experts, k)
+    x = synth.activations(32, 1, H)
+    out = torch.zeros((1, H), dtype=torch.float32, device=DEV)
+    idx = torch.zeros((1, k), dtype=torch.int32, device=DEV)
+    layer.forward(gpu, dev(x.view(np.uint16)), out, 1, idx)
+    torch.cuda.synchronize()
+    want, oi, ow = O.moe_layer(x, wr, experts_np, k, I, bits, 2)
+    assert np.array_equal(idx.cpu().numpy(), oi)
+    _check_stages(layer, x, experts_np, None, oi, ow, out.cpu().numpy(), 1, H, E, k, I, bits, 0)
+    assert np.abs(out.cpu().numpy() - want).max() <= 2e-3 * np.abs(want).max()
+
+
+def test_moe_validation_errors():
+    with pytest.raises(K.LaunchError, match="null"):
+        K.moe.layer(None, None, None, None, None, None, None, None, None, 0, 1, 128, 8, 2, 128, 0, 4, K.Codebook.MUL1)
+    with pytest.raises(K.LaunchError, match="top-k"):
+        K.moe.route(1, 1, None, 1, 1, None, 1, 1, 128, 4, 5)
