@@ -30,6 +30,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per GEMV launch of the default workload, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs scaled by a 1 GiB copy (profiles/exl3_gemv_4bpw_batch1_27b_linear_set.md)
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {4: int((24589 + 428) * 1024)}
 ORDER = ["q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"]
 OUT_FP32 = {"q_proj": False, "k_proj": False, "v_proj": False, "o_proj": True,
             "gate_proj": False, "up_proj": False, "down_proj": True}
@@ -63,6 +66,52 @@ def cpu_baseline(bits: int, seconds: float):
                       f"({K * N * reps / dt / 1e6:.0f} M weights/s)"}
 
 
+def moe_bench(gpu, steps: int, warmup: int):
+    """BASELINE.json configs[3]: hidden 2048, 128 experts, top-8 softmax routing,
+    expert intermediate 768, 4 bpw, router fp16 N(0, 0.02); batch 1 and 64.  One
+    call = route + permute + grouped gate/up + SiLU gate + grouped down + combine."""
+    import torch
+
+    from berth_amd import synth
+    from berth_amd.device import Exl3Linear
+    from berth_amd.moe import MoeLayer
+
+    H, E, k, I, bits = 2048, 128, 8, 768, 4
+    layers = []
+    for li in range(2):
+        experts = []
+        for e in range(E):
+            s = 100000 * (li + 1) + 10 * e
+            experts.append(tuple(Exl3Linear(gpu, f"layers.{li}.experts.{e}.{n}", *synth.linear(s + 3 * j, *shape, bits))
+                                 for j, (n, shape) in enumerate((("gate_proj", (H, I)), ("up_proj", (H, I)),
+                                                                 ("down_proj", (I, H))))))
+        layers.append(MoeLayer(gpu, synth.router_weight(77 + li, H, E), experts, k))
+    expert_bytes = 3 * H * I * bits // 8 + 2 * (2 * (H + I) + (I + H))
+    res = {}
+    for T in (1, 64):
+        xs = [gpu.upload(synth.activations(300 + i, T, H).view(np.uint16)) for i in range(16)]
+        out = torch.zeros((T, H), dtype=torch.float32, device=gpu.device)
+        idx = torch.zeros((T, k), dtype=torch.int32, device=gpu.device)
+        hit = 0
+        for i in range(16):
+            layers[i % 2].forward(gpu, xs[i], out, T, idx)
+            hit += len(np.unique(idx.cpu().numpy()))
+        hit /= 16.0
+        for i in range(warmup):
+            layers[i % 2].forward(gpu, xs[i % 16], out, T)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            layers[i % 2].forward(gpu, xs[i % 16], out, T)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        nbytes = 2 * H * E + hit * expert_bytes + 2 * T * H + 4 * T * H
+        res[f"T{T}"] = {"us_per_layer": round(dt / steps * 1e6, 2), "us_per_token": round(dt / steps / T * 1e6, 3),
+                        "experts_hit": round(hit, 1), "algorithmic_GBps": round(nbytes * steps / dt / 1e9, 1)}
+    res["config"] = "hidden 2048, 128 experts, top-8, intermediate 768, 4 bpw, mul1"
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -72,6 +121,10 @@ def main():
     ap.add_argument("--bits", type=int, default=4)
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-moe", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only a plain 1 GiB device copy kernel a few times (reference reading for "
+                         "the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path is single-GPU by design); "
@@ -88,6 +141,16 @@ def main():
     Kn.load()
     gpu = Gpu(0)
     bits = args.bits
+
+    if args.copy_calibration:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=gpu.device)     # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": {"bytes_read": src.numel() * 4, "bytes_written": src.numel() * 4,
+                                               "launches": 4}}))
+        return
 
     layers = []
     for li in range(args.layers):
@@ -146,11 +209,16 @@ def main():
                    "layers_rotated": len(layers), "bytes_per_step": step_bytes,
                    "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(bits) if len(layers) == 8 else None,
                      "kernel": Kn.last_launch().split(" grid=")[0],
                      "avg_launch_us": round(avg_launch_us, 3),
                      "bytes_per_launch": step_bytes // len(ORDER)},
     }
+    if not args.no_moe:
+        del layers
+        torch.cuda.empty_cache()
+        line["moe_layer"] = moe_bench(gpu, max(20, args.steps // 2), max(5, args.warmup // 2))
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(bits, args.cpu_seconds)
     print(json.dumps(line))
