@@ -153,14 +153,12 @@ __global__ __launch_bounds__(256) void exl3_gemv_kernel(GemvParams p)
         const half2_t sc = ((const half2_t*)(lin.suh + kb * 128))[lane];
 #pragma unroll
         for (int m = 0; m < MMAX; ++m) {
-            half2_t x = {(_Float16)0, (_Float16)0};
-            if (m < rows) {
-                x = ((const half2_t*)(p.a + (size_t)src[m] * p.K + kb * 128))[lane];
-                if (p.a_up) {
-                    const half2_t u = ((const half2_t*)(p.a_up + (size_t)src[m] * p.K + kb * 128))[lane];
-                    x.x = silu_mul_h(x.x, u.x);
-                    x.y = silu_mul_h(x.y, u.y);
-                }
+            if (MMAX > 1 && m >= rows) break;               // wave-uniform; rows past `rows` are never read
+            half2_t x = ((const half2_t*)(p.a + (size_t)src[m] * p.K + kb * 128))[lane];
+            if (p.a_up) {
+                const half2_t u = ((const half2_t*)(p.a_up + (size_t)src[m] * p.K + kb * 128))[lane];
+                x.x = silu_mul_h(x.x, u.x);
+                x.y = silu_mul_h(x.y, u.y);
             }
             float v0 = (float)x.x * (float)sc.x;
             float v1 = (float)x.y * (float)sc.y;
@@ -169,7 +167,7 @@ __global__ __launch_bounds__(256) void exl3_gemv_kernel(GemvParams p)
             r.x = (_Float16)(v0 * kRsqrt128);
             r.y = (_Float16)(v1 * kRsqrt128);
             xs[wave][m][lane] = as_u32(r);
-            if (p.a_had && nb == 0 && m < rows)
+            if (p.a_had && nb == 0)
                 ((half2_t*)(p.a_had + (size_t)(row0 + m) * p.K + kb * 128))[lane] = r;
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

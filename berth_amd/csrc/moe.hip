@@ -23,8 +23,9 @@ constexpr int kRouteSeg = 64;       // rows of the router weight per partial sum
 constexpr int kRouteTT = 4;         // tokens per route workgroup
 constexpr int kMaxExperts = 1024;
 constexpr int kMaxTopK = 32;
-constexpr int kValuRows = 8;        // experts with at most this many rows take the VALU kernel
-constexpr int kGemmRows = 128;      // rows per MFMA problem
+constexpr int kValuPairs = 8;       // calls with at most this many (token, slot) pairs use the VALU kernel only
+constexpr int kGemmRows = 32;       // rows per MFMA problem
+constexpr int kMaxPairsLds = 8192;  // pairs staged in LDS by the permute kernel
 
 // ------------------------------------------------------------------ route
 
@@ -97,8 +98,18 @@ __global__ __launch_bounds__(256) void moe_route_kernel(RouteParams p)
         if (e < p.E) {
             v = 0.0f;
             const float* src = p.parts + (size_t)t * p.nseg * p.E + e;
-            for (int sg = 0; sg < p.nseg; ++sg)
-                v += __hip_atomic_load(src + (size_t)sg * p.E, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // eight loads in flight at a time; the adds stay in segment order
+            for (int s0 = 0; s0 < p.nseg; s0 += 8) {
+                float part[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    part[j] = (s0 + j < p.nseg)
+                        ? __hip_atomic_load(src + (size_t)(s0 + j) * p.E, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                        : 0.0f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (s0 + j < p.nseg) v += part[j];
+            }
             if (p.bias) v += p.bias[e];
             if (p.logits) p.logits[(size_t)t * p.E + e] = v;
         }
@@ -152,57 +163,87 @@ struct PermuteParams {
     int32_t* offsets;       // [E + 1]
     int32_t* perm;          // [P] sorted position -> pair
     int32_t* inv;           // [P] pair -> sorted position
-    int32_t* row_rows;      // [P] sorted position -> number of rows of its expert
     int32_t* row_expert;    // [P] sorted position -> expert
     int32_t* counts;        // [2] number of VALU problems, number of MFMA problems
     GroupProblem* vprob;
     GroupProblem* mprob;
     int P, E;
+    int use_valu;           // 1: every expert is one VALU problem (P <= 8); 0: MFMA problems of <= 32 rows
 };
 
-// One workgroup.  Thread e scans the pairs in order and places those of expert
-// e: a stable counting sort whose result does not depend on scheduling.
+// One workgroup.  The pairs are cut into `parts` contiguous segments; thread
+// (part, e) counts and later places the pairs of expert e inside its segment, in
+// order: a stable counting sort whose result does not depend on scheduling.
 __global__ __launch_bounds__(1024) void moe_permute_kernel(PermuteParams p)
 {
-    __shared__ int cnt[kMaxExperts + 1];
+    __shared__ int cnt[1024];                   // [part][e]
+    __shared__ int base[1024];                  // first sorted position of (part, e)
     __shared__ int off[kMaxExperts + 1];
+    __shared__ int pfirst[kMaxExperts + 1];     // first problem index of each expert
+    __shared__ int s_idx[kMaxPairsLds];
     const int tid = threadIdx.x;
-    for (int e = tid; e <= p.E; e += 1024) cnt[e] = 0;
+    const bool staged = p.P <= kMaxPairsLds;
+    if (staged)
+        for (int q = tid; q < p.P; q += 1024) s_idx[q] = p.idx[q];
     __syncthreads();
-    for (int e = tid; e < p.E; e += 1024) {
+    const int* idx = staged ? s_idx : p.idx;
+    const int parts = max(1, 1024 / p.E);
+    const int seg = (p.P + parts - 1) / parts;
+    const int e = tid % p.E, part = tid / p.E;
+    const bool mine = part < parts;             // E <= 1024, so every expert has a thread
+    const int q0 = min(p.P, part * seg), q1 = min(p.P, q0 + seg);
+    if (mine) {
         int c = 0;
-        for (int q = 0; q < p.P; ++q) c += (p.idx[q] == e);
-        cnt[e] = c;
+#pragma unroll 8
+        for (int q = q0; q < q1; ++q) c += (idx[q] == e);
+        cnt[part * p.E + e] = c;
+    }
+    __syncthreads();
+    if (tid < p.E) {                            // total of expert tid, kept in pfirst for now
+        int c = 0;
+        for (int pt = 0; pt < parts; ++pt) c += cnt[pt * p.E + tid];
+        pfirst[tid] = c;
     }
     __syncthreads();
     if (tid == 0) {
-        int run = 0, nv = 0, nm = 0;
-        for (int e = 0; e < p.E; ++e) {
-            off[e] = run;
-            const int m = cnt[e];
-            if (m > 0 && m <= kValuRows) {
-                p.vprob[nv++] = GroupProblem{e, run, m, 0};
-            } else if (m > kValuRows) {
-                for (int r = 0; r < m; r += kGemmRows)
-                    p.mprob[nm++] = GroupProblem{e, run + r, min(kGemmRows, m - r), 0};
-            }
+        int run = 0, np = 0;
+        for (int x = 0; x < p.E; ++x) {
+            const int m = pfirst[x];
+            off[x] = run;
+            pfirst[x] = np;
+            if (m > 0) np += p.use_valu ? 1 : (m + kGemmRows - 1) / kGemmRows;
             run += m;
         }
         off[p.E] = run;
-        p.counts[0] = nv;
-        p.counts[1] = nm;
+        pfirst[p.E] = np;
+        p.counts[0] = p.use_valu ? np : 0;
+        p.counts[1] = p.use_valu ? 0 : np;
     }
     __syncthreads();
-    for (int e = tid; e <= p.E; e += 1024) p.offsets[e] = off[e];
-    for (int e = tid; e < p.E; e += 1024) {
-        int at = off[e];
-        const int m = cnt[e];
-        if (!m) continue;
-        for (int q = 0; q < p.P; ++q) {
-            if (p.idx[q] == e) {
+    for (int x = tid; x <= p.E; x += 1024) p.offsets[x] = off[x];
+    if (tid < p.E) {
+        int run = off[tid];
+        for (int pt = 0; pt < parts; ++pt) {
+            base[pt * p.E + tid] = run;
+            run += cnt[pt * p.E + tid];
+        }
+        const int m = off[tid + 1] - off[tid];
+        if (m > 0) {
+            if (p.use_valu) {
+                p.vprob[pfirst[tid]] = GroupProblem{tid, off[tid], m, 0};
+            } else {
+                for (int r = 0, j = pfirst[tid]; r < m; r += kGemmRows, ++j)
+                    p.mprob[j] = GroupProblem{tid, off[tid] + r, min(kGemmRows, m - r), 0};
+            }
+        }
+    }
+    __syncthreads();
+    if (mine && cnt[part * p.E + e] > 0) {
+        int at = base[part * p.E + e];
+        for (int q = q0; q < q1; ++q) {
+            if (idx[q] == e) {
                 p.perm[at] = q;
                 p.inv[q] = at;
-                p.row_rows[at] = m;
                 p.row_expert[at] = e;
                 ++at;
             }
@@ -217,7 +258,6 @@ struct HadRowsParams {
     const _Float16* a_up;       // with a_up: input = silu(a[r]) * a_up[r]
     const int32_t* gather;      // source row = gather[r] / gather_div, or r
     int gather_div;
-    const int32_t* row_rows;
     const int32_t* row_expert;
     const ExpertLin* experts;
     int lins_per_expert, lin_base;
@@ -229,7 +269,6 @@ __global__ __launch_bounds__(256) void moe_had_rows_kernel(HadRowsParams p)
 {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = blockIdx.y;
-    if (p.row_rows[r] <= kValuRows) return;            // that expert takes the VALU kernel
     const int kb = blockIdx.x * 4 + wave;
     if (kb * 128 >= p.K) return;
     const int which = blockIdx.z;
@@ -279,7 +318,7 @@ thread_local std::string g_moe_err, g_moe_launch;
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct MoeLayout {
-    size_t idx, w, parts, offsets, perm, inv, row_rows, row_expert, counts, vprob, mprob;
+    size_t idx, w, parts, offsets, perm, inv, row_expert, counts, vprob, mprob;
     size_t ah0, ah1, g, u, ahd, slot_out, sg, su, s_ahad, shared_out, total;
     int max_v, max_m, nseg;
 };
@@ -289,8 +328,9 @@ MoeLayout moe_layout(int T, int H, int E, int k, int I, int shared_I)
     MoeLayout L{};
     const size_t P = (size_t)T * k;
     L.nseg = (H + kRouteSeg - 1) / kRouteSeg;
-    L.max_v = (int)std::min<size_t>((size_t)E, P);
-    L.max_m = P > (size_t)kValuRows ? (int)(P / (kValuRows + 1) + P / kGemmRows + 1) : 0;
+    const bool use_valu = P <= (size_t)kValuPairs;
+    L.max_v = use_valu ? (int)std::min<size_t>((size_t)E, P) : 0;
+    L.max_m = use_valu ? 0 : (int)(std::min<size_t>((size_t)E, P) + P / kGemmRows + 1);
     size_t at = 0;
     auto take = [&](size_t bytes) { size_t r = at; at = align_up(at + bytes); return r; };
     L.idx = take(P * 4);
@@ -299,10 +339,9 @@ MoeLayout moe_layout(int T, int H, int E, int k, int I, int shared_I)
     L.offsets = take((size_t)(E + 1) * 4);
     L.perm = take(P * 4);
     L.inv = take(P * 4);
-    L.row_rows = take(P * 4);
     L.row_expert = take(P * 4);
     L.counts = take(16);
-    L.vprob = take((size_t)L.max_v * sizeof(GroupProblem));
+    L.vprob = take((size_t)std::max(L.max_v, 1) * sizeof(GroupProblem));
     L.mprob = take((size_t)std::max(L.max_m, 1) * sizeof(GroupProblem));
     L.ah0 = take(L.max_m ? P * H * 2 : 0);
     L.ah1 = take(L.max_m ? P * H * 2 : 0);
@@ -358,13 +397,13 @@ std::string run_permute(const int32_t* idx, unsigned char* wsb, const MoeLayout&
     p.offsets = (int32_t*)(wsb + L.offsets);
     p.perm = (int32_t*)(wsb + L.perm);
     p.inv = (int32_t*)(wsb + L.inv);
-    p.row_rows = (int32_t*)(wsb + L.row_rows);
     p.row_expert = (int32_t*)(wsb + L.row_expert);
     p.counts = (int32_t*)(wsb + L.counts);
     p.vprob = (GroupProblem*)(wsb + L.vprob);
     p.mprob = (GroupProblem*)(wsb + L.mprob);
     p.P = P;
     p.E = E;
+    p.use_valu = L.max_v > 0 ? 1 : 0;
     hipLaunchKernelGGL(moe_permute_kernel, dim3(1), dim3(1024), 0, stream, p);
     hip_ok(hipGetLastError(), "moe_permute_kernel launch");
     return "moe_permute_kernel";
@@ -427,13 +466,13 @@ extern "C" int berth_moe_permute(const int32_t* idx, int32_t* offsets, int32_t* 
     p.perm = perm;
     p.inv = inv;
     size_t at = 0;
-    p.row_rows = (int32_t*)(sb + at); at = align_up(at + P * 4);
     p.row_expert = (int32_t*)(sb + at); at = align_up(at + P * 4);
     p.counts = (int32_t*)(sb + at); at = align_up(at + 16);
     p.vprob = (GroupProblem*)(sb + at); at = align_up(at + (std::min<size_t>(E, P)) * sizeof(GroupProblem));
     p.mprob = (GroupProblem*)(sb + at);
     p.P = (int)P;
     p.E = E;
+    p.use_valu = P <= (size_t)kValuPairs ? 1 : 0;
     hipLaunchKernelGGL(moe_permute_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, p);
     hip_ok(hipGetLastError(), "moe_permute_kernel launch");
     g_moe_launch = "moe_permute_kernel";
@@ -446,10 +485,9 @@ extern "C" size_t berth_moe_permute_scratch_bytes(int T, int k, int E)
     const size_t P = (size_t)T * k;
     size_t at = 0;
     at = align_up(at + P * 4);
-    at = align_up(at + P * 4);
     at = align_up(at + 16);
     at = align_up(at + std::min<size_t>(E, P) * sizeof(GroupProblem));
-    at = align_up(at + (P / (kValuRows + 1) + P / kGemmRows + 2) * sizeof(GroupProblem));
+    at = align_up(at + (std::min<size_t>(E, P) + P / kGemmRows + 2) * sizeof(GroupProblem));
     return at;
 }
 
@@ -502,16 +540,17 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
     g.size_k = H;
     g.size_n = I;
     g.out_fp32 = 0;
-    g.problems = wsb + L.vprob;
-    g.num_problems = (const int*)(wsb + L.counts);
-    g.max_problems = L.max_v;
-    desc += " + " + launch_gemv_grouped(g);
+    if (L.max_v > 0) {
+        g.problems = wsb + L.vprob;
+        g.num_problems = (const int*)(wsb + L.counts);
+        g.max_problems = L.max_v;
+        desc += " + " + launch_gemv_grouped(g);
+    }
     if (L.max_m > 0) {
         HadRowsParams h{};
         h.a = (const _Float16*)x;
         h.gather = (const int32_t*)(wsb + L.perm);
         h.gather_div = k;
-        h.row_rows = (const int32_t*)(wsb + L.row_rows);
         h.row_expert = (const int32_t*)(wsb + L.row_expert);
         h.experts = (const ExpertLin*)experts;
         h.lins_per_expert = 3;
@@ -542,16 +581,17 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
     g.size_k = I;
     g.size_n = H;
     g.out_fp32 = 1;
-    g.problems = wsb + L.vprob;
-    g.num_problems = (const int*)(wsb + L.counts);
-    g.max_problems = L.max_v;
-    desc += " + " + launch_gemv_grouped(g);
+    if (L.max_v > 0) {
+        g.problems = wsb + L.vprob;
+        g.num_problems = (const int*)(wsb + L.counts);
+        g.max_problems = L.max_v;
+        desc += " + " + launch_gemv_grouped(g);
+    }
     if (L.max_m > 0) {
         HadRowsParams h{};
         h.a = (const _Float16*)(wsb + L.g);
         h.a_up = (const _Float16*)(wsb + L.u);
         h.gather_div = 1;
-        h.row_rows = (const int32_t*)(wsb + L.row_rows);
         h.row_expert = (const int32_t*)(wsb + L.row_expert);
         h.experts = (const ExpertLin*)experts;
         h.lins_per_expert = 3;

@@ -194,6 +194,17 @@ def test_gemm_other_rates(bits, cb):
     assert bad == 0, (bad, worst)
 
 
+@pytest.mark.parametrize("m,Kk,N", [(16, 4096, 256), (24, 5120, 1024), (32, 2048, 768), (33, 2048, 512), (100, 4096, 256)])
+def test_gemm_split_k(m, Kk, N):
+    got, want, ah, want_ah, launch = _run_linear(m, Kk, N, 4, 2, True, 300 + m, prefill=True)
+    assert "split_k=" in launch and "split_k=1 " not in launch, launch
+    assert np.array_equal(ah, want_ah)
+    bad, worst = close(got, want)
+    assert bad == 0, (bad, worst, launch)
+    got2, _, _, _, _ = _run_linear(m, Kk, N, 4, 2, True, 300 + m, prefill=True)
+    assert np.array_equal(got.view(np.uint32), got2.view(np.uint32))
+
+
 def test_linear_through_decode_entry_with_many_rows():
     """forward_n passes rows 2..144 of a K = 6 linear to the m = 1 entry
     (crates/berth-engine/src/device.rs:338-352)."""
