@@ -5,8 +5,10 @@ Workload (BASELINE.json configs[1] at the bit rate the metric is quoted on): the
 dense 27B-shaped decode linear set at batch 1, 4 bpw, mul1 codebook — q_proj
 5120x6144, k/v_proj 5120x1024, o_proj 6144x5120, gate/up 5120x17408, down
 17408x5120 — fp16 activations N(0,1), uniform random trellis words, suh/svh
-random signs times lognormal(0,0.1).  One step = the seven linears of one layer,
-each through berth_exl3_linear (one fused kernel launch per linear).  Steps rotate
+random signs times lognormal(0,0.1).  One step = the seven linears of one layer in
+four launches: q/k/v as one sliced multi-linear (berth_ops_mgemm, as the
+reference bundles them), o_proj (berth_exl3_linear), gate+up as one multi-linear,
+down_proj.  Steps rotate
 over `--layers` distinct weight sets (default 8 = 1.36 GB) so that reads come
 from HBM, not from the 256 MB memory-side cache.  Inputs are resident in HBM
 before the timed region.
@@ -122,6 +124,7 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-moe", action="store_true")
+    ap.add_argument("--unfused", action="store_true", help="seven separate launches instead of four")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 1 GiB device copy kernel a few times (reference reading for "
                          "the FETCH_SIZE / WRITE_SIZE counters)")
@@ -135,7 +138,7 @@ def main():
 
     from berth_amd import kernels as Kn
     from berth_amd import synth
-    from berth_amd.device import Exl3Linear, Gpu
+    from berth_amd.device import Exl3Linear, Exl3MultiLinear, Gpu
     from berth_amd.kernels import OutDtype
 
     Kn.load()
@@ -159,6 +162,9 @@ def main():
             K, N = synth.SHAPES_27B[name]
             tr, suh, svh = synth.linear(1000 * li + 10 * j, K, N, bits)
             lin[name] = Exl3Linear(gpu, f"layers.{li}.{name}", tr, suh, svh)
+        if not args.unfused:
+            lin["qkv"] = Exl3MultiLinear(gpu, [lin["q_proj"], lin["k_proj"], lin["v_proj"]])
+            lin["gate_up"] = Exl3MultiLinear(gpu, [lin["gate_proj"], lin["up_proj"]])
         layers.append(lin)
 
     xin = {K: gpu.upload(synth.activations(5, 1, K).view(np.uint16)) for K in (5120, 6144, 17408)}
@@ -167,11 +173,20 @@ def main():
 
     step_bytes = sum(linear_bytes(*synth.SHAPES_27B[n], bits, 1, 4 if OUT_FP32[n] else 2) for n in ORDER)
 
+    f16, f32 = OutDtype.F16, OutDtype.F32
+    launches_per_step = len(ORDER) if args.unfused else 4
+
     def step(i):
         lin = layers[i % len(layers)]
-        for name in ORDER:
-            l = lin[name]
-            l.forward(gpu, xin[l.size_k], outs[name], OutDtype.F32 if OUT_FP32[name] else OutDtype.F16)
+        if args.unfused:
+            for name in ORDER:
+                l = lin[name]
+                l.forward(gpu, xin[l.size_k], outs[name], f32 if OUT_FP32[name] else f16)
+            return
+        lin["qkv"].forward(gpu, xin[5120], [outs["q_proj"], outs["k_proj"], outs["v_proj"]], f16)
+        lin["o_proj"].forward(gpu, xin[6144], outs["o_proj"], f32)
+        lin["gate_up"].forward(gpu, xin[5120], [outs["gate_proj"], outs["up_proj"]], f16)
+        lin["down_proj"].forward(gpu, xin[17408], outs["down_proj"], f32)
 
     for i in range(args.warmup):
         step(i)
@@ -188,7 +203,7 @@ def main():
     ms_per_step = wall_ms / args.steps
     value = step_bytes * args.steps / (wall_ms * 1e-3) / 1e9
 
-    launches = args.steps * len(ORDER)
+    launches = args.steps * launches_per_step
     avg_launch_us = ev_ms * 1e3 / launches
     achieved = step_bytes * args.steps / (ev_ms * 1e-3) / 1e9
 
@@ -210,10 +225,10 @@ def main():
                    "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(bits) if len(layers) == 8 else None,
+                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(bits) if len(layers) == 8 and not args.unfused else None,
                      "kernel": Kn.last_launch().split(" grid=")[0],
                      "avg_launch_us": round(avg_launch_us, 3),
-                     "bytes_per_launch": step_bytes // len(ORDER)},
+                     "bytes_per_launch": step_bytes // launches_per_step},
     }
     if not args.no_moe:
         del layers

@@ -238,5 +238,49 @@ extern "C" int berth_ops_silu_mul(const void* gate, const void* up, void* out, i
     }
 }
 
+// crates/berth-kernels/csrc/ops/mgemm.cu:125-272,296-340: same checks in the same order
+extern "C" int berth_ops_mgemm(const void* a, const void* b_list, void* c, const void* suh_list,
+                               void* a_had, const void* svh_list, int size_m, int size_k, int size_n,
+                               int k_bits, int codebook, int c_fp32, int bszm_in, int bszm_out,
+                               const int* size_n_list, const void* c_ptrs, const int* n_stride_list,
+                               const int* had_src_list, int num_had_src, void* stream)
+{
+    try {
+        g_ops_err.clear();
+        g_ops_launch.clear();
+        if (!a || !b_list || !c || !suh_list || !a_had || !svh_list)
+            throw std::runtime_error("exl3_mgemm: null device pointer");
+        if (size_m < 1 || size_k < 1 || size_n < 1 || bszm_in < 1 || bszm_out < 1)
+            throw std::runtime_error("exl3_mgemm: sizes must be positive");
+        if (size_k % 16 != 0) throw std::runtime_error("exl3_mgemm: size_k must be a multiple of 16");
+        if (size_n % 128 != 0) throw std::runtime_error("exl3_mgemm: size_n must be a multiple of 128");
+        if (k_bits < 1 || k_bits > 8) throw std::runtime_error("exl3_mgemm: K must be in 1..=8");
+        if (codebook < 0 || codebook > 2) throw std::runtime_error("exl3_mgemm: codebook must be 0, 1, or 2");
+        if (c_fp32 != 0 && c_fp32 != 1) throw std::runtime_error("exl3_mgemm: c_fp32 must be 0 (fp16) or 1 (fp32)");
+        const bool any_list = size_n_list || c_ptrs || n_stride_list || had_src_list;
+        if (any_list) {
+            if (!size_n_list || !c_ptrs || !n_stride_list || !had_src_list)
+                throw std::runtime_error(
+                    "exl3_mgemm: sliced mode requires size_n_list, c_ptrs, n_stride_list, and had_src_list");
+            if (num_had_src < 1) throw std::runtime_error("exl3_mgemm: sliced mode needs one suh entry per source");
+            if (bszm_in != 1) throw std::runtime_error("exl3_mgemm: sliced mode is single-input");
+        } else {
+            if (num_had_src != 0) throw std::runtime_error("exl3_mgemm: num_had_src requires had_src_list");
+            if (bszm_in != 1 && bszm_in != bszm_out)
+                throw std::runtime_error("exl3_mgemm: bszm_in must be 1 or equal to bszm_out");
+        }
+        MgemmArgs m{a, b_list, c, suh_list, a_had, svh_list, size_m, size_k, size_n, k_bits, codebook, c_fp32,
+                    bszm_in, bszm_out, size_n_list, c_ptrs, n_stride_list, had_src_list, num_had_src,
+                    (hipStream_t)stream};
+        g_ops_launch = launch_mgemm(m);
+        return 1;
+    } catch (const std::exception& err) {
+        g_ops_err = err.what();
+        g_ops_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
 extern "C" const char* berth_ops_last_error(void) { return g_ops_err.c_str(); }
 extern "C" const char* berth_ops_last_launch(void) { return g_ops_launch.c_str(); }

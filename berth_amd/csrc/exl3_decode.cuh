@@ -36,6 +36,18 @@ constexpr float kRsqrt128 = 0.088388347648f;  // crates/berth-kernels/csrc/prefi
 __host__ __device__ constexpr int pair_col_half(int p) { return (p >> 1) & 1; }          // f
 __host__ __device__ constexpr int pair_kk(int p) { return (p >> 2) + 4 * (p & 1); }      // k/2 in the tile
 
+// Pointers that reach a kernel through memory (device tables of pointers) lose
+// their address space; these casts restore "global" so that loads and stores are
+// global_* instructions rather than flat_* ones.
+#ifndef BERTH_HOST_EMU
+template <typename T>
+using global_ptr = __attribute__((address_space(1))) T*;
+template <typename T>
+__device__ __forceinline__ global_ptr<const T> as_global(const T* p) { return (global_ptr<const T>)p; }
+template <typename T>
+__device__ __forceinline__ global_ptr<T> as_global(T* p) { return (global_ptr<T>)p; }
+#endif
+
 __device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
 __device__ __forceinline__ uint32_t as_u32(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
 
@@ -125,16 +137,17 @@ __device__ __forceinline__ void decode_lane(const uint32_t (&own)[BITS], uint32_
         w2[p] = decode_pair<CB>(win.state(2 * p), win.state(2 * p + 1));
 }
 
-// byte address, for ds_bpermute, of the lane that owns the previous 32 stream
-// positions of the same tile (octet-local rotate by one)
-__device__ __forceinline__ int prev_lane_addr(int lane)
+// The dword just before a lane's own dwords belongs to the previous lane of its
+// octet (octet-local rotate by one: lane u = 0 takes it from lane u = 7).  Two DPP
+// moves inside the 16-lane row and a select; no LDS traffic.
+#ifndef BERTH_HOST_EMU
+__device__ __forceinline__ uint32_t fetch_prev(int lane, uint32_t last_own)
 {
-    return ((lane & ~7) | ((lane + 7) & 7)) << 2;
+    const int v = (int)last_own;
+    const int from_below = __builtin_amdgcn_update_dpp(v, v, 0x111, 0xF, 0xF, false);   // row_shr:1, lane i <- i-1
+    const int from_above = __builtin_amdgcn_update_dpp(v, v, 0x107, 0xF, 0xF, false);   // row_shl:7, lane i <- i+7
+    return (uint32_t)((lane & 7) ? from_below : from_above);
 }
-
-__device__ __forceinline__ uint32_t fetch_prev(int addr, uint32_t last_own)
-{
-    return (uint32_t)__builtin_amdgcn_ds_bpermute(addr, (int)last_own);
-}
+#endif
 
 }  // namespace berth

@@ -85,7 +85,6 @@ __global__ __launch_bounds__(256) void exl3_gemm_kernel(GemmParams p)
     const int tn = p.N >> 4;
     constexpr int tile_dw = 8 * BITS;
     const size_t row_dw = (size_t)tn * tile_dw;
-    const int paddr = prev_lane_addr(lane);
     const int KB = p.K >> 7;
 
     float16_t acc[MB][2];
@@ -142,7 +141,7 @@ __global__ __launch_bounds__(256) void exl3_gemm_kernel(GemmParams p)
         if (active) {
 #pragma unroll
             for (int st = 0; st < 4; ++st) {
-                uint32_t prev = fetch_prev(paddr, cur[st][BITS - 1]);
+                uint32_t prev = fetch_prev(lane, cur[st][BITS - 1]);
                 uint32_t w2[16];
                 decode_lane<BITS, CB>(cur[st], prev, w2);
                 half8_t b[2][2];

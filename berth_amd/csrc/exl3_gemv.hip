@@ -22,38 +22,17 @@
 
 namespace berth {
 
-template <int BITS, int CB>
-static void launch_rows(const GemvParams& p, int mmax, dim3 grid, hipStream_t stream)
-{
-    switch (mmax) {
-    case 1: hipLaunchKernelGGL((exl3_gemv_kernel<BITS, CB, 1>), grid, dim3(256), 0, stream, p); break;
-    case 2: hipLaunchKernelGGL((exl3_gemv_kernel<BITS, CB, 2>), grid, dim3(256), 0, stream, p); break;
-    case 4: hipLaunchKernelGGL((exl3_gemv_kernel<BITS, CB, 4>), grid, dim3(256), 0, stream, p); break;
-    default: hipLaunchKernelGGL((exl3_gemv_kernel<BITS, CB, 8>), grid, dim3(256), 0, stream, p); break;
-    }
-}
-
-template <int BITS>
-static void launch_cb(const GemvParams& p, int cb, int mmax, dim3 grid, hipStream_t stream)
-{
-    switch (cb) {
-    case 0: launch_rows<BITS, 0>(p, mmax, grid, stream); break;
-    case 1: launch_rows<BITS, 1>(p, mmax, grid, stream); break;
-    default: launch_rows<BITS, 2>(p, mmax, grid, stream); break;
-    }
-}
+// one translation unit per codebook (exl3_gemv_cb{0,1,2}.hip) keeps the build parallel
+void launch_gemv_cb0(const GemvParams& p, int bits, int mmax, dim3 grid, hipStream_t stream);
+void launch_gemv_cb1(const GemvParams& p, int bits, int mmax, dim3 grid, hipStream_t stream);
+void launch_gemv_cb2(const GemvParams& p, int bits, int mmax, dim3 grid, hipStream_t stream);
 
 static void launch_bits(const GemvParams& p, int bits, int cb, int mmax, dim3 grid, hipStream_t stream)
 {
-    switch (bits) {
-    case 1: launch_cb<1>(p, cb, mmax, grid, stream); break;
-    case 2: launch_cb<2>(p, cb, mmax, grid, stream); break;
-    case 3: launch_cb<3>(p, cb, mmax, grid, stream); break;
-    case 4: launch_cb<4>(p, cb, mmax, grid, stream); break;
-    case 5: launch_cb<5>(p, cb, mmax, grid, stream); break;
-    case 6: launch_cb<6>(p, cb, mmax, grid, stream); break;
-    case 7: launch_cb<7>(p, cb, mmax, grid, stream); break;
-    default: launch_cb<8>(p, cb, mmax, grid, stream); break;
+    switch (cb) {
+    case 0: launch_gemv_cb0(p, bits, mmax, grid, stream); break;
+    case 1: launch_gemv_cb1(p, bits, mmax, grid, stream); break;
+    default: launch_gemv_cb2(p, bits, mmax, grid, stream); break;
     }
 }
 
@@ -67,12 +46,13 @@ static int wg_per_cu()
     return v;
 }
 
-// split-K factor: enough workgroups to cover the chip several times, at most one
-// k-block per wave, within the workspace
+// split-K factor: about wg_per_cu workgroups per compute unit (2-3 waves per SIMD
+// keep the vector ALU busy; each wave then walks several k-blocks with its loads
+// one k-block ahead), at most one k-block per wave, within the workspace
 static int pick_split(const Workspace& ws, long units, int KB, int mmax)
 {
     const long target_wg = (long)ws.cu_count * wg_per_cu();
-    long S = (target_wg + units - 1) / units;
+    long S = (target_wg + units / 2) / units;
     const int s_max = (KB + 3) / 4;
     if (S > s_max) S = s_max;
     if (S < 1) S = 1;
@@ -85,7 +65,7 @@ std::string launch_gemv(const LinearArgs& a)
     if (a.size_m < 1 || a.size_m > 8) throw std::runtime_error("exl3 gemv: rows must be in 1..=8");
     if (a.size_k % 128 != 0) throw std::runtime_error("exl3 linear: size_k must be a multiple of 128");
     Workspace& ws = workspace_for_current_device();
-    const int mmax = a.size_m == 1 ? 1 : a.size_m == 2 ? 2 : a.size_m <= 4 ? 4 : 8;
+    const int mmax = a.size_m == 1 ? 1 : 8;
 
     GemvParams p{};
     p.a = (const _Float16*)a.a;
@@ -110,6 +90,46 @@ std::string launch_gemv(const LinearArgs& a)
     return "exl3_gemv_kernel<" + std::to_string(a.k_bits) + "," + std::to_string(a.codebook) + "," +
            std::to_string(mmax) + "> grid=" + std::to_string(grid) + " block=256 split_k=" +
            std::to_string(p.S) + (a.out_fp32 ? " out=f32" : " out=f16");
+}
+
+std::string launch_mgemm(const MgemmArgs& m)
+{
+    if (m.size_k % 128 != 0) throw std::runtime_error("exl3_mgemm: size_k must be a multiple of 128");
+    if (m.size_m > 8) throw std::runtime_error("exl3_mgemm: more than 8 rows is not built (use one linear per call)");
+    Workspace& ws = workspace_for_current_device();
+    const bool sliced = m.had_src_list != nullptr;
+    const int mmax = m.size_m == 1 ? 1 : 8;
+    GemvParams p{};
+    p.a = (const _Float16*)m.a;
+    p.rows = m.size_m;
+    p.c[0] = m.c;
+    p.a_had = (_Float16*)m.a_had;
+    p.b_list = (const uint64_t*)m.b_list;
+    p.suh_list = (const uint64_t*)m.suh_list;
+    p.svh_list = (const uint64_t*)m.svh_list;
+    p.c_ptrs = (const uint64_t*)m.c_ptrs;
+    p.size_n_list = m.size_n_list;
+    p.n_stride_list = m.n_stride_list;
+    p.had_src_list = m.had_src_list;
+    p.multi = sliced ? 2 : 1;
+    p.multi_in_rows = (!sliced && m.bszm_in > 1) ? m.size_m : 0;
+    p.partials = ws.partials;
+    p.counters = ws.counters;
+    p.K = m.size_k;
+    p.N = m.size_n;
+    p.NB = m.size_n / 128;
+    p.KB = m.size_k / 128;
+    p.out_fp32 = m.c_fp32;
+    const long units = (long)m.bszm_out * p.NB;
+    if (units > kCounters) throw std::runtime_error("exl3_mgemm: too many (slice, column block) units");
+    p.S = pick_split(ws, units, p.KB, mmax);
+    dim3 grid((unsigned)(m.bszm_out * p.NB * p.S));
+    launch_bits(p, m.k_bits, m.codebook, mmax, grid, m.stream);
+    hip_ok(hipGetLastError(), "exl3_gemv_kernel multi launch");
+    return "exl3_gemv_kernel<" + std::to_string(m.k_bits) + "," + std::to_string(m.codebook) + "," +
+           std::to_string(mmax) + "> " + (sliced ? "sliced" : "uniform") + " x" + std::to_string(m.bszm_out) +
+           " grid=" + std::to_string(grid.x) + " block=256 split_k=" + std::to_string(p.S) +
+           (m.c_fp32 ? " out=f32" : " out=f16");
 }
 
 std::string launch_gemv_grouped(const GroupedArgs& g)

@@ -57,6 +57,19 @@ struct GemvParams {
     const int* num_problems;
     int lins_per_expert;
     int lin_base;
+    // multi-linear mode (multi != 0), the argument lists of
+    // crates/berth-kernels/src/ops.rs:264-293, all device arrays: one problem per
+    // entry of b_list; multi == 2 is the sliced form (per-slice width, row stride
+    // and source index; outputs through c_ptrs), multi == 1 the uniform form
+    const uint64_t* b_list;
+    const uint64_t* suh_list;
+    const uint64_t* svh_list;
+    const uint64_t* c_ptrs;
+    const int* size_n_list;
+    const int* n_stride_list;
+    const int* had_src_list;
+    int multi;
+    int multi_in_rows;          // rows between the inputs of consecutive problems (0: shared input)
     void* c[2];                 // output per blockIdx.y, rows in problem order
     _Float16* a_had;            // optional (dense mode only)
     float* partials;            // [problem][lin][NB][S][MMAX][128]
@@ -75,38 +88,153 @@ __device__ __forceinline__ _Float16 silu_mul_h(_Float16 g, _Float16 u)
     return t * u;
 }
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
 template <int BITS>
-__device__ __forceinline__ void load_tile_dwords(const uint32_t* __restrict__ p, uint32_t (&out)[BITS])
+__device__ __forceinline__ void load_tile_dwords(global_ptr<const uint32_t> p, uint32_t (&out)[BITS])
 {
     if constexpr (BITS % 4 == 0) {
-        const uint4* q = (const uint4*)p;
 #pragma unroll
         for (int j = 0; j < BITS / 4; ++j) {
-            uint4 v = q[j];
+            const u32x4_t v = *((global_ptr<const u32x4_t>)p + j);
             out[4 * j] = v.x; out[4 * j + 1] = v.y; out[4 * j + 2] = v.z; out[4 * j + 3] = v.w;
         }
     } else if constexpr (BITS % 2 == 0) {
-        const uint2* q = (const uint2*)p;
 #pragma unroll
         for (int j = 0; j < BITS / 2; ++j) {
-            uint2 v = q[j];
+            const u32x2_t v = *((global_ptr<const u32x2_t>)p + j);
             out[2 * j] = v.x; out[2 * j + 1] = v.y;
         }
     } else {
 #pragma unroll
-        for (int j = 0; j < BITS; ++j) out[j] = p[j];
+        for (int j = 0; j < BITS; ++j) out[j] = *((global_ptr<const uint32_t>)p + j);
     }
 }
 
-template <int BITS, int CB, int MMAX>
-__global__ __launch_bounds__(256) void exl3_gemv_kernel(GemvParams p)
+// what one wave needs to walk its k-blocks
+struct GemvWalk {
+    global_ptr<const uint32_t> tbase;   // tile row 0 of the wave's column block
+    global_ptr<const half2_t> suh;
+    global_ptr<const _Float16> a;
+    global_ptr<const _Float16> a_up;
+    global_ptr<_Float16> a_had;         // row 0 of this problem's slab
+    size_t row_dw;                      // dwords per tile row
+    int K, KB, kb0, step, rows;
+};
+
+// The K loop of one wave.  Rolling prefetch: the 8 tile rows of a k-block live in
+// registers; as soon as a tile row has been decoded its registers are reloaded
+// with the same tile row of the wave's next k-block, so loads stay one k-block
+// ahead of the decode.  The loop body is straight-line code with loads only (the
+// a_had store lives in its own instantiation, used by the column-block-0
+// workgroups): with a store or a branch in the body the compiler's wait counts
+// degrade to "wait for everything", which serialises the pipeline.
+template <int BITS, int CB, int MMAX, bool SILU, bool WRITE_HAD>
+__device__ __forceinline__ void gemv_accumulate(const GemvWalk& w, const int (&src)[MMAX],
+                                                uint32_t (&xs)[MMAX][64], float (&acc)[MMAX][2])
+{
+    const int lane = threadIdx.x & 63;
+    const int lane_dw = lane * BITS;
+    const int rows = w.rows;
+#pragma unroll
+    for (int m = 0; m < MMAX; ++m) acc[m][0] = acc[m][1] = 0.0f;
+
+    uint32_t own[8][BITS];
+    half2_t xr[MMAX], ur[MMAX], sc;
+    int kb = w.kb0;
+    if (kb >= w.KB) return;
+    {
+        // same issue order as inside the loop (activation first, then the tile rows),
+        // so that the wait counts the compiler derives at the loop head stay exact
+        sc = w.suh[kb * 64 + lane];
+#pragma unroll
+        for (int m = 0; m < MMAX; ++m) {
+            if (MMAX > 1 && m >= rows) break;
+            xr[m] = ((global_ptr<const half2_t>)(w.a + (size_t)src[m] * w.K + kb * 128))[lane];
+            if (SILU) ur[m] = ((global_ptr<const half2_t>)(w.a_up + (size_t)src[m] * w.K + kb * 128))[lane];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        const global_ptr<const uint32_t> base = w.tbase + (size_t)(kb * 8) * w.row_dw;
+#pragma unroll
+        for (int tr = 0; tr < 8; ++tr) {
+            load_tile_dwords<BITS>(base + tr * w.row_dw + lane_dw, own[tr]);
+            __builtin_amdgcn_sched_barrier(0);          // tile row 0 must be the oldest load in flight
+        }
+    }
+
+    for (; kb < w.KB; kb += w.step) {
+        const int nkb = kb + w.step;
+        const bool has_next = nkb < w.KB;
+        const int pkb = has_next ? nkb : kb;            // k-block whose activation is prefetched
+        // rotate this k-block of the activation: Hh(x * suh), rounded to fp16
+#pragma unroll
+        for (int m = 0; m < MMAX; ++m) {
+            if (MMAX > 1 && m >= rows) break;           // wave-uniform; rows past `rows` are never read
+            half2_t x = xr[m];
+            if (SILU) {
+                x.x = silu_mul_h(x.x, ur[m].x);
+                x.y = silu_mul_h(x.y, ur[m].y);
+            }
+            float v0 = (float)x.x * (float)sc.x;
+            float v1 = (float)x.y * (float)sc.y;
+            had128_wave(v0, v1, lane);
+            half2_t r;
+            r.x = (_Float16)(v0 * kRsqrt128);
+            r.y = (_Float16)(v1 * kRsqrt128);
+            xs[m][lane] = as_u32(r);
+            if (WRITE_HAD) ((global_ptr<half2_t>)(w.a_had + (size_t)m * w.K + kb * 128))[lane] = r;
+        }
+        sc = w.suh[pkb * 64 + lane];
+#pragma unroll
+        for (int m = 0; m < MMAX; ++m) {
+            if (MMAX > 1 && m >= rows) break;
+            xr[m] = ((global_ptr<const half2_t>)(w.a + (size_t)src[m] * w.K + pkb * 128))[lane];
+            if (SILU) ur[m] = ((global_ptr<const half2_t>)(w.a_up + (size_t)src[m] * w.K + pkb * 128))[lane];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_sched_barrier(0);
+
+        // No branch inside the tile-row loop (the compiler would sink the decode below
+        // it): a wave on its last k-block re-reads tile row 0 of its column block,
+        // always the same cached KiB, and ignores the result.
+        const global_ptr<const uint32_t> nbase = w.tbase + (has_next ? (size_t)(nkb * 8) * w.row_dw : (size_t)0);
+        const size_t nrow_dw = has_next ? w.row_dw : 0;
+#pragma unroll
+        for (int tr = 0; tr < 8; ++tr) {
+            uint32_t prev = fetch_prev(lane, own[tr][BITS - 1]);
+            uint32_t w2[16];
+            decode_lane<BITS, CB>(own[tr], prev, w2);
+            load_tile_dwords<BITS>(nbase + tr * nrow_dw + lane_dw, own[tr]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int m = 0; m < MMAX; ++m) {
+                if (MMAX > 1 && m >= rows) break;       // wave-uniform
+                const uint4* xp = (const uint4*)&xs[m][tr * 8];
+                uint4 xa = xp[0], xb = xp[1];
+                const uint32_t xk[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+#pragma unroll
+                for (int q = 0; q < 16; ++q)
+                    acc[m][pair_col_half(q)] = __builtin_amdgcn_fdot2(
+                        as_half2(w2[q]), as_half2(xk[pair_kk(q)]), acc[m][pair_col_half(q)], false);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+template <int BITS, int CB, int MMAX, bool SILU>
+__global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
 {
     __shared__ uint32_t xs[4][MMAX][64];    // wave-private: rotated k-block, one half2 per entry
     __shared__ float red[4][MMAX][128];
     __shared__ unsigned s_last;
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    // wave-uniform on purpose: everything derived from it (k-block, addresses) stays in SGPRs
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int per_problem = p.NB * p.S;
     const int prob = blockIdx.x / per_problem;
     const int local = blockIdx.x - prob * per_problem;
@@ -123,75 +251,57 @@ __global__ __launch_bounds__(256) void exl3_gemv_kernel(GemvParams p)
         row0 = gp.row0;
         rows = gp.nrows;
     }
+    int n_stride = p.N;             // columns of the full weight: tile-row stride and output row stride
+    int in_row0 = 0;                // first input row of this problem
+    int had_slab = 0;               // a_had slab of this problem
+    void* cout = p.c[which];
+    if (p.multi) {
+        lin.trellis = (const uint32_t*)p.b_list[prob];
+        lin.svh = (const _Float16*)p.svh_list[prob];
+        if (p.multi == 2) {
+            if (nb * 128 >= p.size_n_list[prob]) return;
+            n_stride = p.n_stride_list[prob];
+            had_slab = p.had_src_list[prob];
+            lin.suh = (const _Float16*)p.suh_list[had_slab];
+            cout = (void*)p.c_ptrs[prob];
+        } else {
+            lin.suh = (const _Float16*)p.suh_list[prob];
+            had_slab = prob;
+            in_row0 = prob * p.multi_in_rows;
+            cout = (char*)p.c[0] + (size_t)prob * p.rows * p.N * (p.out_fp32 ? 4 : 2);
+        }
+    }
     const int unit = (prob * (int)gridDim.y + which) * p.NB + nb;   // counter / partial slot
 
     const int wc = p.S * 4;
-    const int tn = p.N >> 4;
+    const int tn = n_stride >> 4;
     constexpr int tile_dw = 8 * BITS;
-    const int paddr = prev_lane_addr(lane);
     const size_t row_dw = (size_t)tn * tile_dw;   // dwords per tile row
 
     // source row of each of this problem's rows
     int src[MMAX];
 #pragma unroll
     for (int m = 0; m < MMAX; ++m) {
-        int r = row0 + (m < rows ? m : 0);
+        int r = row0 + in_row0 + (m < rows ? m : 0);
         src[m] = p.gather ? p.gather[r] / p.gather_div : r;
     }
 
     float acc[MMAX][2];
-#pragma unroll
-    for (int m = 0; m < MMAX; ++m) acc[m][0] = acc[m][1] = 0.0f;
-
-    for (int kb = s * 4 + wave; kb < p.KB; kb += wc) {
-        uint32_t own[8][BITS];
-        const uint32_t* base = lin.trellis + (size_t)(kb * 8) * row_dw + (size_t)(nb * 8) * tile_dw + lane * BITS;
-#pragma unroll
-        for (int tr = 0; tr < 8; ++tr) load_tile_dwords<BITS>(base + tr * row_dw, own[tr]);
-
-        // rotate this k-block of the activation: Hh(x * suh), rounded to fp16
-        const half2_t sc = ((const half2_t*)(lin.suh + kb * 128))[lane];
-#pragma unroll
-        for (int m = 0; m < MMAX; ++m) {
-            if (MMAX > 1 && m >= rows) break;               // wave-uniform; rows past `rows` are never read
-            half2_t x = ((const half2_t*)(p.a + (size_t)src[m] * p.K + kb * 128))[lane];
-            if (p.a_up) {
-                const half2_t u = ((const half2_t*)(p.a_up + (size_t)src[m] * p.K + kb * 128))[lane];
-                x.x = silu_mul_h(x.x, u.x);
-                x.y = silu_mul_h(x.y, u.y);
-            }
-            float v0 = (float)x.x * (float)sc.x;
-            float v1 = (float)x.y * (float)sc.y;
-            had128_wave(v0, v1, lane);
-            half2_t r;
-            r.x = (_Float16)(v0 * kRsqrt128);
-            r.y = (_Float16)(v1 * kRsqrt128);
-            xs[wave][m][lane] = as_u32(r);
-            if (p.a_had && nb == 0)
-                ((half2_t*)(p.a_had + (size_t)(row0 + m) * p.K + kb * 128))[lane] = r;
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-#pragma unroll
-        for (int tr = 0; tr < 8; ++tr) {
-            uint32_t prev = fetch_prev(paddr, own[tr][BITS - 1]);
-            uint32_t w2[16];
-            decode_lane<BITS, CB>(own[tr], prev, w2);
-#pragma unroll
-            for (int m = 0; m < MMAX; ++m) {
-                if (MMAX > 1 && m >= rows) break;           // wave-uniform
-                const uint4* xp = (const uint4*)&xs[wave][m][tr * 8];
-                uint4 xa = xp[0], xb = xp[1];
-                const uint32_t xk[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
-#pragma unroll
-                for (int q = 0; q < 16; ++q)
-                    acc[m][pair_col_half(q)] = __builtin_amdgcn_fdot2(
-                        as_half2(w2[q]), as_half2(xk[pair_kk(q)]), acc[m][pair_col_half(q)], false);
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
+    {
+        GemvWalk w;
+        w.tbase = as_global(lin.trellis) + (size_t)(nb * 8) * tile_dw;
+        w.suh = (global_ptr<const half2_t>)as_global(lin.suh);
+        w.a = as_global(p.a);
+        w.a_up = as_global(p.a_up);
+        w.a_had = as_global(p.a_had) + ((size_t)had_slab * rows + row0) * p.K;
+        w.row_dw = row_dw;
+        w.K = p.K;
+        w.KB = p.KB;
+        w.kb0 = s * 4 + wave;
+        w.step = wc;
+        w.rows = rows;
+        if (p.a_had && nb == 0) gemv_accumulate<BITS, CB, MMAX, SILU, true>(w, src, xs[wave], acc);
+        else gemv_accumulate<BITS, CB, MMAX, SILU, false>(w, src, xs[wave], acc);
     }
 
     // ---- reduce the 4 waves (k split inside the workgroup), wave order
@@ -222,7 +332,8 @@ __global__ __launch_bounds__(256) void exl3_gemv_kernel(GemvParams p)
         if (t < 128) {
 #pragma unroll
             for (int m = 0; m < MMAX; ++m)
-                __hip_atomic_store(mine + m * 128 + t, z[m], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (MMAX == 1 || m < rows)
+                    __hip_atomic_store(mine + m * 128 + t, z[m], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
@@ -237,19 +348,20 @@ __global__ __launch_bounds__(256) void exl3_gemv_kernel(GemvParams p)
             const float* all = p.partials + ((size_t)((size_t)unit * p.S) * MMAX) * 128;
 #pragma unroll
             for (int m = 0; m < MMAX; ++m) z[m] = 0.0f;
-            // loads in flight eight splits at a time; the adds stay in split order
-            for (int s0 = 0; s0 < p.S; s0 += 8) {
-                float part[8][MMAX];
+            // all loads of a batch in flight together; the adds stay in split order
+            constexpr int PB = MMAX == 1 ? 16 : 4;
+            for (int s0 = 0; s0 < p.S; s0 += PB) {
+                float part[PB][MMAX];
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
+                for (int j = 0; j < PB; ++j)
 #pragma unroll
                     for (int m = 0; m < MMAX; ++m)
-                        part[j][m] = (s0 + j < p.S)
+                        part[j][m] = (s0 + j < p.S && (MMAX == 1 || m < rows))
                             ? __hip_atomic_load(all + ((size_t)(s0 + j) * MMAX + m) * 128 + t, __ATOMIC_RELAXED,
                                                 __HIP_MEMORY_SCOPE_AGENT)
                             : 0.0f;
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
+                for (int j = 0; j < PB; ++j)
 #pragma unroll
                     for (int m = 0; m < MMAX; ++m)
                         if (s0 + j < p.S) z[m] += part[j][m];
@@ -265,15 +377,14 @@ __global__ __launch_bounds__(256) void exl3_gemv_kernel(GemvParams p)
         for (int m = 0; m < MMAX; ++m) red[0][m][t] = z[m];
     }
     __syncthreads();
-    const half2_t sv = ((const half2_t*)(lin.svh + nb * 128))[lane];
-    void* cout = p.c[which];
+    const half2_t sv = ((global_ptr<const half2_t>)as_global(lin.svh + nb * 128))[lane];
     for (int m = wave; m < rows; m += 4) {
         float v0 = red[0][m][2 * lane];
         float v1 = red[0][m][2 * lane + 1];
         had128_wave(v0, v1, lane);
         v0 = (v0 * kRsqrt128) * (float)sv.x;
         v1 = (v1 * kRsqrt128) * (float)sv.y;
-        size_t at = (size_t)(row0 + m) * p.N + nb * 128 + 2 * lane;
+        size_t at = (size_t)(row0 + m) * n_stride + nb * 128 + 2 * lane;
         if (p.out_fp32) {
             float2_t o = {v0, v1};
             *(float2_t*)((float*)cout + at) = o;

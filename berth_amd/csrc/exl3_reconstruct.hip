@@ -26,7 +26,7 @@ __global__ __launch_bounds__(256) void exl3_reconstruct_kernel(
     const uint32_t* src = trellis + ((size_t)kt * tiles_n_full + tile_n_offset + nb * 8) * tile_dw + lane * BITS;
 #pragma unroll
     for (int j = 0; j < BITS; ++j) own[j] = src[j];
-    uint32_t prev = fetch_prev(prev_lane_addr(lane), own[BITS - 1]);
+    uint32_t prev = fetch_prev(lane, own[BITS - 1]);
     uint32_t w2[16];
     decode_lane<BITS, CB>(own, prev, w2);
 

@@ -61,6 +61,24 @@ struct GroupedArgs {
 std::string launch_gemv_grouped(const GroupedArgs& args);
 std::string launch_gemm_grouped(const GroupedArgs& args);
 
+// multi-linear launch (crates/berth-kernels/src/ops.rs:247-367); every list is a device array
+struct MgemmArgs {
+    const void* a;
+    const void* b_list;
+    void* c;
+    const void* suh_list;
+    void* a_had;
+    const void* svh_list;
+    int size_m, size_k, size_n, k_bits, codebook, c_fp32, bszm_in, bszm_out;
+    const int* size_n_list;
+    const void* c_ptrs;
+    const int* n_stride_list;
+    const int* had_src_list;
+    int num_had_src;
+    hipStream_t stream;
+};
+std::string launch_mgemm(const MgemmArgs& args);
+
 // rows 1..8: VALU dot-product kernel.  Returns the launch description.
 std::string launch_gemv(const LinearArgs& args);
 // any row count: fp16 MFMA kernel (rows padded to 32 inside the kernel).

@@ -129,6 +129,64 @@ class Exl3Linear:
                                       self.codebook, out, gpu.raw_stream())
 
 
+class Exl3MultiLinear:
+    """Several EXL3 linears that share one input, launched as one sliced
+    `exl3_mgemm` (the qkv bundles of crates/berth-engine/src/attn.rs:1934-1973 and
+    gdn.rs:1102-1130; list layout from crates/berth-kernels/src/ops.rs:264-293):
+    every source is cut into slices of the greatest common width."""
+
+    def __init__(self, gpu: Gpu, sources: list[Exl3Linear]):
+        import math
+        k = {s.size_k for s in sources}
+        bits = {s.k_bits for s in sources}
+        cbs = {s.codebook for s in sources}
+        if len(k) != 1 or len(bits) != 1 or len(cbs) != 1:
+            raise InputError("multi-linear: sources must share in-features, bit rate and codebook")
+        self.sources = sources
+        self.size_k, self.k_bits, self.codebook = k.pop(), bits.pop(), cbs.pop()
+        width = 0
+        for s in sources:
+            width = math.gcd(width, s.size_n)
+        if width % 128:
+            raise InputError("multi-linear: slice width must be a multiple of 128")
+        self.width = width
+        b, svh, stride, src, n0s = [], [], [], [], []
+        tile_bytes = 16 * self.k_bits * 2
+        for si, s in enumerate(sources):
+            for n0 in range(0, s.size_n, width):
+                b.append(s.trellis.data_ptr() + (n0 // 16) * tile_bytes)
+                svh.append(s.svh.data_ptr() + n0 * 2)
+                stride.append(s.size_n)
+                src.append(si)
+                n0s.append(n0)
+        self.slices = len(b)
+        self._src, self._n0 = src, n0s
+        i64 = lambda v: torch.tensor(v, dtype=torch.int64, device=gpu.device)
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=gpu.device)
+        self.b_list, self.svh_list = i64(b), i64(svh)
+        self.suh_list = i64([s.suh.data_ptr() for s in sources])
+        self.size_n_list, self.n_stride_list, self.had_src_list = i32([width] * len(b)), i32(stride), i32(src)
+        self.a_had = torch.zeros(len(sources) * self.size_k, dtype=torch.float16, device=gpu.device)
+        self._c_key, self._c_ptrs = None, None
+
+    def forward(self, gpu: Gpu, a: torch.Tensor, outs: list[torch.Tensor], out: OutDtype, rows: int = 1) -> None:
+        """a fp16 [rows][K]; outs[i] [rows][N_i] of `out` for source i."""
+        if rows < 1 or rows > 8:
+            raise InputError("multi-linear: rows must be in 1..=8")
+        if rows * self.size_k > self.a_had.numel() // len(self.sources):
+            self.a_had = torch.zeros(len(self.sources) * rows * self.size_k, dtype=torch.float16, device=gpu.device)
+        esz = 4 if out == OutDtype.F32 else 2
+        key = tuple(o.data_ptr() for o in outs) + (esz,)
+        if key != self._c_key:
+            ptrs = [outs[s].data_ptr() + n0 * esz for s, n0 in zip(self._src, self._n0)]
+            self._c_ptrs = torch.tensor(ptrs, dtype=torch.int64, device=gpu.device)
+            self._c_key = key
+        K.ops.exl3_mgemm(ptr(a), ptr(self.b_list), ptr(outs[0]), ptr(self.suh_list), ptr(self.a_had),
+                         ptr(self.svh_list), rows, self.size_k, self.width, self.k_bits, self.codebook, out,
+                         1, self.slices, ptr(self.size_n_list), ptr(self._c_ptrs), ptr(self.n_stride_list),
+                         ptr(self.had_src_list), len(self.sources), gpu.raw_stream())
+
+
 class MlpLayer:
     """gate -> up -> silu_mul -> down (mlp.rs:118-150 decode, :219-303 prefill)."""
 

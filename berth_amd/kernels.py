@@ -50,6 +50,7 @@ def load() -> C.CDLL:
         L.berth_prefill_reconstruct.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, vp]
         L.berth_prefill_had_r_128.argtypes = [vp, vp, vp, ci, ci, ci, ci, vp]
         L.berth_ops_silu_mul.argtypes = [vp, vp, vp, C.c_int64, C.c_float, vp]
+        L.berth_ops_mgemm.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, vp, vp, vp, vp, ci, vp]
         for name in ("berth_exl3_last_error", "berth_exl3_last_launch", "berth_prefill_last_error",
                      "berth_prefill_last_launch", "berth_ops_last_error", "berth_ops_last_launch"):
             getattr(L, name).restype = C.c_char_p
@@ -143,6 +144,18 @@ class prefill_lin:
 
 class ops:
     """crates/berth-kernels/src/ops.rs (the EXL3-path subset)."""
+
+    @staticmethod
+    def exl3_mgemm(a, b_list, c, suh_list, a_had, svh_list, size_m, size_k, size_n, k_bits,
+                   codebook: Codebook, out: OutDtype, bszm_in, bszm_out, size_n_list=None, c_ptrs=None,
+                   n_stride_list=None, had_src_list=None, num_had_src=0, stream=None) -> int:
+        """crates/berth-kernels/src/ops.rs:317-367; returns the positive tag."""
+        rc = load().berth_ops_mgemm(a, b_list, c, suh_list, a_had, svh_list, size_m, size_k, size_n, k_bits,
+                                    int(codebook), int(out), bszm_in, bszm_out, size_n_list, c_ptrs,
+                                    n_stride_list, had_src_list, num_had_src, stream)
+        if rc > 0:
+            return rc
+        raise LaunchError(ops.last_error() or f"exl3_mgemm launch failed ({rc})")
 
     @staticmethod
     def silu_mul(gate, up, out, numel: int, act_limit: float = 0.0, stream=None) -> None:

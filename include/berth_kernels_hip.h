@@ -81,6 +81,23 @@ int berth_prefill_had_r_128(const void* input, void* output, const void* scale, 
  * alias up. */
 int berth_ops_silu_mul(const void* gate, const void* up, void* out, int64_t numel,
                        float act_limit, void* stream);
+/* replaces crates/berth-kernels/src/ops.rs:17-38,247-367 / csrc/ops/mgemm.cu:296-340:
+ * several EXL3 linears in one launch.  Every list is a DEVICE array.  Sliced
+ * mode (all four slice lists given, bszm_in == 1): bszm_out slices sharing the
+ * input a [size_m][size_k]; b_list[s] = trellis of the source advanced to the
+ * slice's first tile column; suh_list[src] per source (num_had_src of them);
+ * svh_list[s] = svh + n0; c_ptrs[s] = output + n0 with row stride
+ * n_stride_list[s] (the source's full N, also the trellis row stride);
+ * size_n_list[s] <= size_n = slice width; had_src_list[s] = source index;
+ * a_had holds num_had_src slabs of size_m*size_k.  Uniform mode (lists NULL):
+ * bszm_out linears of one shape, inputs a[i] (bszm_in == bszm_out) or a[0]
+ * (bszm_in == 1), outputs c[i] contiguous.  size_m <= 8.  Returns 1 on success
+ * (the reference returns its kernel-shape tag there), -1 on error. */
+int berth_ops_mgemm(const void* a, const void* b_list, void* c, const void* suh_list, void* a_had,
+                    const void* svh_list, int size_m, int size_k, int size_n, int k_bits,
+                    int codebook, int c_fp32, int bszm_in, int bszm_out, const int* size_n_list,
+                    const void* c_ptrs, const int* n_stride_list, const int* had_src_list,
+                    int num_had_src, void* stream);
 const char* berth_ops_last_error(void);    /* ops.rs:145 */
 const char* berth_ops_last_launch(void);   /* ops.rs:146 */
 

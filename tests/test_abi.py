@@ -95,3 +95,14 @@ def test_silu_mul_validation():
     with pytest.raises(LaunchError, match="positive and even"):
         K.ops.silu_mul(P, P, P, 0)
     assert K.ops.last_launch() == ""
+
+
+def test_mgemm_validation():
+    with pytest.raises(LaunchError, match="null"):
+        K.ops.exl3_mgemm(None, P, P, P, P, P, 1, 128, 128, 4, Codebook.MUL1, OutDtype.F16, 1, 2)
+    with pytest.raises(LaunchError, match="sliced mode requires"):
+        K.ops.exl3_mgemm(P, P, P, P, P, P, 1, 128, 128, 4, Codebook.MUL1, OutDtype.F16, 1, 2, size_n_list=P)
+    with pytest.raises(LaunchError, match="single-input"):
+        K.ops.exl3_mgemm(P, P, P, P, P, P, 1, 128, 128, 4, Codebook.MUL1, OutDtype.F16, 2, 2, P, P, P, P, 1)
+    with pytest.raises(LaunchError, match="num_had_src requires"):
+        K.ops.exl3_mgemm(P, P, P, P, P, P, 1, 128, 128, 4, Codebook.MUL1, OutDtype.F16, 1, 2, num_had_src=1)

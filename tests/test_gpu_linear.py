@@ -261,3 +261,48 @@ def test_full_size_gemv_round_trip_property():
     sub = tr[:, 16:32, :]                       # columns 256..511
     want, _ = O.linear(x1, sub, suh, svh[256:512], Kk, 256, 4, 2, out_fp32=True)
     assert close(y1[256:512], want.reshape(-1))[0] == 0
+
+
+# ---- multi-linear (exl3_mgemm)
+@pytest.mark.parametrize("rows,fp32", [(1, False), (1, True), (3, False)])
+def test_mgemm_sliced_qkv_bundle(rows, fp32):
+    from berth_amd.device import Exl3Linear, Exl3MultiLinear, Gpu
+    gpu = Gpu(0)
+    Kk, Ns = 512, (768, 256, 256)
+    lins_np = [synth.linear(700 + i, Kk, n, 4) for i, n in enumerate(Ns)]
+    lins = [Exl3Linear(gpu, f"l{i}", *l) for i, l in enumerate(lins_np)]
+    multi = Exl3MultiLinear(gpu, lins)
+    assert multi.width == 256 and multi.slices == 5
+    x = synth.activations(710, rows, Kk)
+    d_x = dev(x.view(np.uint16))
+    outs = [torch.zeros((rows, n), dtype=torch.float32 if fp32 else torch.float16, device=DEV) for n in Ns]
+    multi.forward(gpu, d_x, outs, OutDtype.F32 if fp32 else OutDtype.F16, rows)
+    torch.cuda.synchronize()
+    assert "sliced x5" in K.ops.last_launch()
+    for i, (tr, suh, svh) in enumerate(lins_np):
+        want, want_had = O.linear(x, tr, suh, svh, Kk, Ns[i], 4, 2, out_fp32=fp32)
+        got = outs[i].cpu().numpy() if fp32 else host_f16(outs[i])
+        assert close(got, want)[0] == 0, i
+        slab = host_u16(multi.a_had)[i * rows * Kk:(i + 1) * rows * Kk]
+        assert np.array_equal(slab, want_had.view(np.uint16).reshape(-1))
+
+
+def test_mgemm_uniform_mode():
+    Kk, N, n_mat = 256, 256, 3
+    lins = [synth.linear(800 + i, Kk, N, 4) for i in range(n_mat)]
+    x = synth.activations(810, n_mat, Kk)            # one row per matrix
+    d = [[dev(t.view(np.uint16)) for t in lin] for lin in lins]
+    i64 = lambda v: torch.tensor(v, dtype=torch.int64, device=DEV)
+    b_list, suh_list, svh_list = (i64([dd[j].data_ptr() for dd in d]) for j in range(3))
+    d_x = dev(x.view(np.uint16))
+    for bszm_in in (n_mat, 1):
+        c = torch.zeros((n_mat, 1, N), dtype=torch.float32, device=DEV)
+        a_had = torch.zeros((n_mat, Kk), dtype=torch.float16, device=DEV)
+        rc = K.ops.exl3_mgemm(d_x.data_ptr(), b_list.data_ptr(), c.data_ptr(), suh_list.data_ptr(), a_had.data_ptr(),
+                              svh_list.data_ptr(), 1, Kk, N, 4, Codebook.MUL1, OutDtype.F32, bszm_in, n_mat)
+        torch.cuda.synchronize()
+        assert rc > 0
+        for i, (tr, suh, svh) in enumerate(lins):
+            xi = x[i:i + 1] if bszm_in > 1 else x[0:1]
+            want, _ = O.linear(xi, tr, suh, svh, Kk, N, 4, 2, out_fp32=True)
+            assert close(c[i].cpu().numpy(), want)[0] == 0
