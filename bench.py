@@ -114,6 +114,41 @@ def moe_bench(gpu, steps: int, warmup: int):
     return res
 
 
+def prefill_bench(gpu, layers, bits: int, rows: int, steps: int):
+    """BASELINE.json configs[2]: the same 27B-shaped linears at `rows` = 512 tokens,
+    fp16 activations N(0,1), fp16/fp32 outputs with fp32 accumulation, through
+    berth_prefill_exl3_linear (Hadamard pre-pass + decode-in-GEMM MFMA kernel)."""
+    import torch
+
+    from berth_amd import synth
+    from berth_amd.device import RowScratch
+    from berth_amd.kernels import OutDtype
+
+    scratch = RowScratch(gpu, rows, 17408, 17408)
+    xin = {K: gpu.upload(synth.activations(9, rows, K).view(np.uint16)) for K in (5120, 6144, 17408)}
+    outs = {n: torch.zeros((rows, synth.SHAPES_27B[n][1]), dtype=torch.float32 if OUT_FP32[n] else torch.float16,
+                           device=gpu.device) for n in ORDER}
+    flops = sum(2.0 * rows * K * N for K, N in (synth.SHAPES_27B[n] for n in ORDER))
+
+    def step(i):
+        lin = layers[i % len(layers)]
+        for n in ORDER:
+            l = lin[n]
+            l.forward_rows(gpu, scratch, xin[l.size_k], outs[n], rows, OutDtype.F32 if OUT_FP32[n] else OutDtype.F16)
+
+    for i in range(3):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    return {"rows": rows, "ms_per_layer_set": round(dt * 1e3, 3), "tflops": round(flops / dt / 1e12, 1),
+            "mfma_peak_tflops": 2500.0, "frac_of_fp16_mfma_peak": round(flops / dt / 2.5e15, 4),
+            "tokens_per_s": round(rows / dt, 0)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -124,6 +159,7 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-moe", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--unfused", action="store_true", help="seven separate launches instead of four")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 1 GiB device copy kernel a few times (reference reading for "
@@ -230,6 +266,8 @@ def main():
                      "avg_launch_us": round(avg_launch_us, 3),
                      "bytes_per_launch": step_bytes // launches_per_step},
     }
+    if not args.no_prefill:
+        line["prefill_gemm"] = prefill_bench(gpu, layers, bits, 512, 10)
     if not args.no_moe:
         del layers
         torch.cuda.empty_cache()

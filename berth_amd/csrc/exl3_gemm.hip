@@ -50,11 +50,11 @@ struct GemmParams {
 constexpr int kAStride = 128 + 8;   // halves per LDS row of the A tile (272 B: conflict-free b128 reads)
 
 template <int BITS, int CB, int MB>  // MB = 32-row blocks per workgroup
-__global__ __launch_bounds__(256) void exl3_gemm_kernel(GemmParams p)
+__global__ __launch_bounds__(256, 2) void exl3_gemm_kernel(GemmParams p)
 {
     constexpr int BM = MB * 32;
     extern __shared__ __align__(16) unsigned char smem[];
-    _Float16* a_tile = (_Float16*)smem;                 // [BM][kAStride]
+    _Float16* a_tile = (_Float16*)smem;                 // [2][BM][kAStride]
     float* z_tile = (float*)smem;                       // epilogue: [32][256 + 4]
     constexpr int kZStride = 256 + 4;
     __shared__ unsigned s_last;
@@ -99,42 +99,59 @@ __global__ __launch_bounds__(256) void exl3_gemm_kernel(GemmParams p)
     const uint32_t* tbase = lin.trellis + (size_t)half_id * row_dw +
                             (size_t)((nw >> 4) + (slot >> 3)) * tile_dw + (slot & 7) * BITS;
 
+    // Both operands run one k-block ahead in registers: the trellis dwords of the
+    // wave's four steps (nxt) and this thread's share of the A tile (a_nxt, 32 bytes
+    // per 256-thread pass).  The A tile is double-buffered in LDS, so a k-block costs
+    // one barrier.
+    constexpr int kAPasses = BM * 8 / 256;
     uint32_t nxt[4][BITS];
-    if (active && split < KB) {
-        const uint32_t* nb = tbase + (size_t)(split * 8) * row_dw;
+    uint4 a_nxt[kAPasses][2];
+    const int a_row = threadIdx.x >> 3, a_ch = threadIdx.x & 7;       // + 32 rows per pass
+    auto load_a = [&](int kb) {
+#pragma unroll
+        for (int ps = 0; ps < kAPasses; ++ps) {
+            const int r = a_row + 32 * ps;
+            uint4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
+            if (m0 + r < m_end) {
+                const uint4* src = (const uint4*)(a_had + (size_t)(m0 + r) * p.K + kb * 128 + a_ch * 16);
+                v0 = src[0];
+                v1 = src[1];
+            }
+            a_nxt[ps][0] = v0;
+            a_nxt[ps][1] = v1;
+        }
+    };
+    auto load_b = [&](int kb) {
+        const uint32_t* nb = tbase + (size_t)(kb * 8) * row_dw;
 #pragma unroll
         for (int st = 0; st < 4; ++st)
 #pragma unroll
             for (int j = 0; j < BITS; ++j) nxt[st][j] = nb[(size_t)(2 * st) * row_dw + j];
+    };
+    if (split < KB) {
+        load_a(split);
+        if (active) load_b(split);
     }
 
-    for (int kb = split; kb < KB; kb += p.S) {
+    int buf = 0;
+    for (int kb = split; kb < KB; kb += p.S, buf ^= 1) {
         uint32_t cur[4][BITS];
 #pragma unroll
         for (int st = 0; st < 4; ++st)
 #pragma unroll
             for (int j = 0; j < BITS; ++j) cur[st][j] = nxt[st][j];
 
-        __syncthreads();        // previous k-block's readers are done with a_tile
-        // stage a_had[m0 .. m0+BM)[kb*128 .. +128) : 16 halves (32 B) per thread per pass
-        for (int idx = threadIdx.x; idx < BM * 8; idx += 256) {
-            const int r = idx >> 3, ch = idx & 7;
-            uint4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
-            if (m0 + r < m_end) {
-                const uint4* src = (const uint4*)(a_had + (size_t)(m0 + r) * p.K + kb * 128 + ch * 16);
-                v0 = src[0];
-                v1 = src[1];
-            }
-            uint4* dst = (uint4*)(a_tile + r * kAStride + ch * 16);
-            dst[0] = v0;
-            dst[1] = v1;
+        // publish this k-block's A tile; the other buffer may still be read by slower waves
+        _Float16* a_buf = a_tile + (size_t)buf * BM * kAStride;
+#pragma unroll
+        for (int ps = 0; ps < kAPasses; ++ps) {
+            uint4* dst = (uint4*)(a_buf + (a_row + 32 * ps) * kAStride + a_ch * 16);
+            dst[0] = a_nxt[ps][0];
+            dst[1] = a_nxt[ps][1];
         }
-        if (active && kb + p.S < KB) {
-            const uint32_t* nb = tbase + (size_t)((kb + p.S) * 8) * row_dw;
-#pragma unroll
-            for (int st = 0; st < 4; ++st)
-#pragma unroll
-                for (int j = 0; j < BITS; ++j) nxt[st][j] = nb[(size_t)(2 * st) * row_dw + j];
+        if (kb + p.S < KB) {
+            load_a(kb + p.S);
+            if (active) load_b(kb + p.S);
         }
         __syncthreads();
 
@@ -156,7 +173,7 @@ __global__ __launch_bounds__(256) void exl3_gemm_kernel(GemmParams p)
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {
                     if (MB > 1 && mb * 32 >= rows_here) break;          // workgroup-uniform
-                    const _Float16* arow = a_tile + (mb * 32 + slot) * kAStride + 32 * st + 16 * half_id;
+                    const _Float16* arow = a_buf + (mb * 32 + slot) * kAStride + 32 * st + 16 * half_id;
                     const half8_t a0 = *(const half8_t*)(arow);
                     const half8_t a1 = *(const half8_t*)(arow + 8);
                     acc[mb][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b[0][0], acc[mb][0], 0, 0, 0);
@@ -274,9 +291,14 @@ template <int BITS, int CB, int MB>
 static void gemm_launch_mb(const GemmParams& p, hipStream_t stream, std::string& desc, dim3 grid)
 {
     constexpr int BM = MB * 32;
-    const size_t smem_a = (size_t)BM * kAStride * sizeof(_Float16);
+    const size_t smem_a = (size_t)2 * BM * kAStride * sizeof(_Float16);     // double-buffered A tile
     const size_t smem_z = (size_t)32 * (256 + 4) * sizeof(float);
     const size_t smem = smem_a > smem_z ? smem_a : smem_z;
+    if (smem > 64 * 1024) {
+        static const hipError_t attr = hipFuncSetAttribute((const void*)exl3_gemm_kernel<BITS, CB, MB>,
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        hip_ok(attr, "exl3_gemm_kernel shared-memory attribute");
+    }
     hipLaunchKernelGGL((exl3_gemm_kernel<BITS, CB, MB>), grid, dim3(256), smem, stream, p);
     desc = "exl3_gemm_kernel<" + std::to_string(BITS) + "," + std::to_string(CB) + "," + std::to_string(BM) +
            "x256> grid=" + std::to_string(grid.x) + "x" + std::to_string(grid.y) + "x" + std::to_string(grid.z) +
