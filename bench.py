@@ -114,6 +114,125 @@ def moe_bench(gpu, steps: int, warmup: int):
     return res
 
 
+def moe_large_bench(gpu, steps: int, resident_layers: int = 48):
+    """BASELINE.json configs[4]: hidden 2048, 512 experts top-10 plus one always-on
+    shared expert, intermediate 512, 3 bpw, 256 tokens, router logits biased so
+    that expert popularity is Zipf(1.1); the weights of 48 such layers (29 GB)
+    stay resident in HBM and the steps rotate over them.  Weights are generated
+    on the device (uniform random trellis words, sign x lognormal(0, 0.1) scales)."""
+    import torch
+
+    from berth_amd import synth
+    from berth_amd.device import Exl3Linear
+    from berth_amd.moe import MoeLayer
+
+    T, H, E, k, I, bits = 256, 2048, 512, 10, 512, 3
+    g = torch.Generator(device=gpu.device)
+    g.manual_seed(4242)
+    words = (H // 16) * (I // 16) * 16 * bits          # u16 words of one expert linear
+    a_had = torch.zeros(H, dtype=torch.float16, device=gpu.device)
+
+    def scales(n):
+        sign = torch.randint(0, 2, (n,), generator=g, device=gpu.device).float() * 2 - 1
+        return (sign * torch.exp(0.1 * torch.randn(n, generator=g, device=gpu.device))).half()
+
+    layers = []
+    for li in range(resident_layers):
+        slab = torch.randint(0, 65536, ((E + 1) * 3, words), generator=g, device=gpu.device,
+                             dtype=torch.int32).to(torch.int16)
+        su = scales((E + 1) * 3 * H).view((E + 1) * 3, H)      # rows of H; the I-sized vectors use a prefix
+        sv = scales((E + 1) * 3 * H).view((E + 1) * 3, H)
+        experts = []
+        for e in range(E + 1):
+            trio = []
+            for j, (kk, nn) in enumerate(((H, I), (H, I), (I, H))):
+                r = 3 * e + j
+                trio.append(Exl3Linear.from_device(f"layers.{li}.experts.{e}.{j}", slab[r], su[r, :kk], sv[r, :nn],
+                                                   bits, a_had=a_had))
+            experts.append(tuple(trio))
+        layers.append(MoeLayer(gpu, synth.router_weight(900 + li, H, E), experts[:E], k, shared=experts[E],
+                               bias=synth.zipf_bias(950 + li, E)))
+    resident = sum(l.trellis_bytes() for l in layers)
+    xs = [gpu.upload(synth.activations(700 + i, T, H).view(np.uint16)) for i in range(8)]
+    out = torch.zeros((T, H), dtype=torch.float32, device=gpu.device)
+    idx = torch.zeros((T, k), dtype=torch.int32, device=gpu.device)
+    hit, hottest = 0.0, 0
+    for i in range(8):
+        layers[i % len(layers)].forward(gpu, xs[i], out, T, idx)
+        c = np.bincount(idx.cpu().numpy().ravel(), minlength=E)
+        hit += float((c > 0).sum()) / 8
+        hottest = max(hottest, int(c.max()))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        layers[i % len(layers)].forward(gpu, xs[i % 8], out, T)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    expert_bytes = 3 * H * I * bits // 8 + 2 * (2 * (H + I) + (I + H))
+    nbytes = 2 * H * E + (hit + 1) * expert_bytes + 2 * T * H + 4 * T * H
+    flops = 2.0 * (T * k + T) * 3 * H * I
+    return {"config": "hidden 2048, 512 experts top-10 + shared expert, intermediate 512, 3 bpw, 256 tokens, "
+                      "Zipf(1.1) router bias, mul1",
+            "resident_layers": len(layers), "resident_weight_GB": round(resident / 1e9, 2),
+            "us_per_layer": round(dt * 1e6, 1), "us_per_token": round(dt / T * 1e6, 3),
+            "experts_hit": round(hit, 1), "hottest_expert_rows": hottest,
+            "algorithmic_GBps": round(nbytes / dt / 1e9, 1), "tflops": round(flops / dt / 1e12, 2)}
+
+
+def bpw_sweep(gpu, rates, steps: int, nlayers: int = 8):
+    """BASELINE.json configs[1] at the other bit rates of its sweep: the same four
+    launches per step over device-generated weights, GB/s of algorithmic bytes."""
+    import torch
+
+    from berth_amd import synth
+    from berth_amd.device import Exl3Linear, Exl3MultiLinear
+    from berth_amd.kernels import OutDtype
+
+    g = torch.Generator(device=gpu.device)
+    g.manual_seed(99)
+    xin = {K: gpu.upload(synth.activations(5, 1, K).view(np.uint16)) for K in (5120, 6144, 17408)}
+    outs = {n: torch.zeros(synth.SHAPES_27B[n][1], dtype=torch.float32 if OUT_FP32[n] else torch.float16,
+                           device=gpu.device) for n in ORDER}
+    res = {}
+    for bits in rates:
+        layers = []
+        for li in range(nlayers):
+            lin = {}
+            for name in ORDER:
+                K, N = synth.SHAPES_27B[name]
+                tr = torch.randint(0, 65536, (K * N * bits // 16,), generator=g, device=gpu.device,
+                                   dtype=torch.int32).to(torch.int16)
+                sc = [((torch.randint(0, 2, (n,), generator=g, device=gpu.device).float() * 2 - 1)
+                       * torch.exp(0.1 * torch.randn(n, generator=g, device=gpu.device))).half() for n in (K, N)]
+                lin[name] = Exl3Linear.from_device(f"layers.{li}.{name}", tr, sc[0], sc[1], bits)
+            lin["qkv"] = Exl3MultiLinear(gpu, [lin["q_proj"], lin["k_proj"], lin["v_proj"]])
+            lin["gate_up"] = Exl3MultiLinear(gpu, [lin["gate_proj"], lin["up_proj"]])
+            layers.append(lin)
+
+        def step(i):
+            lin = layers[i % nlayers]
+            lin["qkv"].forward(gpu, xin[5120], [outs["q_proj"], outs["k_proj"], outs["v_proj"]], OutDtype.F16)
+            lin["o_proj"].forward(gpu, xin[6144], outs["o_proj"], OutDtype.F32)
+            lin["gate_up"].forward(gpu, xin[5120], [outs["gate_proj"], outs["up_proj"]], OutDtype.F16)
+            lin["down_proj"].forward(gpu, xin[17408], outs["down_proj"], OutDtype.F32)
+
+        for i in range(10):
+            step(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            step(i)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        nbytes = sum(linear_bytes(*synth.SHAPES_27B[n], bits, 1, 4 if OUT_FP32[n] else 2) for n in ORDER)
+        res[f"{bits}bpw"] = {"GBps": round(nbytes / dt / 1e9, 1), "us_per_step": round(dt * 1e6, 2),
+                             "frac_of_hbm_peak": round(nbytes / dt / 1e9 / HBM_PEAK_GBS, 4),
+                             "Gweights_per_s": round(340787200 / dt / 1e9, 1)}
+        del layers
+        torch.cuda.empty_cache()
+    return res
+
+
 def prefill_bench(gpu, layers, bits: int, rows: int, steps: int):
     """BASELINE.json configs[2]: the same 27B-shaped linears at `rows` = 512 tokens,
     fp16 activations N(0,1), fp16/fp32 outputs with fp32 accumulation, through
@@ -160,6 +279,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-moe", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--moe-resident-layers", type=int, default=48)
     ap.add_argument("--unfused", action="store_true", help="seven separate launches instead of four")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 1 GiB device copy kernel a few times (reference reading for "
@@ -268,10 +389,17 @@ def main():
     }
     if not args.no_prefill:
         line["prefill_gemm"] = prefill_bench(gpu, layers, bits, 512, 10)
+    if not args.no_sweep:
+        line["bpw_sweep"] = bpw_sweep(gpu, [b for b in (2, 3, 4, 5) if b != bits], max(20, args.steps // 2))
+        line["bpw_sweep"][f"{bits}bpw"] = {"GBps": line["value"], "us_per_step": round(ms_per_step * 1e3, 2),
+                                          "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+                                          "Gweights_per_s": round(340787200 / ms_per_step / 1e6, 1)}
     if not args.no_moe:
         del layers
         torch.cuda.empty_cache()
         line["moe_layer"] = moe_bench(gpu, max(20, args.steps // 2), max(5, args.warmup // 2))
+        torch.cuda.empty_cache()
+        line["moe_large_layer"] = moe_large_bench(gpu, 96, args.moe_resident_layers)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(bits, args.cpu_seconds)
     print(json.dumps(line))

@@ -220,6 +220,26 @@ extern "C" int berth_prefill_had_r_128(const void* input, void* output, const vo
 extern "C" const char* berth_prefill_last_error(void) { return g_prefill_err.c_str(); }
 extern "C" const char* berth_prefill_last_launch(void) { return g_prefill_launch.c_str(); }
 
+extern "C" int berth_exl3_unpack_signs(const void* packed, void* out, int64_t packed_bytes, void* stream)
+{
+    try {
+        g_exl3_err.clear();
+        g_exl3_launch.clear();
+        if (packed_bytes < 0 || (packed_bytes & 1))
+            throw std::runtime_error("su: packed sign bytes " + std::to_string(packed_bytes) +
+                                     " are not a multiple of 2");
+        if (packed_bytes == 0) return 0;
+        if (!packed || !out) throw std::runtime_error("su: null device pointer");
+        g_exl3_launch = launch_unpack_signs(packed, out, packed_bytes / 2, (hipStream_t)stream);
+        return 0;
+    } catch (const std::exception& err) {
+        g_exl3_err = err.what();
+        g_exl3_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
 extern "C" int berth_ops_silu_mul(const void* gate, const void* up, void* out, int64_t numel,
                                   float act_limit, void* stream)
 {

@@ -93,4 +93,27 @@ std::string launch_silu_mul(const void* gate, const void* up, void* out, int64_t
     return "silu_mul_kernel block=256 grid=" + std::to_string(blocks);
 }
 
+// crates/berth-exl3/src/signs.rs:25-46: packed su / sv -> fp16 signs.  Little-endian
+// u16 words, bit i of a word is element i of its 16; a set bit is -1.0 (0xBC00),
+// a clear bit +1.0 (0x3C00).  One thread per output pair.
+__global__ __launch_bounds__(256) void unpack_signs_kernel(const uint16_t* __restrict__ packed,
+                                                           uint32_t* __restrict__ out, int64_t pairs)
+{
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= pairs) return;
+    const uint32_t word = packed[i >> 3];
+    const uint32_t two = (word >> (2 * (i & 7))) & 3u;
+    out[i] = 0x3C003C00u | ((two & 1u) << 15) | ((two & 2u) << 30);
+}
+
+std::string launch_unpack_signs(const void* packed, void* out, int64_t words, hipStream_t stream)
+{
+    const int64_t pairs = words * 8;
+    const unsigned blocks = (unsigned)((pairs + 255) / 256);
+    hipLaunchKernelGGL(unpack_signs_kernel, dim3(blocks), dim3(256), 0, stream, (const uint16_t*)packed,
+                       (uint32_t*)out, pairs);
+    hip_ok(hipGetLastError(), "unpack_signs launch");
+    return "unpack_signs_kernel block=256 grid=" + std::to_string(blocks);
+}
+
 }  // namespace berth

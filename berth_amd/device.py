@@ -83,6 +83,40 @@ class Exl3Linear:
         self.svh = gpu.upload(svh.view(np.uint16))
         self.a_had = torch.zeros(self.size_k, dtype=torch.float16, device=gpu.device)
 
+    @classmethod
+    def from_device(cls, prefix: str, trellis: torch.Tensor, suh: torch.Tensor, svh: torch.Tensor, k_bits: int,
+                    codebook: Codebook = Codebook.MUL1, a_had: torch.Tensor | None = None) -> "Exl3Linear":
+        """Adopt tensors that already live on the device (16-bit element types:
+        trellis (K/16)(N/16)(16 k_bits) words, suh [K], svh [N]); a_had may be shared
+        between linears that never run concurrently."""
+        self = cls.__new__(cls)
+        self.prefix, self.k_bits, self.codebook = prefix, int(k_bits), codebook
+        self.size_k, self.size_n = int(suh.numel()), int(svh.numel())
+        if self.size_k % 128 or self.size_n % 128 or \
+           trellis.numel() != (self.size_k // 16) * (self.size_n // 16) * 16 * self.k_bits or \
+           trellis.element_size() != 2 or suh.element_size() != 2 or svh.element_size() != 2:
+            raise InputError(f"{prefix}: trellis shape does not match suh / svh")
+        self.trellis, self.suh, self.svh = trellis, suh, svh
+        self.a_had = a_had if a_had is not None else torch.zeros(self.size_k, dtype=torch.float16, device=trellis.device)
+        return self
+
+    @classmethod
+    def from_packed_signs(cls, gpu: Gpu, prefix: str, trellis: np.ndarray, su: np.ndarray, sv: np.ndarray,
+                          codebook: Codebook = Codebook.MUL1) -> "Exl3Linear":
+        """A linear stored with packed sign tensors `su` [K/16] / `sv` [N/16] (int16
+        words, one bit per channel: crates/berth-exl3/src/linear.rs:122-141): the
+        words are uploaded and expanded to fp16 +-1 on the device."""
+        halves = []
+        for name, words in (("su", su), ("sv", sv)):
+            raw = np.ascontiguousarray(words).view(np.uint8).ravel()
+            d_raw = torch.from_numpy(raw.copy()).to(gpu.device)
+            out = torch.zeros(raw.size * 8, dtype=torch.float16, device=gpu.device)
+            K.unpack_signs(ptr(d_raw), ptr(out), raw.size, gpu.raw_stream())
+            halves.append(out)
+        gpu.synchronize()
+        return cls.from_device(prefix, gpu.upload(trellis.view(np.uint16)).reshape(-1), halves[0], halves[1],
+                               trellis.shape[2] // 16, codebook)
+
     def trellis_bytes(self) -> int:
         return self.trellis.numel() * 2
 

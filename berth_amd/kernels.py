@@ -50,6 +50,8 @@ def load() -> C.CDLL:
         L.berth_prefill_reconstruct.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, vp]
         L.berth_prefill_had_r_128.argtypes = [vp, vp, vp, ci, ci, ci, ci, vp]
         L.berth_ops_silu_mul.argtypes = [vp, vp, vp, C.c_int64, C.c_float, vp]
+        L.berth_exl3_unpack_signs.argtypes = [vp, vp, C.c_int64, vp]
+        L.berth_exl3_unpack_signs.restype = C.c_int
         L.berth_ops_mgemm.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, vp, vp, vp, vp, ci, vp]
         for name in ("berth_exl3_last_error", "berth_exl3_last_launch", "berth_prefill_last_error",
                      "berth_prefill_last_launch", "berth_ops_last_error", "berth_ops_last_launch"):
@@ -83,6 +85,14 @@ def exl3_linear(a, trellis, c, suh, a_had, svh, size_m, size_k, size_n, k_bits,
                              int(codebook), int(out), stream)
     if rc != 0:
         raise LaunchError(last_error() or f"exl3 linear launch failed ({rc})")
+
+
+def unpack_signs(packed, out, packed_bytes: int, stream=None) -> None:
+    """crates/berth-exl3/src/signs.rs:25-46 on device memory: packed su / sv words
+    -> fp16 signs (16 per u16 word)."""
+    rc = load().berth_exl3_unpack_signs(packed, out, packed_bytes, stream)
+    if rc != 0:
+        raise LaunchError(last_error() or f"unpack_signs launch failed ({rc})")
 
 
 def last_launch() -> str:

@@ -75,6 +75,14 @@ int berth_prefill_reconstruct(void* unpacked, const void* packed, int size_k, in
 int berth_prefill_had_r_128(const void* input, void* output, const void* scale, int pre_scale,
                             int rows, int cols, int fp32, void* stream);
 
+/* ---- packed signs --------------------------------------------------------------
+ * replaces crates/berth-exl3/src/signs.rs:25-46 for tensors that are already on
+ * the device: packed su / sv (little-endian u16 words, bit i of a word = element
+ * i, set = -1.0) -> fp16 signs, 16 per word.  packed_bytes must be even (the
+ * reference's error text otherwise); errors and launch text go to
+ * berth_exl3_last_error / berth_exl3_last_launch. */
+int berth_exl3_unpack_signs(const void* packed, void* out, int64_t packed_bytes, void* stream);
+
 /* ---- ops -------------------------------------------------------------------
  * replaces crates/berth-kernels/src/ops.rs:82-90 / csrc/ops/act.cu:35-69:
  * out = silu(gate) * up, fp16, numel even, act_limit 0 = no clamp; out may

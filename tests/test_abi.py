@@ -97,6 +97,15 @@ def test_silu_mul_validation():
     assert K.ops.last_launch() == ""
 
 
+def test_unpack_signs_validation():
+    # crates/berth-exl3/src/signs.rs:26-34: odd byte counts are rejected before anything runs
+    with pytest.raises(LaunchError, match="su.*not a multiple of 2"):
+        K.unpack_signs(P, P, 3)
+    with pytest.raises(LaunchError, match="null"):
+        K.unpack_signs(None, P, 4)
+    K.unpack_signs(None, None, 0)       # empty input: nothing to do
+
+
 def test_mgemm_validation():
     with pytest.raises(LaunchError, match="null"):
         K.ops.exl3_mgemm(None, P, P, P, P, P, 1, 128, 128, 4, Codebook.MUL1, OutDtype.F16, 1, 2)

@@ -11,6 +11,7 @@ import torch
 
 from berth_amd import kernels as K
 from berth_amd import synth
+from berth_amd.device import Exl3Linear, Gpu
 from berth_amd.kernels import Codebook, OutDtype
 from oracle import oracle as O
 from tests.gpu_util import DEV, close, dev, host_f16, host_u16
@@ -306,3 +307,47 @@ def test_mgemm_uniform_mode():
             xi = x[i:i + 1] if bszm_in > 1 else x[0:1]
             want, _ = O.linear(xi, tr, suh, svh, Kk, N, 4, 2, out_fp32=True)
             assert close(c[i].cpu().numpy(), want)[0] == 0
+
+
+def test_unpack_signs_known_answers():
+    """The five known-answer cases of crates/berth-exl3/src/signs.rs:48-92 and a
+    random tensor against the oracle, on the device."""
+    ONE, NEG = 0x3C00, 0xBC00
+
+    def run(words):
+        raw = np.asarray(words, dtype="<u2").view(np.uint8)
+        d_in = torch.from_numpy(raw.copy()).to(DEV)
+        d_out = torch.zeros(raw.size * 8, dtype=torch.int16, device=DEV)
+        K.unpack_signs(d_in.data_ptr(), d_out.data_ptr(), raw.size)
+        torch.cuda.synchronize()
+        return d_out.cpu().numpy().view(np.uint16)
+
+    s = run([1])
+    assert len(s) == 16 and s[0] == NEG and (s[1:] == ONE).all()
+    s = run([0x8000])
+    assert (s[:15] == ONE).all() and s[15] == NEG
+    assert (run([0]) == ONE).all() and (run([0xFFFF]) == NEG).all()
+    s = run([5, 1])
+    assert len(s) == 32 and (s[0], s[1], s[2], s[16], s[17]) == (NEG, ONE, NEG, NEG, ONE)
+    words = np.random.default_rng(8).integers(0, 65536, size=1088, dtype=np.uint16)
+    assert np.array_equal(run(words), np.asarray(O.unpack_signs(words.astype("<u2").tobytes()), dtype=np.uint16))
+
+
+def test_linear_from_packed_signs():
+    """A linear whose su / sv are packed sign words gives the same output as the
+    one built from the expanded fp16 signs."""
+    gpu = Gpu(0)
+    Kk, N, bits = 256, 384, 4
+    tr = synth.trellis_words(70, Kk, N, bits)
+    rng = np.random.default_rng(71)
+    su = rng.integers(0, 65536, size=Kk // 16, dtype=np.uint16)
+    sv = rng.integers(0, 65536, size=N // 16, dtype=np.uint16)
+    suh = np.asarray(O.unpack_signs(su.astype("<u2").tobytes()), dtype=np.uint16).view(np.float16)
+    svh = np.asarray(O.unpack_signs(sv.astype("<u2").tobytes()), dtype=np.uint16).view(np.float16)
+    x = synth.activations(72, 1, Kk)
+    lin = Exl3Linear.from_packed_signs(gpu, "packed", tr, su, sv)
+    c = torch.zeros(N, dtype=torch.float32, device=DEV)
+    lin.forward(gpu, dev(x.view(np.uint16)), c, OutDtype.F32)
+    torch.cuda.synchronize()
+    want, _ = O.linear(x, tr, suh, svh, Kk, N, bits, 2, out_fp32=True)
+    assert close(c.cpu().numpy(), want.ravel())[0] == 0

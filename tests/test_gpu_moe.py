@@ -198,6 +198,31 @@ def test_moe_config3_shape_decode_token():
     assert np.abs(out.cpu().numpy() - want).max() <= 2e-3 * np.abs(want).max()
 
 
+def test_moe_config4_shape_zipf_shared():
+    """hidden 2048, 512 experts top-10 plus an always-on shared expert, intermediate
+    512, 3 bpw, 256 tokens, Zipf(1.1)-biased router: skewed problem list (hot
+    experts with several 32-row chunks, many cold experts with a row or none)."""
+    gpu = Gpu(0)
+    T, H, E, k, I, bits = 256, 2048, 512, 10, 512, 3
+    # router scaled by sqrt(H) to compensate the 1/sqrt(H) token scale: same logits as N(0,1) tokens
+    wr, experts_np, experts, shared_np, shared = _make_layer(gpu, 7000, H, E, I, bits, I, float(np.sqrt(H)))
+    bias = synth.zipf_bias(41, E)
+    layer = MoeLayer(gpu, wr, experts, k, shared=shared, bias=bias)
+    x = (synth.activations(43, T, H).astype(np.float32) / np.sqrt(H)).astype(np.float16)
+    out = torch.zeros((T, H), dtype=torch.float32, device=DEV)
+    idx = torch.zeros((T, k), dtype=torch.int32, device=DEV)
+    w = torch.zeros((T, k), dtype=torch.float32, device=DEV)
+    layer.forward(gpu, dev(x.view(np.uint16)), out, T, idx, w)
+    torch.cuda.synchronize()
+    want, oi, ow = O.moe_layer(x, wr, experts_np, k, I, bits, 2, bias=bias, shared=shared_np, shared_I=I)
+    assert np.array_equal(idx.cpu().numpy(), oi)
+    counts = np.bincount(oi.ravel(), minlength=E)
+    assert counts.max() > 64 and (counts == 0).sum() > 0, "routing is not skewed"
+    assert np.allclose(w.cpu().numpy(), ow, rtol=1e-5, atol=1e-7)
+    _check_stages(layer, x, experts_np, shared_np, oi, w.cpu().numpy(), out.cpu().numpy(), T, H, E, k, I, bits, I)
+    assert np.abs(out.cpu().numpy() - want).max() <= 2e-3 * np.abs(want).max()
+
+
 def test_moe_validation_errors():
     with pytest.raises(K.LaunchError, match="null"):
         K.moe.layer(None, None, None, None, None, None, None, None, None, 0, 1, 128, 8, 2, 128, 0, 4, K.Codebook.MUL1)
