@@ -219,15 +219,24 @@ def bpw_sweep(gpu, rates, steps: int, nlayers: int = 8):
         for i in range(10):
             step(i)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(steps):
-            step(i)
-        torch.cuda.synchronize()
-        dt = (time.perf_counter() - t0) / steps
+        dt, wall = None, None
+        for _ in range(2):                                  # best of two passes
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0 = time.perf_counter()
+            e0.record()
+            for i in range(steps):
+                step(i)
+            e1.record()
+            torch.cuda.synchronize()
+            w = (time.perf_counter() - t0) / steps
+            d = e0.elapsed_time(e1) * 1e-3 / steps          # device time between the two events
+            if dt is None or d < dt:
+                dt, wall = d, w
         nbytes = sum(linear_bytes(*synth.SHAPES_27B[n], bits, 1, 4 if OUT_FP32[n] else 2) for n in ORDER)
         res[f"{bits}bpw"] = {"GBps": round(nbytes / dt / 1e9, 1), "us_per_step": round(dt * 1e6, 2),
                              "frac_of_hbm_peak": round(nbytes / dt / 1e9 / HBM_PEAK_GBS, 4),
-                             "Gweights_per_s": round(340787200 / dt / 1e9, 1)}
+                             "Gweights_per_s": round(340787200 / dt / 1e9, 1),
+                             "host_us_per_step": round(wall * 1e6, 2)}
         del layers
         torch.cuda.empty_cache()
     return res
@@ -387,13 +396,13 @@ def main():
                      "avg_launch_us": round(avg_launch_us, 3),
                      "bytes_per_launch": step_bytes // launches_per_step},
     }
-    if not args.no_prefill:
-        line["prefill_gemm"] = prefill_bench(gpu, layers, bits, 512, 10)
     if not args.no_sweep:
         line["bpw_sweep"] = bpw_sweep(gpu, [b for b in (2, 3, 4, 5) if b != bits], max(20, args.steps // 2))
         line["bpw_sweep"][f"{bits}bpw"] = {"GBps": line["value"], "us_per_step": round(ms_per_step * 1e3, 2),
                                           "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
                                           "Gweights_per_s": round(340787200 / ms_per_step / 1e6, 1)}
+    if not args.no_prefill:
+        line["prefill_gemm"] = prefill_bench(gpu, layers, bits, 512, 10)
     if not args.no_moe:
         del layers
         torch.cuda.empty_cache()

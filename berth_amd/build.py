@@ -21,7 +21,8 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
 
 LIBRARIES = {
     "libberth_kernels_hip.so": ["api.hip", "exl3_gemv.hip", "exl3_gemv_cb0.hip", "exl3_gemv_cb1.hip",
-                                "exl3_gemv_cb2.hip", "exl3_gemm.hip",
+                                "exl3_gemv_cb2.hip", "exl3_gemm.hip", "exl3_gemm_cb0.hip", "exl3_gemm_cb1.hip",
+                                "exl3_gemm_cb2.hip",
                                 "exl3_reconstruct.hip", "elementwise.hip", "moe.hip"],
     "libberth_hip.so": ["berth_hip.hip"],
 }

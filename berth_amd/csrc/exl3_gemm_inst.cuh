@@ -1,0 +1,53 @@
+// Per-codebook instantiations of the MFMA GEMM kernel (included by
+// exl3_gemm_cb{0,1,2}.hip with BERTH_GEMM_CB defined): 32-row and 128-row tiles for
+// every bit rate.
+#include "exl3_gemm_kernel.cuh"
+#include "launch.h"
+
+namespace berth {
+
+template <int BITS, int CB, int MB>
+static void gemm_launch_mb(const GemmParams& p, hipStream_t stream, std::string& desc, dim3 grid)
+{
+    constexpr int BM = MB * 32;
+    const size_t smem_a = (size_t)2 * BM * kAStride * sizeof(_Float16);     // double-buffered A tile
+    const size_t smem_z = (size_t)32 * (256 + 4) * sizeof(float);
+    const size_t smem = smem_a > smem_z ? smem_a : smem_z;
+    if (smem > 64 * 1024) {
+        static const hipError_t attr = hipFuncSetAttribute((const void*)exl3_gemm_kernel<BITS, CB, MB>,
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        hip_ok(attr, "exl3_gemm_kernel shared-memory attribute");
+    }
+    hipLaunchKernelGGL((exl3_gemm_kernel<BITS, CB, MB>), grid, dim3(256), smem, stream, p);
+    desc = "exl3_gemm_kernel<" + std::to_string(BITS) + "," + std::to_string(CB) + "," + std::to_string(BM) +
+           "x256> grid=" + std::to_string(grid.x) + "x" + std::to_string(grid.y) + "x" + std::to_string(grid.z) +
+           " split_k=" + std::to_string(p.S) + " smem=" + std::to_string(smem);
+}
+
+template <int BITS, int CB>
+static void gemm_launch(const GemmParams& p, int mb, hipStream_t stream, std::string& desc, dim3 grid)
+{
+    if (mb == 1) gemm_launch_mb<BITS, CB, 1>(p, stream, desc, grid);
+    else gemm_launch_mb<BITS, CB, 4>(p, stream, desc, grid);
+}
+
+#define BERTH_CAT2(a, b) a##b
+#define BERTH_CAT(a, b) BERTH_CAT2(a, b)
+
+void BERTH_CAT(launch_gemm_cb, BERTH_GEMM_CB)(const GemmParams& p, int bits, int mb, hipStream_t stream,
+                                              std::string& desc, dim3 grid)
+{
+    constexpr int CB = BERTH_GEMM_CB;
+    switch (bits) {
+    case 1: gemm_launch<1, CB>(p, mb, stream, desc, grid); break;
+    case 2: gemm_launch<2, CB>(p, mb, stream, desc, grid); break;
+    case 3: gemm_launch<3, CB>(p, mb, stream, desc, grid); break;
+    case 4: gemm_launch<4, CB>(p, mb, stream, desc, grid); break;
+    case 5: gemm_launch<5, CB>(p, mb, stream, desc, grid); break;
+    case 6: gemm_launch<6, CB>(p, mb, stream, desc, grid); break;
+    case 7: gemm_launch<7, CB>(p, mb, stream, desc, grid); break;
+    default: gemm_launch<8, CB>(p, mb, stream, desc, grid); break;
+    }
+}
+
+}  // namespace berth

@@ -19,6 +19,7 @@
 #include "launch.h"
 
 #include <cstdlib>
+#include <cstring>
 
 namespace berth {
 
@@ -147,6 +148,8 @@ std::string launch_gemv_grouped(const GroupedArgs& g)
     p.num_problems = g.num_problems;
     p.lins_per_expert = g.lins_per_expert;
     p.lin_base = g.lin_base;
+    p.shared_expert = g.shared ? g.shared_expert : -1;
+    if (g.shared) std::memcpy(p.shared, g.shared, sizeof(p.shared));
     p.c[0] = g.c0;
     p.c[1] = g.c1;
     p.partials = ws.partials;
@@ -158,11 +161,13 @@ std::string launch_gemv_grouped(const GroupedArgs& g)
     p.out_fp32 = g.out_fp32;
     const long units = (long)g.max_problems * g.num_lins * p.NB;
     if (units > kCounters) throw std::runtime_error("moe grouped linear: too many (problem, column block) units");
-    p.S = pick_split(ws, units, p.KB, 8);
+    const int mmax = g.single_row ? 1 : 8;
+    p.S = pick_split(ws, units, p.KB, mmax);
     dim3 grid((unsigned)(g.max_problems * p.NB * p.S), (unsigned)g.num_lins);
-    launch_bits(p, g.k_bits, g.codebook, 8, grid, g.stream);
+    launch_bits(p, g.k_bits, g.codebook, mmax, grid, g.stream);
     hip_ok(hipGetLastError(), "exl3_gemv_kernel grouped launch");
-    return "exl3_gemv_kernel<" + std::to_string(g.k_bits) + "," + std::to_string(g.codebook) + ",8> grouped grid=" +
+    return "exl3_gemv_kernel<" + std::to_string(g.k_bits) + "," + std::to_string(g.codebook) + "," +
+           std::to_string(mmax) + "> grouped grid=" +
            std::to_string(grid.x) + "x" + std::to_string(grid.y) + " split_k=" + std::to_string(p.S);
 }
 

@@ -1,7 +1,7 @@
 // Per-codebook instantiations of the GEMV kernel (included by exl3_gemv_cb{0,1,2}.hip
 // with BERTH_GEMV_CB defined).  Instantiated row capacities: 1 (decode) and 8 (small
-// batches, grouped problems); the SiLU-gated input only exists for the grouped down
-// projection.
+// batches, grouped problems); the SiLU-gated input exists for the grouped down
+// projection (one row per problem, or up to 8).
 #include "exl3_gemv_kernel.cuh"
 #include "launch.h"
 
@@ -10,7 +10,8 @@ namespace berth {
 template <int BITS, int CB>
 static void launch_rows(const GemvParams& p, int mmax, dim3 grid, hipStream_t stream)
 {
-    if (p.a_up) hipLaunchKernelGGL((exl3_gemv_kernel<BITS, CB, 8, true>), grid, dim3(256), 0, stream, p);
+    if (p.a_up && mmax == 1) hipLaunchKernelGGL((exl3_gemv_kernel<BITS, CB, 1, true>), grid, dim3(256), 0, stream, p);
+    else if (p.a_up) hipLaunchKernelGGL((exl3_gemv_kernel<BITS, CB, 8, true>), grid, dim3(256), 0, stream, p);
     else if (mmax == 1) hipLaunchKernelGGL((exl3_gemv_kernel<BITS, CB, 1, false>), grid, dim3(256), 0, stream, p);
     else hipLaunchKernelGGL((exl3_gemv_kernel<BITS, CB, 8, false>), grid, dim3(256), 0, stream, p);
 }

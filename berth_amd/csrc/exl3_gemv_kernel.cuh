@@ -57,6 +57,8 @@ struct GemvParams {
     const int* num_problems;
     int lins_per_expert;
     int lin_base;
+    ExpertLin shared[3];        // an always-on expert passed by value (problem.expert == shared_expert)
+    int shared_expert;
     // multi-linear mode (multi != 0), the argument lists of
     // crates/berth-kernels/src/ops.rs:264-293, all device arrays: one problem per
     // entry of b_list; multi == 2 is the sliced form (per-slice width, row stride
@@ -247,7 +249,8 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
     if (p.problems) {
         if (prob >= *p.num_problems) return;
         const GroupProblem gp = p.problems[prob];
-        lin = p.experts[gp.expert * p.lins_per_expert + p.lin_base + which];
+        lin = gp.expert == p.shared_expert ? p.shared[p.lin_base + which]
+                                           : p.experts[gp.expert * p.lins_per_expert + p.lin_base + which];
         row0 = gp.row0;
         rows = gp.nrows;
     }

@@ -63,6 +63,23 @@ __device__ __forceinline__ float had_stage_swap32(float v, float sgn)
     return __builtin_fmaf(hi, sgn, lo);
 }
 
+// value of lane (lane ^ 16) / (lane ^ 32): after the swap one of the two registers
+// holds the partner's value in every lane (the lower rows find it in hi, the upper
+// rows in lo)
+__device__ __forceinline__ float lane_xor_swap16(float v)
+{
+    float lo = v, hi = v;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+    return (__lane_id() & 16) ? lo : hi;
+}
+
+__device__ __forceinline__ float lane_xor_swap32(float v)
+{
+    float lo = v, hi = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+    return (__lane_id() & 32) ? lo : hi;
+}
+
 // lane l holds elements 2l (v0) and 2l+1 (v1) of a 128 vector
 __device__ __forceinline__ void had128_wave(float& v0, float& v1, int lane)
 {
@@ -83,6 +100,37 @@ __device__ __forceinline__ void had128_wave(float& v0, float& v1, int lane)
     // the result is lo + hi in the lower lane and lo - hi in the upper lane
     v0 = had_stage_swap16(v0, s16);  v1 = had_stage_swap16(v1, s16);
     v0 = had_stage_swap32(v0, s32);  v1 = had_stage_swap32(v1, s32);
+}
+
+// 128-point Hadamard with eight consecutive elements per lane and sixteen lanes
+// (one DPP row) per vector, so a wave rotates four vectors at once: stages 1, 2, 4
+// stay inside the lane, stages 8 .. 64 are DPP exchanges inside the row.  Same
+// butterfly order and the same exact sums as had128_wave.
+__device__ __forceinline__ void had128_row16(float (&v)[8], int lane)
+{
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if ((i & h) == 0) {
+                const float a = v[i], b = v[i + h];
+                v[i] = a + b;
+                v[i + h] = a - b;
+            }
+        }
+    }
+    const float s1 = (lane & 1) ? -1.0f : 1.0f;
+    const float s2 = (lane & 2) ? -1.0f : 1.0f;
+    const float s4 = (lane & 4) ? -1.0f : 1.0f;
+    const float s8 = (lane & 8) ? -1.0f : 1.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = had_stage_dpp<1>(v[i], s1);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = had_stage_dpp<2>(v[i], s2);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = had_stage_dpp<4>(v[i], s4);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = had_stage_dpp<8>(v[i], s8);
 }
 
 }  // namespace berth

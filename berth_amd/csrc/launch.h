@@ -47,6 +47,10 @@ struct GroupedArgs {
     const int32_t* gather;      // optional: source row = gather[r] / gather_div
     int gather_div;
     const void* experts;        // ExpertLin[num_experts * lins_per_expert]
+    const void* shared;         // host: three {trellis, suh, svh} of the always-on expert, or null
+    int shared_expert;          // expert index the problem list uses for it (-1: none)
+    int single_row;             // every problem has exactly one row
+    int mb;                     // MFMA path: rows per problem / 32 (1 or 4)
     const void* problems;       // GroupProblem[max_problems]
     const int* num_problems;
     int max_problems;

@@ -17,15 +17,17 @@
 
 #include "../../include/berth_kernels_hip.h"
 
+#include <cstdlib>
+
 namespace berth {
 
 constexpr int kRouteSeg = 64;       // rows of the router weight per partial sum
 constexpr int kRouteTT = 4;         // tokens per route workgroup
 constexpr int kMaxExperts = 1024;
 constexpr int kMaxTopK = 32;
-constexpr int kValuPairs = 8;       // calls with at most this many (token, slot) pairs use the VALU kernel only
-constexpr int kGemmRows = 32;       // rows per MFMA problem
-constexpr int kMaxPairsLds = 8192;  // pairs staged in LDS by the permute kernel
+constexpr int kValuPairs = 8;       // calls with one token or at most this many rows use the VALU kernel only
+constexpr int kGemmRows = 32;       // rows per small MFMA problem
+constexpr int kGemmBigRows = 128;   // rows per big MFMA problem
 
 // ------------------------------------------------------------------ route
 
@@ -40,6 +42,59 @@ struct RouteParams {
     float* logits;          // [T][E] or null
     int T, H, E, k, nseg, renorm;
 };
+
+// Top-k of one token by one wave: lane holds the logits of experts lane + 64 i.
+// Largest first, ties to the lowest expert index; weights exp(l - max) normalised
+// over the selected k (renorm) or over all experts.
+constexpr int kRoutePer = kMaxExperts / 64;
+
+__device__ __forceinline__ void route_topk(const float (&lg)[kRoutePer], int lane, const RouteParams& p, int t)
+{
+    constexpr int PER = kRoutePer;
+    unsigned taken = 0;
+    float sel_logit = 0.0f;         // lane j keeps the logit of slot j
+    int sel_idx = 0;
+    for (int j = 0; j < p.k; ++j) {
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int e = lane + 64 * i;
+            if (e < p.E && !((taken >> i) & 1u) && (bi == 0x7fffffff || lg[i] > bv)) { bv = lg[i]; bi = e; }
+        }
+        auto merge = [&](float ov, int oi) {
+            const bool take = (oi != 0x7fffffff) && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi));
+            if (take) { bv = ov; bi = oi; }
+        };
+        merge(lane_xor_dpp<1>(bv), __builtin_bit_cast(int, lane_xor_dpp<1>(__builtin_bit_cast(float, bi))));
+        merge(lane_xor_dpp<2>(bv), __builtin_bit_cast(int, lane_xor_dpp<2>(__builtin_bit_cast(float, bi))));
+        merge(lane_xor_dpp<4>(bv), __builtin_bit_cast(int, lane_xor_dpp<4>(__builtin_bit_cast(float, bi))));
+        merge(lane_xor_dpp<8>(bv), __builtin_bit_cast(int, lane_xor_dpp<8>(__builtin_bit_cast(float, bi))));
+        merge(lane_xor_swap16(bv), __builtin_bit_cast(int, lane_xor_swap16(__builtin_bit_cast(float, bi))));
+        merge(lane_xor_swap32(bv), __builtin_bit_cast(int, lane_xor_swap32(__builtin_bit_cast(float, bi))));
+        if ((bi & 63) == lane) taken |= 1u << (bi >> 6);
+        if (lane == j) { sel_logit = bv; sel_idx = bi; }
+    }
+    const float mx = __shfl(sel_logit, 0, 64);
+    float ev = (lane < p.k) ? expf(sel_logit - mx) : 0.0f;
+    float denom = 0.0f;
+    if (p.renorm) {
+        for (int j = 0; j < p.k; ++j) denom += __shfl(ev, j, 64);       // slot order
+    } else {
+        float loc = 0.0f;
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+            if (lane + 64 * i < p.E) loc += expf(lg[i] - mx);
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) loc += __shfl_xor(loc, d, 64);
+        denom = loc;
+    }
+    if (lane < p.k) {
+        p.idx[(size_t)t * p.k + lane] = sel_idx;
+        p.w[(size_t)t * p.k + lane] = ev / denom;
+    }
+}
+
 
 __global__ __launch_bounds__(256) void moe_route_kernel(RouteParams p)
 {
@@ -89,7 +144,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(RouteParams p)
     const int lane = tid & 63, tt = tid >> 6;
     const int t = t0 + tt;
     if (t >= p.T) return;
-    constexpr int PER = kMaxExperts / 64;
+    constexpr int PER = kRoutePer;
     float lg[PER];
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
@@ -115,138 +170,273 @@ __global__ __launch_bounds__(256) void moe_route_kernel(RouteParams p)
         }
         lg[i] = v;
     }
-    unsigned taken = 0;
-    float sel_logit = 0.0f;         // lane j keeps the logit of slot j
-    int sel_idx = 0;
-    for (int j = 0; j < p.k; ++j) {
-        float bv = -INFINITY;
-        int bi = 0x7fffffff;
+    route_topk(lg, lane, p, t);
+}
+
+// Many tokens: the same arithmetic in two launches, so that the segment sums of a
+// token are added by a workgroup of its own instead of the last workgroup of a
+// token group.  First launch: partial sums of kRouteBigTT tokens x one 64-row
+// segment; second launch: one workgroup per token adds the segments in order,
+// adds the bias and selects.
+constexpr int kRouteBigTT = 16;
+constexpr int kRouteBigT = 32;      // calls with at least this many tokens take the two-launch path
+
+// partial sums of kRouteBigTT tokens x two neighbouring experts over one segment.
+// EVEN: the expert count is even, so the pair is one aligned 4-byte load per row.
+// Eight rows of the router weight are loaded back to back (no branch in between:
+// the loads are what the loop waits for); the fma chains stay in row order.
+template <bool EVEN>
+__device__ __forceinline__ void route_pair_segment(const RouteParams& p, const float (*xs)[kRouteBigTT], int e0,
+                                                   int h0, int hn, float (&part)[2][kRouteBigTT])
+{
+    const bool two = e0 + 1 < p.E;
+    const _Float16* wcol = p.wr + (size_t)h0 * p.E + e0;
+    const int second = two ? 1 : 0;                     // odd counts: the last expert has no neighbour
+    // the weights of the next eight rows are loaded before the fma chains of the
+    // current eight start (rows past the segment re-read its last row)
+    auto load8 = [&](int hb, half2_t (&wv)[8], float (&s0)[8], float (&s1)[8]) {
 #pragma unroll
-        for (int i = 0; i < PER; ++i) {
-            const int e = lane + 64 * i;
-            if (e < p.E && !((taken >> i) & 1u) && (bi == 0x7fffffff || lg[i] > bv)) { bv = lg[i]; bi = e; }
+        for (int i = 0; i < 8; ++i) {
+            const int h = hb + i < hn ? hb + i : hn - 1;
+            if (EVEN) {
+                wv[i] = *(const half2_t*)(wcol + (size_t)h * p.E);
+            } else {
+                s0[i] = (float)wcol[(size_t)h * p.E];
+                s1[i] = (float)wcol[(size_t)h * p.E + second];
+            }
         }
+    };
+    half2_t wn[8];
+    float sn0[8], sn1[8];
+    load8(0, wn, sn0, sn1);
+    for (int hb = 0; hb < hn; hb += 8) {
+        float w0[8], w1[8];
 #pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const float ov = __shfl_xor(bv, d, 64);
-            const int oi = __shfl_xor(bi, d, 64);
-            const bool take = (oi != 0x7fffffff) && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi));
-            if (take) { bv = ov; bi = oi; }
+        for (int i = 0; i < 8; ++i) {
+            w0[i] = EVEN ? (float)wn[i].x : sn0[i];
+            w1[i] = EVEN ? (float)wn[i].y : sn1[i];
         }
-        if ((bi & 63) == lane) taken |= 1u << (bi >> 6);
-        if (lane == j) { sel_logit = bv; sel_idx = bi; }
-    }
-    const float mx = __shfl(sel_logit, 0, 64);
-    float ev = (lane < p.k) ? expf(sel_logit - mx) : 0.0f;
-    float denom = 0.0f;
-    if (p.renorm) {
-        for (int j = 0; j < p.k; ++j) denom += __shfl(ev, j, 64);       // slot order
-    } else {
-        float loc = 0.0f;
+        load8(hb + 8 < hn ? hb + 8 : hb, wn, sn0, sn1);
 #pragma unroll
-        for (int i = 0; i < PER; ++i)
-            if (lane + 64 * i < p.E) loc += expf(lg[i] - mx);
+        for (int i = 0; i < 8; ++i) {
+            // rows past the segment hold zeros in xs: they add +-0 to the partial sum, and
+            // the sign of a zero partial sum never reaches a logit (0 + partial comes first)
+            const float4_t* xrow = (const float4_t*)&xs[hb + i][0];
 #pragma unroll
-        for (int d = 32; d >= 1; d >>= 1) loc += __shfl_xor(loc, d, 64);
-        denom = loc;
+            for (int q = 0; q < kRouteBigTT / 4; ++q) {
+                const float4_t xv = xrow[q];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    part[0][4 * q + j] = __builtin_fmaf(xv[j], w0[i], part[0][4 * q + j]);
+                    part[1][4 * q + j] = __builtin_fmaf(xv[j], w1[i], part[1][4 * q + j]);
+                }
+            }
+        }
     }
-    if (lane < p.k) {
-        p.idx[(size_t)t * p.k + lane] = sel_idx;
-        p.w[(size_t)t * p.k + lane] = ev / denom;
+}
+
+__global__ __launch_bounds__(256) void moe_route_partial_kernel(RouteParams p)
+{
+    __shared__ __align__(16) float xs[kRouteSeg][kRouteBigTT];      // [row][token]: one b128 read per 4 tokens
+    const int seg = blockIdx.x, grp = blockIdx.y;
+    const int t0 = grp * kRouteBigTT;
+    const int h0 = seg * kRouteSeg;
+    const int hn = min(kRouteSeg, p.H - h0);
+    const int tid = threadIdx.x;
+    for (int i = tid; i < kRouteBigTT * kRouteSeg; i += 256) {
+        const int tt = i / kRouteSeg, h = i % kRouteSeg;
+        float v = 0.0f;
+        if (t0 + tt < p.T && h < hn) v = (float)p.x[(size_t)(t0 + tt) * p.H + h0 + h];
+        xs[h][tt] = v;
     }
+    __syncthreads();
+    const bool even = (p.E & 1) == 0;
+    for (int e0 = 2 * tid; e0 < p.E; e0 += 512) {
+        float part[2][kRouteBigTT];
+#pragma unroll
+        for (int tt = 0; tt < kRouteBigTT; ++tt) part[0][tt] = part[1][tt] = 0.0f;
+        if (even) route_pair_segment<true>(p, xs, e0, h0, hn, part);
+        else route_pair_segment<false>(p, xs, e0, h0, hn, part);
+        const bool two = e0 + 1 < p.E;
+#pragma unroll
+        for (int tt = 0; tt < kRouteBigTT; ++tt) {
+            if (t0 + tt < p.T) {
+                float* dst = p.parts + ((size_t)(t0 + tt) * p.nseg + seg) * p.E + e0;
+                dst[0] = part[0][tt];
+                if (two) dst[1] = part[1][tt];
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void moe_route_finish_kernel(RouteParams p)
+{
+    __shared__ float s_logit[kMaxExperts];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    // two experts per pass, 32 segment loads of each in flight together (indices past
+    // the end re-read the last segment / the last expert and are ignored)
+    for (int e = tid; e < p.E; e += 512) {
+        const int e2 = e + 256 < p.E ? e + 256 : e;
+        const float* src0 = p.parts + (size_t)t * p.nseg * p.E + e;
+        const float* src1 = p.parts + (size_t)t * p.nseg * p.E + e2;
+        float v0 = 0.0f, v1 = 0.0f;
+        for (int s0 = 0; s0 < p.nseg; s0 += 32) {
+            float part0[32], part1[32];
+#pragma unroll
+            for (int j = 0; j < 32; ++j) {
+                const size_t at = (size_t)min(s0 + j, p.nseg - 1) * p.E;
+                part0[j] = src0[at];
+                part1[j] = src1[at];
+            }
+#pragma unroll
+            for (int j = 0; j < 32; ++j) {
+                const float n0 = v0 + part0[j], n1 = v1 + part1[j];
+                v0 = s0 + j < p.nseg ? n0 : v0;
+                v1 = s0 + j < p.nseg ? n1 : v1;
+            }
+        }
+        if (p.bias) { v0 += p.bias[e]; v1 += p.bias[e2]; }
+        if (p.logits) {
+            p.logits[(size_t)t * p.E + e] = v0;
+            if (e2 != e) p.logits[(size_t)t * p.E + e2] = v1;
+        }
+        s_logit[e] = v0;
+        if (e2 != e) s_logit[e2] = v1;
+    }
+    __syncthreads();
+    if (tid >= 64) return;
+    float lg[kRoutePer];
+#pragma unroll
+    for (int i = 0; i < kRoutePer; ++i) {
+        const int e = tid + 64 * i;
+        lg[i] = e < p.E ? s_logit[e] : -INFINITY;
+    }
+    route_topk(lg, tid, p, t);
 }
 
 // ---------------------------------------------------------------- permute
 
 struct PermuteParams {
-    const int32_t* idx;     // [P] expert of each (token, slot) pair, P = T * k
+    const int32_t* idx;     // [P] expert of each (token, slot) pair, P = T * k; distinct within a token
     int32_t* offsets;       // [E + 1]
-    int32_t* perm;          // [P] sorted position -> pair
+    int32_t* perm;          // [R] sorted position -> pair (pair / k = token)
     int32_t* inv;           // [P] pair -> sorted position
-    int32_t* row_expert;    // [P] sorted position -> expert
-    int32_t* counts;        // [2] number of VALU problems, number of MFMA problems
+    int32_t* row_expert;    // [R] sorted position -> expert
+    int32_t* counts;        // [3] number of VALU problems, small MFMA problems, big MFMA problems
     GroupProblem* vprob;
-    GroupProblem* mprob;
-    int P, E;
-    int use_valu;           // 1: every expert is one VALU problem (P <= 8); 0: MFMA problems of <= 32 rows
+    GroupProblem* mprob;    // <= 32 rows each
+    GroupProblem* bprob;    // <= 128 rows each
+    int T, k, E;
+    int use_valu;           // 1: every expert is one VALU problem (<= 8 rows each); 0: MFMA problems: an
+                            // expert's rows go to big problems of 128 and the rest to small ones of <= 32
+    int shared_rows;        // 1: rows P .. P + T - 1 belong to an always-on expert with index E (token order)
+    int big_min;            // a remainder of at least this many rows becomes a (partial) big problem
 };
 
-// One workgroup.  The pairs are cut into `parts` contiguous segments; thread
-// (part, e) counts and later places the pairs of expert e inside its segment, in
-// order: a stable counting sort whose result does not depend on scheduling.
+// One workgroup.  Counting sort by expert, stable in pair order: the pairs of one
+// expert come from distinct tokens, so the rank of pair (t, slot) inside its expert
+// is the number of earlier tokens that chose the expert.  Tokens are taken 64 at a
+// time: a 64-bit mask per expert records which of them chose it, and the rank is a
+// population count below the token's bit.  Nothing depends on scheduling.
 __global__ __launch_bounds__(1024) void moe_permute_kernel(PermuteParams p)
 {
-    __shared__ int cnt[1024];                   // [part][e]
-    __shared__ int base[1024];                  // first sorted position of (part, e)
-    __shared__ int off[kMaxExperts + 1];
-    __shared__ int pfirst[kMaxExperts + 1];     // first problem index of each expert
-    __shared__ int s_idx[kMaxPairsLds];
-    const int tid = threadIdx.x;
-    const bool staged = p.P <= kMaxPairsLds;
-    if (staged)
-        for (int q = tid; q < p.P; q += 1024) s_idx[q] = p.idx[q];
+    __shared__ int tot[kMaxExperts + 1];                    // rows per expert
+    __shared__ int off[kMaxExperts + 2];                    // first sorted row of each expert
+    __shared__ int pfirst[kMaxExperts + 2];                 // first (small or VALU) problem of each expert
+    __shared__ int bfirst[kMaxExperts + 2];                 // first big problem of each expert
+    __shared__ int done[kMaxExperts + 1];                   // rows of the expert placed so far
+    __shared__ unsigned long long mask[kMaxExperts + 1];
+    __shared__ unsigned long long wave_sum[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int P = p.T * p.k;
+    const int E1 = p.E + (p.shared_rows ? 1 : 0);           // experts including the always-on one
+
+    for (int e = tid; e <= p.E; e += 1024) { tot[e] = 0; done[e] = 0; mask[e] = 0; }
     __syncthreads();
-    const int* idx = staged ? s_idx : p.idx;
-    const int parts = max(1, 1024 / p.E);
-    const int seg = (p.P + parts - 1) / parts;
-    const int e = tid % p.E, part = tid / p.E;
-    const bool mine = part < parts;             // E <= 1024, so every expert has a thread
-    const int q0 = min(p.P, part * seg), q1 = min(p.P, q0 + seg);
-    if (mine) {
-        int c = 0;
-#pragma unroll 8
-        for (int q = q0; q < q1; ++q) c += (idx[q] == e);
-        cnt[part * p.E + e] = c;
-    }
+    for (int q = tid; q < P; q += 1024) atomicAdd(&tot[p.idx[q]], 1);
+    if (p.shared_rows && tid == 0) tot[p.E] = p.T;
     __syncthreads();
-    if (tid < p.E) {                            // total of expert tid, kept in pfirst for now
-        int c = 0;
-        for (int pt = 0; pt < parts; ++pt) c += cnt[pt * p.E + tid];
-        pfirst[tid] = c;
-    }
-    __syncthreads();
-    if (tid == 0) {
-        int run = 0, np = 0;
-        for (int x = 0; x < p.E; ++x) {
-            const int m = pfirst[x];
-            off[x] = run;
-            pfirst[x] = np;
-            if (m > 0) np += p.use_valu ? 1 : (m + kGemmRows - 1) / kGemmRows;
-            run += m;
+
+    // exclusive scan over the experts of (rows, small problems, big problems), packed
+    // in one 64-bit add: 22 + 21 + 21 bits
+    {
+        const int c = tid < E1 ? tot[tid] : 0;
+        int nbig = 0, nsmall = 0;
+        if (c > 0) {
+            if (p.use_valu) nsmall = 1;
+            else {
+                nbig = p.big_min <= kGemmBigRows ? c / kGemmBigRows : 0;
+                int rem = c - nbig * kGemmBigRows;
+                if (rem >= p.big_min) { ++nbig; rem = 0; }
+                nsmall = (rem + kGemmRows - 1) / kGemmRows;
+            }
         }
-        off[p.E] = run;
-        pfirst[p.E] = np;
-        p.counts[0] = p.use_valu ? np : 0;
-        p.counts[1] = p.use_valu ? 0 : np;
+        const unsigned long long mine = ((unsigned long long)nbig << 43) | ((unsigned long long)nsmall << 22) | (unsigned)c;
+        unsigned long long v = mine;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const unsigned long long o = __shfl_up(v, d, 64);
+            if (lane >= d) v += o;
+        }
+        if (lane == 63) wave_sum[wave] = v;
+        __syncthreads();
+        unsigned long long before = 0;
+        for (int w = 0; w < wave; ++w) before += wave_sum[w];
+        const unsigned long long excl = before + v - mine;
+        if (tid < E1) {
+            off[tid] = (int)(excl & 0x3fffffu);
+            pfirst[tid] = (int)((excl >> 22) & 0x1fffffu);
+            bfirst[tid] = (int)(excl >> 43);
+        }
+        if (tid == E1 - 1) {
+            const unsigned long long all = excl + mine;
+            off[E1] = (int)(all & 0x3fffffu);
+            const int total_small = (int)((all >> 22) & 0x1fffffu);
+            p.counts[0] = p.use_valu ? total_small : 0;
+            p.counts[1] = p.use_valu ? 0 : total_small;
+            p.counts[2] = (int)(all >> 43);
+        }
     }
     __syncthreads();
     for (int x = tid; x <= p.E; x += 1024) p.offsets[x] = off[x];
-    if (tid < p.E) {
-        int run = off[tid];
-        for (int pt = 0; pt < parts; ++pt) {
-            base[pt * p.E + tid] = run;
-            run += cnt[pt * p.E + tid];
-        }
-        const int m = off[tid + 1] - off[tid];
+    if (tid < E1) {
+        const int m = tot[tid];
         if (m > 0) {
             if (p.use_valu) {
                 p.vprob[pfirst[tid]] = GroupProblem{tid, off[tid], m, 0};
             } else {
-                for (int r = 0, j = pfirst[tid]; r < m; r += kGemmRows, ++j)
+                int r = 0;
+                for (int j = bfirst[tid]; m - r >= p.big_min; r += kGemmBigRows, ++j)
+                    p.bprob[j] = GroupProblem{tid, off[tid] + r, min(kGemmBigRows, m - r), 0};
+                for (int j = pfirst[tid]; r < m; r += kGemmRows, ++j)
                     p.mprob[j] = GroupProblem{tid, off[tid] + r, min(kGemmRows, m - r), 0};
             }
         }
     }
-    __syncthreads();
-    if (mine && cnt[part * p.E + e] > 0) {
-        int at = base[part * p.E + e];
-        for (int q = q0; q < q1; ++q) {
-            if (idx[q] == e) {
-                p.perm[at] = q;
-                p.inv[q] = at;
-                p.row_expert[at] = e;
-                ++at;
-            }
+
+    for (int t0 = 0; t0 < p.T; t0 += 64) {
+        const int nq = min(64, p.T - t0) * p.k;
+        const int q0 = t0 * p.k;
+        for (int i = tid; i < nq; i += 1024) atomicOr(&mask[p.idx[q0 + i]], 1ull << (i / p.k));
+        __syncthreads();
+        for (int i = tid; i < nq; i += 1024) {
+            const int q = q0 + i, e = p.idx[q];
+            const int at = off[e] + done[e] + __popcll(mask[e] & ((1ull << (i / p.k)) - 1ull));
+            p.perm[at] = q;
+            p.inv[q] = at;
+            p.row_expert[at] = e;
+        }
+        __syncthreads();
+        for (int e = tid; e < p.E; e += 1024) {
+            done[e] += __popcll(mask[e]);
+            mask[e] = 0;
+        }
+        __syncthreads();
+    }
+    if (p.shared_rows) {
+        for (int t = tid; t < p.T; t += 1024) {
+            p.perm[P + t] = t * p.k;
+            p.row_expert[P + t] = p.E;
         }
     }
 }
@@ -260,6 +450,8 @@ struct HadRowsParams {
     int gather_div;
     const int32_t* row_expert;
     const ExpertLin* experts;
+    ExpertLin shared[3];        // the always-on expert (row_expert == shared_expert)
+    int shared_expert;
     int lins_per_expert, lin_base;
     _Float16* out[2];           // per blockIdx.z
     int P, K;
@@ -268,26 +460,32 @@ struct HadRowsParams {
 __global__ __launch_bounds__(256) void moe_had_rows_kernel(HadRowsParams p)
 {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int r = blockIdx.y;
-    const int kb = blockIdx.x * 4 + wave;
-    if (kb * 128 >= p.K) return;
-    const int which = blockIdx.z;
-    const ExpertLin lin = p.experts[p.row_expert[r] * p.lins_per_expert + p.lin_base + which];
+    const int r = blockIdx.x;
+    const int which = blockIdx.y;
+    const int ex = p.row_expert[r];
+    const ExpertLin lin = ex == p.shared_expert ? p.shared[p.lin_base + which]
+                                                : p.experts[ex * p.lins_per_expert + p.lin_base + which];
     const int src = p.gather ? p.gather[r] / p.gather_div : r;
-    half2_t x = ((const half2_t*)(p.a + (size_t)src * p.K + kb * 128))[lane];
-    if (p.a_up) {
-        const half2_t u = ((const half2_t*)(p.a_up + (size_t)src * p.K + kb * 128))[lane];
-        x.x = silu_mul_h(x.x, u.x);
-        x.y = silu_mul_h(x.y, u.y);
+    const half2_t* xrow = (const half2_t*)(p.a + (size_t)src * p.K);
+    const half2_t* urow = p.a_up ? (const half2_t*)(p.a_up + (size_t)src * p.K) : nullptr;
+    const half2_t* srow = (const half2_t*)lin.suh;
+    half2_t* orow = (half2_t*)(p.out[which] + (size_t)r * p.K);
+    for (int kb = wave; kb * 128 < p.K; kb += 4) {
+        half2_t x = xrow[kb * 64 + lane];
+        if (urow) {
+            const half2_t u = urow[kb * 64 + lane];
+            x.x = silu_mul_h(x.x, u.x);
+            x.y = silu_mul_h(x.y, u.y);
+        }
+        const half2_t sc = srow[kb * 64 + lane];
+        float v0 = (float)x.x * (float)sc.x;
+        float v1 = (float)x.y * (float)sc.y;
+        had128_wave(v0, v1, lane);
+        half2_t o;
+        o.x = (_Float16)(v0 * kRsqrt128);
+        o.y = (_Float16)(v1 * kRsqrt128);
+        orow[kb * 64 + lane] = o;
     }
-    const half2_t sc = ((const half2_t*)(lin.suh + kb * 128))[lane];
-    float v0 = (float)x.x * (float)sc.x;
-    float v1 = (float)x.y * (float)sc.y;
-    had128_wave(v0, v1, lane);
-    half2_t o;
-    o.x = (_Float16)(v0 * kRsqrt128);
-    o.y = (_Float16)(v1 * kRsqrt128);
-    ((half2_t*)(p.out[which] + (size_t)r * p.K + kb * 128))[lane] = o;
 }
 
 // ---------------------------------------------------------------- combine
@@ -318,41 +516,73 @@ thread_local std::string g_moe_err, g_moe_launch;
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct MoeLayout {
-    size_t idx, w, parts, offsets, perm, inv, row_expert, counts, vprob, mprob;
+    size_t idx, w, parts, offsets, perm, inv, row_expert, counts, vprob, mprob, bprob;
     size_t ah0, ah1, g, u, ahd, slot_out, sg, su, s_ahad, shared_out, total;
-    int max_v, max_m, nseg;
+    int max_v, max_m, max_b, nseg;
 };
+
+// Experts with many rows can be cut into 128-row MFMA problems (a remainder of at
+// least BERTH_MOE_BIG_MIN rows, 65 is the natural value, becomes one more).  Off by
+// default: at the measured shapes 32-row problems alone are faster, because the
+// 128-row tile spends more time per k-block than four 32-row tiles running side by
+// side.
+int moe_big_min()
+{
+    static const int v = [] {
+        const char* e = std::getenv("BERTH_MOE_BIG_MIN");
+        return e ? std::atoi(e) : 0;
+    }();
+    return v;
+}
+
+// The always-on expert runs as one more expert of the grouped launches (rows P ..
+// P + T - 1, token order) when it has the routed experts' intermediate size.
+bool shared_is_folded(int I, int shared_I) { return shared_I > 0 && shared_I == I; }
 
 MoeLayout moe_layout(int T, int H, int E, int k, int I, int shared_I)
 {
     MoeLayout L{};
     const size_t P = (size_t)T * k;
+    const bool fold = shared_is_folded(I, shared_I);
+    const size_t R = P + (fold ? (size_t)T : 0);        // rows of the grouped launches
     L.nseg = (H + kRouteSeg - 1) / kRouteSeg;
-    const bool use_valu = P <= (size_t)kValuPairs;
-    L.max_v = use_valu ? (int)std::min<size_t>((size_t)E, P) : 0;
-    L.max_m = use_valu ? 0 : (int)(std::min<size_t>((size_t)E, P) + P / kGemmRows + 1);
+    const bool use_valu = T == 1 || R <= (size_t)kValuPairs;      // one row per problem, or very few rows
+    L.max_v = use_valu ? (int)(std::min<size_t>((size_t)E, P) + (fold ? 1 : 0)) : 0;
+    // an expert leaves at most two small problems (fewer than 65 rows) next to its big ones
+    const size_t E1 = (size_t)E + (fold ? 1 : 0);
+    const int big_min = moe_big_min();
+    const bool big = big_min > 0 && big_min <= kGemmBigRows;
+    L.max_m = use_valu ? 0 : (int)(big ? std::min<size_t>(((size_t)big_min / kGemmRows + 1) * E1, R)
+                                       : std::min<size_t>(E1, R) + R / kGemmRows + 1);
+    L.max_b = (use_valu || !big) ? 0 : (int)(R / big_min);
     size_t at = 0;
     auto take = [&](size_t bytes) { size_t r = at; at = align_up(at + bytes); return r; };
     L.idx = take(P * 4);
     L.w = take(P * 4);
     L.parts = take((size_t)T * L.nseg * E * 4);
     L.offsets = take((size_t)(E + 1) * 4);
-    L.perm = take(P * 4);
+    L.perm = take(R * 4);
     L.inv = take(P * 4);
-    L.row_expert = take(P * 4);
+    L.row_expert = take(R * 4);
     L.counts = take(16);
     L.vprob = take((size_t)std::max(L.max_v, 1) * sizeof(GroupProblem));
     L.mprob = take((size_t)std::max(L.max_m, 1) * sizeof(GroupProblem));
-    L.ah0 = take(L.max_m ? P * H * 2 : 0);
-    L.ah1 = take(L.max_m ? P * H * 2 : 0);
-    L.g = take(P * I * 2);
-    L.u = take(P * I * 2);
-    L.ahd = take(L.max_m ? P * I * 2 : 0);
-    L.slot_out = take(P * H * 4);
-    L.sg = take((size_t)T * shared_I * 2);
-    L.su = take((size_t)T * shared_I * 2);
-    L.s_ahad = take((size_t)T * std::max(H, shared_I) * 2);
-    L.shared_out = take(shared_I ? (size_t)T * H * 4 : 0);
+    L.bprob = take((size_t)std::max(L.max_b, 1) * sizeof(GroupProblem));
+    L.ah0 = take(L.max_m ? R * H * 2 : 0);
+    L.ah1 = take(L.max_m ? R * H * 2 : 0);
+    L.g = take(R * I * 2);
+    L.u = take(R * I * 2);
+    L.ahd = take(L.max_m ? R * I * 2 : 0);
+    L.slot_out = take(R * H * 4);
+    if (fold) {
+        L.sg = L.su = L.s_ahad = at;
+        L.shared_out = L.slot_out + P * H * 4;
+    } else {
+        L.sg = take((size_t)T * shared_I * 2);
+        L.su = take((size_t)T * shared_I * 2);
+        L.s_ahad = take((size_t)T * std::max(H, shared_I) * 2);
+        L.shared_out = take(shared_I ? (size_t)T * H * 4 : 0);
+    }
     L.total = at;
     return L;
 }
@@ -383,14 +613,23 @@ std::string run_route(const void* x, const void* wr, const float* bias, int32_t*
     p.nseg = (H + kRouteSeg - 1) / kRouteSeg;
     const int groups = (T + kRouteTT - 1) / kRouteTT;
     if (groups > kCounters) throw std::runtime_error("moe route: too many tokens for the counter table");
+    if (T >= kRouteBigT) {
+        dim3 grid(p.nseg, (T + kRouteBigTT - 1) / kRouteBigTT);
+        hipLaunchKernelGGL(moe_route_partial_kernel, grid, dim3(256), 0, stream, p);
+        hip_ok(hipGetLastError(), "moe_route_partial_kernel launch");
+        hipLaunchKernelGGL(moe_route_finish_kernel, dim3(T), dim3(256), 0, stream, p);
+        hip_ok(hipGetLastError(), "moe_route_finish_kernel launch");
+        return "moe_route_partial_kernel grid=" + std::to_string(grid.x) + "x" + std::to_string(grid.y) +
+               " + moe_route_finish_kernel grid=" + std::to_string(T);
+    }
     dim3 grid(p.nseg, groups);
     hipLaunchKernelGGL(moe_route_kernel, grid, dim3(256), 0, stream, p);
     hip_ok(hipGetLastError(), "moe_route_kernel launch");
     return "moe_route_kernel grid=" + std::to_string(grid.x) + "x" + std::to_string(grid.y);
 }
 
-std::string run_permute(const int32_t* idx, unsigned char* wsb, const MoeLayout& L, int P, int E,
-                        hipStream_t stream)
+std::string run_permute(const int32_t* idx, unsigned char* wsb, const MoeLayout& L, int T, int k, int E,
+                        bool fold, hipStream_t stream)
 {
     PermuteParams p{};
     p.idx = idx;
@@ -401,9 +640,13 @@ std::string run_permute(const int32_t* idx, unsigned char* wsb, const MoeLayout&
     p.counts = (int32_t*)(wsb + L.counts);
     p.vprob = (GroupProblem*)(wsb + L.vprob);
     p.mprob = (GroupProblem*)(wsb + L.mprob);
-    p.P = P;
+    p.bprob = (GroupProblem*)(wsb + L.bprob);
+    p.T = T;
+    p.k = k;
     p.E = E;
     p.use_valu = L.max_v > 0 ? 1 : 0;
+    p.shared_rows = fold ? 1 : 0;
+    p.big_min = L.max_b > 0 ? moe_big_min() : (1 << 30);
     hipLaunchKernelGGL(moe_permute_kernel, dim3(1), dim3(1024), 0, stream, p);
     hip_ok(hipGetLastError(), "moe_permute_kernel launch");
     return "moe_permute_kernel";
@@ -470,9 +713,13 @@ extern "C" int berth_moe_permute(const int32_t* idx, int32_t* offsets, int32_t* 
     p.counts = (int32_t*)(sb + at); at = align_up(at + 16);
     p.vprob = (GroupProblem*)(sb + at); at = align_up(at + (std::min<size_t>(E, P)) * sizeof(GroupProblem));
     p.mprob = (GroupProblem*)(sb + at);
-    p.P = (int)P;
+    p.bprob = p.mprob;
+    p.T = T;
+    p.k = k;
     p.E = E;
-    p.use_valu = P <= (size_t)kValuPairs ? 1 : 0;
+    p.use_valu = (T == 1 || P <= (size_t)kValuPairs) ? 1 : 0;
+    p.shared_rows = 0;
+    p.big_min = 1 << 30;
     hipLaunchKernelGGL(moe_permute_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, p);
     hip_ok(hipGetLastError(), "moe_permute_kernel launch");
     g_moe_launch = "moe_permute_kernel";
@@ -508,21 +755,31 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
     if (shared && (shared_I < 128 || shared_I % 128))
         throw std::runtime_error("moe layer: shared intermediate size must be a multiple of 128");
     if (!shared) shared_I = 0;
+    const bool fold = shared_is_folded(I, shared_I);
+    if (fold && E + 1 > kMaxExperts) throw std::runtime_error("moe: at most 1023 routed experts next to a shared expert");
     const MoeLayout L = moe_layout(T, H, E, k, I, shared_I);
     if (workspace_bytes < L.total)
         throw std::runtime_error("moe layer: workspace too small (" + std::to_string(workspace_bytes) + " < " +
                                  std::to_string(L.total) + ")");
     unsigned char* wsb = (unsigned char*)workspace;
     const int P = T * k;
+    const int R = P + (fold ? T : 0);
     int32_t* idx = (int32_t*)(wsb + L.idx);
     float* w = (float*)(wsb + L.w);
     std::string desc;
+    if (shared)
+        for (int i = 0; i < 3; ++i)
+            if (!shared[i].trellis || !shared[i].suh || !shared[i].svh)
+                throw std::runtime_error("moe layer: null shared-expert pointer");
 
     desc += run_route(x, wr, bias, idx, w, nullptr, (float*)(wsb + L.parts), T, H, E, k, renorm, stream);
-    desc += " + " + run_permute(idx, wsb, L, P, E, stream);
+    desc += " + " + run_permute(idx, wsb, L, T, k, E, fold, stream);
 
     GroupedArgs g{};
     g.experts = experts;
+    g.shared = fold ? shared : nullptr;
+    g.shared_expert = fold ? E : -1;
+    g.single_row = T == 1 ? 1 : 0;
     g.lins_per_expert = 3;
     g.k_bits = k_bits;
     g.codebook = codebook;
@@ -553,20 +810,31 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
         h.gather_div = k;
         h.row_expert = (const int32_t*)(wsb + L.row_expert);
         h.experts = (const ExpertLin*)experts;
+        h.shared_expert = g.shared_expert;
+        if (fold) for (int i = 0; i < 3; ++i) h.shared[i] = ExpertLin{(const uint32_t*)shared[i].trellis, (const _Float16*)shared[i].suh, (const _Float16*)shared[i].svh};
         h.lins_per_expert = 3;
         h.lin_base = 0;
         h.out[0] = (_Float16*)(wsb + L.ah0);
         h.out[1] = (_Float16*)(wsb + L.ah1);
-        h.P = P;
+        h.P = R;
         h.K = H;
-        hipLaunchKernelGGL(moe_had_rows_kernel, dim3((H / 128 + 3) / 4, P, 2), dim3(256), 0, stream, h);
+        hipLaunchKernelGGL(moe_had_rows_kernel, dim3(R, 2), dim3(256), 0, stream, h);
         hip_ok(hipGetLastError(), "moe_had_rows_kernel launch");
+        g.a_had = wsb + L.ah0;
+        g.a_had2 = wsb + L.ah1;
+        desc += " + moe_had_rows_kernel";
+        if (L.max_b > 0) {
+            g.problems = wsb + L.bprob;
+            g.num_problems = (const int*)(wsb + L.counts) + 2;
+            g.max_problems = L.max_b;
+            g.mb = kGemmBigRows / 32;
+            desc += " + " + launch_gemm_grouped(g);
+        }
         g.problems = wsb + L.mprob;
         g.num_problems = (const int*)(wsb + L.counts) + 1;
         g.max_problems = L.max_m;
-        g.a_had = wsb + L.ah0;
-        g.a_had2 = wsb + L.ah1;
-        desc += " + moe_had_rows_kernel + " + launch_gemm_grouped(g);
+        g.mb = 1;
+        desc += " + " + launch_gemm_grouped(g);
     }
 
     // down: input silu(g) * u evaluated while the activation is rotated, fp32 out
@@ -594,27 +862,38 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
         h.gather_div = 1;
         h.row_expert = (const int32_t*)(wsb + L.row_expert);
         h.experts = (const ExpertLin*)experts;
+        h.shared_expert = g.shared_expert;
+        if (fold) for (int i = 0; i < 3; ++i) h.shared[i] = ExpertLin{(const uint32_t*)shared[i].trellis, (const _Float16*)shared[i].suh, (const _Float16*)shared[i].svh};
         h.lins_per_expert = 3;
         h.lin_base = 2;
         h.out[0] = (_Float16*)(wsb + L.ahd);
-        h.P = P;
+        h.P = R;
         h.K = I;
-        hipLaunchKernelGGL(moe_had_rows_kernel, dim3((I / 128 + 3) / 4, P, 1), dim3(256), 0, stream, h);
+        hipLaunchKernelGGL(moe_had_rows_kernel, dim3(R, 1), dim3(256), 0, stream, h);
         hip_ok(hipGetLastError(), "moe_had_rows_kernel launch");
+        g.a_had = wsb + L.ahd;
+        g.a_had2 = nullptr;
+        desc += " + moe_had_rows_kernel";
+        if (L.max_b > 0) {
+            g.problems = wsb + L.bprob;
+            g.num_problems = (const int*)(wsb + L.counts) + 2;
+            g.max_problems = L.max_b;
+            g.mb = kGemmBigRows / 32;
+            desc += " + " + launch_gemm_grouped(g);
+        }
         g.problems = wsb + L.mprob;
         g.num_problems = (const int*)(wsb + L.counts) + 1;
         g.max_problems = L.max_m;
-        g.a_had = wsb + L.ahd;
-        g.a_had2 = nullptr;
-        desc += " + moe_had_rows_kernel + " + launch_gemm_grouped(g);
+        g.mb = 1;
+        desc += " + " + launch_gemm_grouped(g);
     }
 
     // shared expert: three dense linears on every token
     const float* shared_out = nullptr;
-    if (shared) {
-        for (int i = 0; i < 3; ++i)
-            if (!shared[i].trellis || !shared[i].suh || !shared[i].svh)
-                throw std::runtime_error("moe layer: null shared-expert pointer");
+    if (fold) {
+        shared_out = (const float*)(wsb + L.shared_out);
+        desc += " (shared expert in the grouped launches)";
+    } else if (shared) {
         auto dense = [&](const void* a, const berth_exl3_lin& lin, void* c, int kk, int nn, int fp32) {
             LinearArgs la{a, lin.trellis, c, lin.suh, wsb + L.s_ahad, lin.svh, T, kk, nn, k_bits, codebook, fp32, stream};
             return T <= 8 ? launch_gemv(la) : launch_gemm(la);

@@ -169,8 +169,10 @@ def test_moe_layer_matches_oracle(T, H, E, k, I, bits, shared_I, scale):
     # whole-layer error relative to the output scale
     err = np.abs(out.cpu().numpy() - want)
     assert err.max() <= 2e-3 * np.abs(want).max(), (err.max(), np.abs(want).max(), launch)
-    if T * k > 8:
+    if T > 1 and T * k + (T if shared_I == I else 0) > 8:
         assert "exl3_gemm_kernel" in launch and "exl3_gemv_kernel" not in launch
+        import os
+        assert ("128x256" in launch) == (os.environ.get("BERTH_MOE_BIG_MIN", "0") not in ("", "0") and T * k >= 65)
     else:
         assert "exl3_gemv_kernel" in launch and "exl3_gemm_kernel" not in launch
     # a second call reuses the workspace and the self-resetting counters
@@ -221,6 +223,22 @@ def test_moe_config4_shape_zipf_shared():
     assert np.allclose(w.cpu().numpy(), ow, rtol=1e-5, atol=1e-7)
     _check_stages(layer, x, experts_np, shared_np, oi, w.cpu().numpy(), out.cpu().numpy(), T, H, E, k, I, bits, I)
     assert np.abs(out.cpu().numpy() - want).max() <= 2e-3 * np.abs(want).max()
+
+
+def test_moe_layer_with_128_row_problems():
+    """The optional 128-row MFMA problems (BERTH_MOE_BIG_MIN, read once per process)
+    in a process of their own: the skewed case and the long-list case again."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, BERTH_MOE_BIG_MIN="65")
+    r = subprocess.run([sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", os.path.abspath(__file__), "-k",
+                        "test_moe_layer_matches_oracle and (70-256 or 300-128)"],
+                       cwd=root, env=env, capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-2000:]
+    assert "2 passed" in r.stdout, r.stdout[-2000:]
 
 
 def test_moe_validation_errors():
