@@ -34,7 +34,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per GEMV launch of the default workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs scaled by a 1 GiB copy (profiles/exl3_gemv_4bpw_batch1_27b_linear_set.md)
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {4: int((24589 + 428) * 1024)}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {4: int((42787 + 604) * 1024)}
 ORDER = ["q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"]
 OUT_FP32 = {"q_proj": False, "k_proj": False, "v_proj": False, "o_proj": True,
             "gate_proj": False, "up_proj": False, "down_proj": True}
@@ -60,7 +60,7 @@ def cpu_baseline(bits: int, seconds: float):
         O.gemv_fused(x, tr, suh, svh, K, N, bits, 2, out_fp32=False)
         reps += 1
         dt = time.perf_counter() - t0
-        if dt >= seconds or reps >= 200:
+        if dt >= seconds:
             break
     nbytes = linear_bytes(K, N, bits, 1, 2) * reps
     return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": O.num_threads(), "kind": "port",

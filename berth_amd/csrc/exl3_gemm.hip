@@ -57,8 +57,11 @@ std::string launch_gemm(const LinearArgs& a)
     p.out_fp32 = a.out_fp32;
     p.partials = ws.partials;
     p.counters = ws.counters;
-    const int mb = a.size_m <= 32 ? 1 : 4;
+    // 128-row tiles decode a weight once per 128 rows, but need enough tiles to spread
+    // over the chip; narrow outputs (few column tiles) run as 32-row tiles instead
     const int nblocks = (a.size_n + 255) / 256;
+    const long tiles128 = (long)nblocks * ((a.size_m + 127) / 128);
+    const int mb = (a.size_m <= 32 || tiles128 * 4 < ws.cu_count) ? 1 : 4;
     const int mtiles = (a.size_m + mb * 32 - 1) / (mb * 32);
     p.S = gemm_split(ws, (long)nblocks * mtiles, a.size_k / 128, mb);
     std::string desc;

@@ -278,30 +278,31 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
             for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
                 for (int f = 0; f < 2; ++f) {
+                    if (mb * 32 >= rows_here) continue;
+                    // sixteen registers x four splits in flight together; adds in split order
+                    float sum[16];
 #pragma unroll
-                    for (int r4 = 0; r4 < 4; ++r4) {
-                        if (mb * 32 + 8 * r4 >= rows_here) continue;
-                        float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-                        for (int ss = 0; ss < p.S; ss += 4) {
-                            float part[4][4];
+                    for (int r = 0; r < 16; ++r) sum[r] = 0.0f;
+                    for (int ss = 0; ss < p.S; ss += 4) {
+                        float part[4][16];
 #pragma unroll
-                            for (int j = 0; j < 4; ++j)
+                        for (int j = 0; j < 4; ++j) {
+                            const int sj = ss + j < p.S ? ss + j : p.S - 1;      // past the end: re-read, ignored
 #pragma unroll
-                                for (int q = 0; q < 4; ++q)
-                                    part[j][q] = (ss + j < p.S)
-                                        ? __hip_atomic_load(all + (size_t)(ss + j) * kPerWg +
-                                                                ((mb * 2 + f) * 16 + 4 * r4 + q) * 64 + lane,
-                                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                                        : 0.0f;
-#pragma unroll
-                            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                                for (int q = 0; q < 4; ++q)
-                                    if (ss + j < p.S) sum[q] += part[j][q];
+                            for (int r = 0; r < 16; ++r)
+                                part[j][r] = __hip_atomic_load(all + (size_t)sj * kPerWg + ((mb * 2 + f) * 16 + r) * 64 + lane,
+                                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         }
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) acc[mb][f][4 * r4 + q] = sum[q];
+                        for (int j = 0; j < 4; ++j)
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) {
+                                const float nv = sum[r] + part[j][r];
+                                sum[r] = ss + j < p.S ? nv : sum[r];
+                            }
                     }
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[mb][f][r] = sum[r];
                 }
         }
     }
