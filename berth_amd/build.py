@@ -54,7 +54,20 @@ def build_all(jobs: int = 8, only: str | None = None) -> list[str]:
         if r.returncode != 0:
             raise RuntimeError(f"link failed for {name}:\n{r.stderr[-4000:]}")
         built.append(out)
+    if only is None:
+        built.append(build_host_check())
     return built
+
+
+def build_host_check() -> str:
+    """The C++ host layer's check program (csrc/host): plain C++ over the two C ABIs."""
+    out = os.path.join(LIB, "berth_host_check")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", os.path.join(CSRC, "host", "host_check.cpp"), "-o", out,
+           "-L" + LIB, "-lberth_kernels_hip", "-lberth_hip", "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"host check build failed:\n{r.stderr[-4000:]}")
+    return out
 
 
 if __name__ == "__main__":

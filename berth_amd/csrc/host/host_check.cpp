@@ -1,0 +1,164 @@
+// Runs the C++ host layer (engine.hpp) on case files written by the test suite and
+// writes the results back, so that the tests can compare them with the CPU oracle:
+//   host_check linear <dir>   meta.txt: K N rows out_fp32 mode(0 forward/forward_n, 1 forward_rows)
+//   host_check mlp <dir>      meta.txt: hidden intermediate rows
+//   host_check moe <dir>      meta.txt: tokens hidden experts top_k intermediate shared(0/1) has_bias(0/1)
+// Tensors are raw little-endian files in <dir>; outputs go to <dir>/y.bin (+ idx.bin).
+#include "engine.hpp"
+
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+#include <sstream>
+
+using namespace berth::engine;
+
+template <typename T>
+static std::vector<T> read_file(const std::string& path)
+{
+    std::ifstream f(path, std::ios::binary | std::ios::ate);
+    if (!f) throw std::runtime_error("cannot open " + path);
+    const std::streamsize n = f.tellg();
+    f.seekg(0);
+    std::vector<T> v((size_t)n / sizeof(T));
+    f.read((char*)v.data(), n);
+    return v;
+}
+
+template <typename T>
+static void write_file(const std::string& path, const std::vector<T>& v)
+{
+    std::ofstream f(path, std::ios::binary);
+    f.write((const char*)v.data(), (std::streamsize)(v.size() * sizeof(T)));
+}
+
+static std::vector<long> read_meta(const std::string& dir)
+{
+    std::ifstream f(dir + "/meta.txt");
+    if (!f) throw std::runtime_error("cannot open " + dir + "/meta.txt");
+    std::vector<long> v;
+    long x;
+    while (f >> x) v.push_back(x);
+    return v;
+}
+
+static Exl3Linear load_linear(const Gpu& gpu, const std::string& dir, const std::string& name, int K, int N)
+{
+    const auto tr = read_file<uint16_t>(dir + "/" + name + ".trellis.bin");
+    const auto suh = read_file<Half>(dir + "/" + name + ".suh.bin");
+    const auto svh = read_file<Half>(dir + "/" + name + ".svh.bin");
+    if ((int)suh.size() != K || (int)svh.size() != N) throw InputError(name + ": suh / svh length");
+    return Exl3Linear(gpu, name, tr.data(), tr.size(), suh.data(), K, svh.data(), N);
+}
+
+static int run_linear(const Gpu& gpu, const std::string& dir)
+{
+    const auto m = read_meta(dir);
+    const int K = (int)m.at(0), N = (int)m.at(1), rows = (int)m.at(2);
+    const OutDtype out = m.at(3) ? OutDtype::F32 : OutDtype::F16;
+    const bool use_rows = m.at(4) != 0;
+    Exl3Linear lin = load_linear(gpu, dir, "lin", K, N);
+    const auto x = DeviceBuffer<Half>::from_host(gpu, read_file<Half>(dir + "/x.bin"));
+    auto c = DeviceBuffer<uint8_t>::zeroed(gpu, (size_t)rows * N * out_bytes(out));
+
+    // a buffer that is too small is refused before anything is launched (device.rs:132-140)
+    bool refused = false;
+    try {
+        lin.forward(gpu, x, c.ptr(), 2, out);
+    } catch (const InputError&) {
+        refused = true;
+    }
+    if (!refused) throw std::runtime_error("short output buffer was not refused");
+
+    berth_hip_event *e0 = nullptr, *e1 = nullptr;
+    device_ok(berth_hip_event_new(gpu.context(), &e0), "event");
+    device_ok(berth_hip_event_new(gpu.context(), &e1), "event");
+    device_ok(berth_hip_event_record(e0, gpu.stream()), "record");
+    if (use_rows) {
+        RowScratch scratch(gpu, rows, K, N);
+        lin.forward_rows(gpu, scratch, x, c.ptr(), c.num_bytes(), rows, out);
+    } else {
+        auto a_had = DeviceBuffer<Half>::zeroed(gpu, (size_t)rows * K);
+        lin.forward_n(gpu, a_had, x, c.ptr(), c.num_bytes(), rows, out);
+    }
+    device_ok(berth_hip_event_record(e1, gpu.stream()), "record");
+    device_ok(berth_hip_event_synchronize(e1), "event synchronize");
+    float ms = -1.0f;
+    device_ok(berth_hip_event_elapsed_ms(e0, e1, &ms), "elapsed");
+    berth_hip_event_free(e0);
+    berth_hip_event_free(e1);
+    write_file(dir + "/y.bin", c.copy_to_host());
+    std::printf("linear ok rows=%d elapsed_ms=%.3f launch=%s\n", rows, ms,
+                rows == 1 ? berth_exl3_last_launch() : berth_prefill_last_launch());
+    return 0;
+}
+
+static int run_mlp(const Gpu& gpu, const std::string& dir)
+{
+    const auto m = read_meta(dir);
+    const int H = (int)m.at(0), I = (int)m.at(1), rows = (int)m.at(2);
+    MlpLayer mlp(gpu, load_linear(gpu, dir, "gate", H, I), load_linear(gpu, dir, "up", H, I),
+                 load_linear(gpu, dir, "down", I, H), rows);
+    const auto x = DeviceBuffer<Half>::from_host(gpu, read_file<Half>(dir + "/x.bin"));
+    auto y = DeviceBuffer<float>::zeroed(gpu, (size_t)rows * H);
+    if (rows == 1) {
+        mlp.forward(gpu, x, y);
+    } else {
+        RowScratch scratch(gpu, rows, H > I ? H : I, H > I ? H : I);
+        mlp.prefill(gpu, scratch, x, y, rows);
+    }
+    gpu.synchronize();
+    write_file(dir + "/y.bin", y.copy_to_host());
+    std::printf("mlp ok rows=%d\n", rows);
+    return 0;
+}
+
+static int run_moe(const Gpu& gpu, const std::string& dir)
+{
+    const auto m = read_meta(dir);
+    const int T = (int)m.at(0), H = (int)m.at(1), E = (int)m.at(2), k = (int)m.at(3), I = (int)m.at(4);
+    const bool shared = m.at(5) != 0, has_bias = m.at(6) != 0;
+    std::vector<MoeLayer::Expert> experts;
+    for (int e = 0; e < E; ++e) {
+        const std::string p = "e" + std::to_string(e);
+        experts.push_back(MoeLayer::Expert{load_linear(gpu, dir, p + ".gate", H, I), load_linear(gpu, dir, p + ".up", H, I),
+                                           load_linear(gpu, dir, p + ".down", I, H)});
+    }
+    const auto router = read_file<Half>(dir + "/router.bin");
+    std::vector<float> bias;
+    if (has_bias) bias = read_file<float>(dir + "/bias.bin");
+    MoeLayer layer(gpu, router.data(), H, E, std::move(experts), k, has_bias ? bias.data() : nullptr);
+    if (shared)
+        layer.set_shared(MoeLayer::Expert{load_linear(gpu, dir, "shared.gate", H, I), load_linear(gpu, dir, "shared.up", H, I),
+                                          load_linear(gpu, dir, "shared.down", I, H)});
+    const auto x = DeviceBuffer<Half>::from_host(gpu, read_file<Half>(dir + "/x.bin"));
+    auto y = DeviceBuffer<float>::zeroed(gpu, (size_t)T * H);
+    auto idx = DeviceBuffer<int32_t>::zeroed(gpu, (size_t)T * k);
+    layer.forward(gpu, x, y, T, &idx);
+    gpu.synchronize();
+    write_file(dir + "/y.bin", y.copy_to_host());
+    write_file(dir + "/idx.bin", idx.copy_to_host());
+    std::printf("moe ok tokens=%d launch=%s\n", T, berth_moe_last_launch());
+    return 0;
+}
+
+int main(int argc, char** argv)
+{
+    if (argc < 3) {
+        std::fprintf(stderr, "usage: host_check linear|mlp|moe <dir>\n");
+        return 2;
+    }
+    try {
+        Gpu gpu(0);
+        const std::string what = argv[1], dir = argv[2];
+        if (what == "linear") return run_linear(gpu, dir);
+        if (what == "mlp") return run_mlp(gpu, dir);
+        if (what == "moe") return run_moe(gpu, dir);
+        std::fprintf(stderr, "unknown case %s\n", what.c_str());
+        return 2;
+    } catch (const std::exception& e) {
+        std::fprintf(stderr, "host_check failed: %s\n", e.what());
+        return 1;
+    }
+}
