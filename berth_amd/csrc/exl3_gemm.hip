@@ -63,10 +63,13 @@ std::string launch_gemm(const LinearArgs& a)
     const long tiles128 = (long)nblocks * ((a.size_m + 127) / 128);
     const int mb = (a.size_m <= 32 || tiles128 * 4 < ws.cu_count) ? 1 : 4;
     const int mtiles = (a.size_m + mb * 32 - 1) / (mb * 32);
-    p.S = gemm_split(ws, (long)nblocks * mtiles, a.size_k / 128, mb);
-    std::string desc;
+    const long tiles = (long)nblocks * mtiles;
+    const int KB = a.size_k / 128;
     p.tiles_y = mtiles;
-    gemm_bits(p, a.k_bits, a.codebook, mb, a.stream, desc, dim3(nblocks * p.S, mtiles, 1));
+    std::string desc;
+    p.tile0 = 0;
+    p.S = gemm_split(ws, tiles, KB, mb);
+    gemm_bits(p, a.k_bits, a.codebook, mb, a.stream, desc, dim3((unsigned)(tiles * p.S), 1, 1));
     hip_ok(hipGetLastError(), "exl3_gemm_kernel launch");
     return d0 + " + " + desc + (a.out_fp32 ? " out=f32" : " out=f16");
 }

@@ -43,6 +43,7 @@ struct GemmParams {
     ExpertLin shared[3];        // an always-on expert passed by value (problem.expert == shared_expert)
     int shared_expert;
     int tiles_y;                // dense: row blocks; grouped: capacity of the problem list
+    int tile0;                  // dense: first (row block, column block) tile of this launch, row-major
     // split-K
     int S;
     float* partials;            // [unit][S][4 waves][MB][2][16][64]
@@ -53,7 +54,8 @@ constexpr int kAStride = 128 + 8;   // halves per LDS row of the A tile (272 B: 
 
 // one output tile: rows of problem / row block `tile_y`, 256 columns
 template <int BITS, int CB, int MB>  // MB = 32-row blocks per workgroup
-__device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y, const int which, unsigned char* smem)
+__device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y, const int nblk, const int split,
+                                          const int which, unsigned char* smem)
 {
     constexpr int BM = MB * 32;
     _Float16* a_tile = (_Float16*)smem;                 // [2][BM][kAStride]
@@ -65,8 +67,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
     const int wave = threadIdx.x >> 6;
     const int half_id = lane >> 5;                      // which of the two tile rows
     const int slot = lane & 31;                         // MFMA row / column slot
-    const int nblk = blockIdx.x / p.S;
-    const int split = blockIdx.x - nblk * p.S;
     const int n0 = nblk * 256;
     int m0 = tile_y * BM;
     int m_end = p.M;
@@ -248,7 +248,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
     // so only registers with 8*(r/4) < rows matter.
     if (p.S > 1) {
         const int nblocks = (p.N + 255) >> 8;
-        const size_t unit = ((size_t)which * p.tiles_y + tile_y) * nblocks + nblk;
+        // dense: tiles of this launch count from 0; grouped: (linear, problem, column block)
+        const size_t unit = p.problems ? ((size_t)which * p.tiles_y + tile_y) * nblocks + nblk
+                                       : (size_t)tile_y * nblocks + nblk - p.tile0;
         constexpr size_t kPerWg = (size_t)4 * MB * 2 * 16 * 64;
         float* mine = p.partials + (unit * p.S + split) * kPerWg + (size_t)wave * MB * 2 * 16 * 64;
         if (active) {
@@ -364,19 +366,25 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
     }
 }
 
-// Dense launches: blockIdx.y is the row block.  Grouped launches: blockIdx.z is the
-// problem and blockIdx.y the linear, so that the workgroups of the (few) real
-// problems of every linear are dispatched before the empty tail of the list.
+// Dense launches: blockIdx.x = (tile - tile0) * S + split with tiles numbered row
+// block by row block, so that one linear can be issued as several launches with
+// different split factors.  Grouped launches: blockIdx.x = column block * S + split,
+// blockIdx.y the linear, blockIdx.z the problem, so that the workgroups of the (few)
+// real problems of every linear are dispatched before the empty tail of the list.
 template <int BITS, int CB, int MB>
 __global__ __launch_bounds__(256, 2) void exl3_gemm_kernel(GemmParams p)
 {
     extern __shared__ __align__(16) unsigned char smem[];
+    const int unit = blockIdx.x / p.S;
+    const int split = blockIdx.x - unit * p.S;
     if (!p.problems) {
-        gemm_tile<BITS, CB, MB>(p, blockIdx.y, 0, smem);
+        const int nblocks = (p.N + 255) >> 8;
+        const int tile = p.tile0 + unit;
+        gemm_tile<BITS, CB, MB>(p, tile / nblocks, tile % nblocks, split, 0, smem);
         return;
     }
     if ((int)blockIdx.z >= *p.num_problems) return;
-    gemm_tile<BITS, CB, MB>(p, blockIdx.z, blockIdx.y, smem);
+    gemm_tile<BITS, CB, MB>(p, blockIdx.z, unit, split, blockIdx.y, smem);
 }
 
 }  // namespace berth

@@ -31,6 +31,23 @@ constexpr int kGemmBigRows = 128;   // rows per big MFMA problem
 
 // ------------------------------------------------------------------ route
 
+struct PermuteParams {
+    const int32_t* idx;     // [P] expert of each (token, slot) pair, P = T * k; distinct within a token
+    int32_t* offsets;       // [E + 1]
+    int32_t* perm;          // [R] sorted position -> pair (pair / k = token)
+    int32_t* inv;           // [P] pair -> sorted position
+    int32_t* row_expert;    // [R] sorted position -> expert
+    int32_t* counts;        // [3] number of VALU problems, small MFMA problems, big MFMA problems
+    GroupProblem* vprob;
+    GroupProblem* mprob;    // <= 32 rows each
+    GroupProblem* bprob;    // <= 128 rows each
+    int T, k, E;
+    int use_valu;           // 1: every expert is one VALU problem (<= 8 rows each); 0: MFMA problems: an
+                            // expert's rows go to big problems of 128 and the rest to small ones of <= 32
+    int shared_rows;        // 1: rows P .. P + T - 1 belong to an always-on expert with index E (token order)
+    int big_min;            // a remainder of at least this many rows becomes a (partial) big problem
+};
+
 struct RouteParams {
     const _Float16* x;      // [T][H]
     const _Float16* wr;     // [H][E]
@@ -41,6 +58,9 @@ struct RouteParams {
     float* w;               // [T][k]
     float* logits;          // [T][E] or null
     int T, H, E, k, nseg, renorm;
+    // one token only: the wave that selected the experts also sorts them and writes
+    // what the permute kernel would (sort.perm != nullptr), saving its launch
+    PermuteParams sort;
 };
 
 // Top-k of one token by one wave: lane holds the logits of experts lane + 64 i.
@@ -48,7 +68,7 @@ struct RouteParams {
 // over the selected k (renorm) or over all experts.
 constexpr int kRoutePer = kMaxExperts / 64;
 
-__device__ __forceinline__ void route_topk(const float (&lg)[kRoutePer], int lane, const RouteParams& p, int t)
+__device__ __forceinline__ int route_topk(const float (&lg)[kRoutePer], int lane, const RouteParams& p, int t)
 {
     constexpr int PER = kRoutePer;
     unsigned taken = 0;
@@ -93,6 +113,44 @@ __device__ __forceinline__ void route_topk(const float (&lg)[kRoutePer], int lan
         p.idx[(size_t)t * p.k + lane] = sel_idx;
         p.w[(size_t)t * p.k + lane] = ev / denom;
     }
+    return sel_idx;     // lane j < k: expert of slot j
+}
+
+// One token: what moe_permute_kernel writes, by the wave that holds the selection
+// (lane j < k has the expert of slot j; the k experts are distinct).  Sorted position
+// of slot j = number of selected experts with a smaller index; every expert is one
+// single-row VALU problem; an always-on expert (shared_rows) takes row k.
+__device__ __forceinline__ void route_sort_one_token(const PermuteParams& q, int lane, int sel_idx)
+{
+    const int k = q.k;
+    int rank = 0;
+    for (int j = 0; j < k; ++j) {
+        const int other = __shfl(sel_idx, j, 64);
+        rank += (lane < k && other < sel_idx) ? 1 : 0;
+    }
+    if (lane < k) {
+        q.perm[rank] = lane;
+        q.inv[lane] = rank;
+        q.row_expert[rank] = sel_idx;
+        q.vprob[rank] = GroupProblem{sel_idx, rank, 1, 0};
+    }
+    // offsets[e] = number of selected experts below e
+    for (int e0 = 0; e0 <= q.E; e0 += 64) {         // wave-uniform loop: every lane takes part in the exchanges
+        const int e = e0 + lane;
+        int below = 0;
+        for (int j = 0; j < k; ++j) below += (__shfl(sel_idx, j, 64) < e) ? 1 : 0;
+        if (e <= q.E) q.offsets[e] = below;
+    }
+    if (lane == 0) {
+        if (q.shared_rows) {
+            q.perm[k] = 0;
+            q.row_expert[k] = q.E;
+            q.vprob[k] = GroupProblem{q.E, k, 1, 0};
+        }
+        q.counts[0] = k + (q.shared_rows ? 1 : 0);
+        q.counts[1] = 0;
+        q.counts[2] = 0;
+    }
 }
 
 
@@ -118,10 +176,15 @@ __global__ __launch_bounds__(256) void moe_route_kernel(RouteParams p)
         float part[kRouteTT];
 #pragma unroll
         for (int tt = 0; tt < kRouteTT; ++tt) part[tt] = 0.0f;
-        for (int h = 0; h < hn; ++h) {
-            const float wv = (float)p.wr[(size_t)(h0 + h) * p.E + e];
+        // the whole segment of router rows in flight at once (rows past the segment
+        // re-read its last row and meet the zeros that pad xs); fma chains in row order
+        _Float16 wv[kRouteSeg];
 #pragma unroll
-            for (int tt = 0; tt < kRouteTT; ++tt) part[tt] = __builtin_fmaf(xs[tt][h], wv, part[tt]);
+        for (int i = 0; i < kRouteSeg; ++i) wv[i] = p.wr[(size_t)(h0 + min(i, hn - 1)) * p.E + e];
+#pragma unroll
+        for (int i = 0; i < kRouteSeg; ++i) {
+#pragma unroll
+            for (int tt = 0; tt < kRouteTT; ++tt) part[tt] = __builtin_fmaf(xs[tt][i], (float)wv[i], part[tt]);
         }
 #pragma unroll
         for (int tt = 0; tt < kRouteTT; ++tt)
@@ -153,24 +216,27 @@ __global__ __launch_bounds__(256) void moe_route_kernel(RouteParams p)
         if (e < p.E) {
             v = 0.0f;
             const float* src = p.parts + (size_t)t * p.nseg * p.E + e;
-            // eight loads in flight at a time; the adds stay in segment order
-            for (int s0 = 0; s0 < p.nseg; s0 += 8) {
-                float part[8];
+            // 32 loads in flight at a time (indices past the end re-read the last segment
+            // and are ignored); the adds stay in segment order
+            for (int s0 = 0; s0 < p.nseg; s0 += 32) {
+                float part[32];
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    part[j] = (s0 + j < p.nseg)
-                        ? __hip_atomic_load(src + (size_t)(s0 + j) * p.E, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                        : 0.0f;
+                for (int j = 0; j < 32; ++j)
+                    part[j] = __hip_atomic_load(src + (size_t)min(s0 + j, p.nseg - 1) * p.E, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    if (s0 + j < p.nseg) v += part[j];
+                for (int j = 0; j < 32; ++j) {
+                    const float nv = v + part[j];
+                    v = s0 + j < p.nseg ? nv : v;
+                }
             }
             if (p.bias) v += p.bias[e];
             if (p.logits) p.logits[(size_t)t * p.E + e] = v;
         }
         lg[i] = v;
     }
-    route_topk(lg, lane, p, t);
+    const int sel = route_topk(lg, lane, p, t);
+    if (p.sort.perm) route_sort_one_token(p.sort, lane, sel);
 }
 
 // Many tokens: the same arithmetic in two launches, so that the segment sums of a
@@ -316,22 +382,6 @@ __global__ __launch_bounds__(256) void moe_route_finish_kernel(RouteParams p)
 
 // ---------------------------------------------------------------- permute
 
-struct PermuteParams {
-    const int32_t* idx;     // [P] expert of each (token, slot) pair, P = T * k; distinct within a token
-    int32_t* offsets;       // [E + 1]
-    int32_t* perm;          // [R] sorted position -> pair (pair / k = token)
-    int32_t* inv;           // [P] pair -> sorted position
-    int32_t* row_expert;    // [R] sorted position -> expert
-    int32_t* counts;        // [3] number of VALU problems, small MFMA problems, big MFMA problems
-    GroupProblem* vprob;
-    GroupProblem* mprob;    // <= 32 rows each
-    GroupProblem* bprob;    // <= 128 rows each
-    int T, k, E;
-    int use_valu;           // 1: every expert is one VALU problem (<= 8 rows each); 0: MFMA problems: an
-                            // expert's rows go to big problems of 128 and the rest to small ones of <= 32
-    int shared_rows;        // 1: rows P .. P + T - 1 belong to an always-on expert with index E (token order)
-    int big_min;            // a remainder of at least this many rows becomes a (partial) big problem
-};
 
 // One workgroup.  Counting sort by expert, stable in pair order: the pairs of one
 // expert come from distinct tokens, so the rank of pair (t, slot) inside its expert
@@ -597,7 +647,7 @@ void check_route_shape(int T, int H, int E, int k)
 
 std::string run_route(const void* x, const void* wr, const float* bias, int32_t* idx, float* w,
                       float* logits, float* parts, int T, int H, int E, int k, int renorm,
-                      hipStream_t stream)
+                      hipStream_t stream, const PermuteParams* sort = nullptr)
 {
     Workspace& ws = workspace_for_current_device();
     RouteParams p{};
@@ -611,6 +661,7 @@ std::string run_route(const void* x, const void* wr, const float* bias, int32_t*
     p.logits = logits;
     p.T = T; p.H = H; p.E = E; p.k = k; p.renorm = renorm;
     p.nseg = (H + kRouteSeg - 1) / kRouteSeg;
+    if (sort && T == 1) p.sort = *sort;
     const int groups = (T + kRouteTT - 1) / kRouteTT;
     if (groups > kCounters) throw std::runtime_error("moe route: too many tokens for the counter table");
     if (T >= kRouteBigT) {
@@ -625,11 +676,11 @@ std::string run_route(const void* x, const void* wr, const float* bias, int32_t*
     dim3 grid(p.nseg, groups);
     hipLaunchKernelGGL(moe_route_kernel, grid, dim3(256), 0, stream, p);
     hip_ok(hipGetLastError(), "moe_route_kernel launch");
-    return "moe_route_kernel grid=" + std::to_string(grid.x) + "x" + std::to_string(grid.y);
+    return "moe_route_kernel grid=" + std::to_string(grid.x) + "x" + std::to_string(grid.y) +
+           (p.sort.perm ? " (with the sort of the one token)" : "");
 }
 
-std::string run_permute(const int32_t* idx, unsigned char* wsb, const MoeLayout& L, int T, int k, int E,
-                        bool fold, hipStream_t stream)
+PermuteParams permute_params(const int32_t* idx, unsigned char* wsb, const MoeLayout& L, int T, int k, int E, bool fold)
 {
     PermuteParams p{};
     p.idx = idx;
@@ -647,6 +698,11 @@ std::string run_permute(const int32_t* idx, unsigned char* wsb, const MoeLayout&
     p.use_valu = L.max_v > 0 ? 1 : 0;
     p.shared_rows = fold ? 1 : 0;
     p.big_min = L.max_b > 0 ? moe_big_min() : (1 << 30);
+    return p;
+}
+
+std::string run_permute(const PermuteParams& p, hipStream_t stream)
+{
     hipLaunchKernelGGL(moe_permute_kernel, dim3(1), dim3(1024), 0, stream, p);
     hip_ok(hipGetLastError(), "moe_permute_kernel launch");
     return "moe_permute_kernel";
@@ -772,8 +828,9 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
             if (!shared[i].trellis || !shared[i].suh || !shared[i].svh)
                 throw std::runtime_error("moe layer: null shared-expert pointer");
 
-    desc += run_route(x, wr, bias, idx, w, nullptr, (float*)(wsb + L.parts), T, H, E, k, renorm, stream);
-    desc += " + " + run_permute(idx, wsb, L, T, k, E, fold, stream);
+    const PermuteParams pp = permute_params(idx, wsb, L, T, k, E, fold);
+    desc += run_route(x, wr, bias, idx, w, nullptr, (float*)(wsb + L.parts), T, H, E, k, renorm, stream, &pp);
+    if (T > 1) desc += " + " + run_permute(pp, stream);
 
     GroupedArgs g{};
     g.experts = experts;

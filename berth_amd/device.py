@@ -30,7 +30,9 @@ class Gpu:
         self.sm_count = K.device_sms(device)
 
     def raw_stream(self):
-        return self.stream.cuda_stream or None
+        """The stream launches go on: torch's current stream of the device (the one
+        captured when a HIP graph is being recorded)."""
+        return torch.cuda.current_stream(self.device).cuda_stream or None
 
     def zeroed(self, nbytes: int) -> torch.Tensor:
         return torch.zeros(nbytes, dtype=torch.uint8, device=self.device)
