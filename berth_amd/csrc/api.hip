@@ -240,6 +240,70 @@ extern "C" int berth_exl3_unpack_signs(const void* packed, void* out, int64_t pa
     }
 }
 
+// validation order and messages of crates/berth-kernels/csrc/ops/norm.cu:108-125
+static void check_rms(const void* x, const void* weight, const void* y, const void* residual, int rows, int dim,
+                      int need_residual, int weight_bf16)
+{
+    if (!x || !weight || !y || (need_residual && !residual)) throw std::runtime_error("rms_norm: null device pointer");
+    if (rows < 1 || dim < 1) throw std::runtime_error("rms_norm: rows and dim must be positive");
+    if (dim % 4 != 0) throw std::runtime_error("rms_norm: dim must be a multiple of 4");
+    if (weight_bf16 != 0 && weight_bf16 != 1) throw std::runtime_error("rms_norm: weight_bf16 must be 0 or 1");
+}
+
+extern "C" int berth_ops_rms_norm(const void* x, const void* weight, void* y, int rows, int dim, float epsilon,
+                                  float constant_bias, float constant_scale, int weight_bf16, void* stream)
+{
+    try {
+        g_ops_err.clear();
+        g_ops_launch.clear();
+        check_rms(x, weight, y, nullptr, rows, dim, 0, weight_bf16);
+        g_ops_launch = launch_rms_norm(x, weight, y, nullptr, rows, dim, epsilon, constant_bias, constant_scale,
+                                       weight_bf16, (hipStream_t)stream);
+        return 0;
+    } catch (const std::exception& err) {
+        g_ops_err = err.what();
+        g_ops_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
+extern "C" int berth_ops_rms_norm_res_in(const void* x, const void* weight, void* y, void* residual, int rows, int dim,
+                                         float epsilon, float constant_bias, float constant_scale, int weight_bf16,
+                                         void* stream)
+{
+    try {
+        g_ops_err.clear();
+        g_ops_launch.clear();
+        check_rms(x, weight, y, residual, rows, dim, 1, weight_bf16);
+        g_ops_launch = launch_rms_norm(x, weight, y, residual, rows, dim, epsilon, constant_bias, constant_scale,
+                                       weight_bf16, (hipStream_t)stream);
+        return 0;
+    } catch (const std::exception& err) {
+        g_ops_err = err.what();
+        g_ops_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
+extern "C" int berth_ops_add_f32(const void* a, const void* b, void* c, int n, void* stream)
+{
+    try {
+        g_ops_err.clear();
+        g_ops_launch.clear();
+        if (!a || !b || !c) throw std::runtime_error("add_f32: null device pointer");
+        if (n < 1) throw std::runtime_error("add_f32: n must be positive");
+        g_ops_launch = launch_add_f32(a, b, c, n, (hipStream_t)stream);
+        return 0;
+    } catch (const std::exception& err) {
+        g_ops_err = err.what();
+        g_ops_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
 extern "C" int berth_ops_silu_mul(const void* gate, const void* up, void* out, int64_t numel,
                                   float act_limit, void* stream)
 {

@@ -93,6 +93,95 @@ std::string launch_silu_mul(const void* gate, const void* up, void* out, int64_t
     return "silu_mul_kernel block=256 grid=" + std::to_string(blocks);
 }
 
+// crates/berth-kernels/csrc/ops/add.cu: c = a + b in fp32 (the residual add after the MLP).
+__global__ __launch_bounds__(256) void add_f32_kernel(const float* a, const float* b, float* c, int n)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) c[i] = a[i] + b[i];
+}
+
+std::string launch_add_f32(const void* a, const void* b, void* c, int n, hipStream_t stream)
+{
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    hipLaunchKernelGGL(add_f32_kernel, dim3(blocks), dim3(256), 0, stream, (const float*)a, (const float*)b, (float*)c, n);
+    hip_ok(hipGetLastError(), "add_f32 launch");
+    return "add_f32 block=256 grid=" + std::to_string(blocks);
+}
+
+// RMS norm of fp32 rows to fp16, optionally with the fused residual
+// (crates/berth-kernels/src/ops.rs:398-500, csrc/ops/norm.cu): residual += x in
+// place (fp32), then y = fp16((v * rmf) * (w + constant_bias) * constant_scale),
+// rmf = fp32(1 / sqrt(mean(v^2) + epsilon)).  The mean is accumulated in double so
+// that it does not depend on the order of the reduction.  One workgroup per row.
+template <bool RES, bool WBF16>
+__global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__ x, const uint16_t* __restrict__ weight,
+                                                       _Float16* __restrict__ y, float* residual, int dim,
+                                                       float epsilon, float constant_bias, float constant_scale)
+{
+    __shared__ double s_part[4];
+    __shared__ float s_rmf;
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const float4_t* xr = (const float4_t*)(x + (size_t)row * dim);
+    float4_t* rr = RES ? (float4_t*)(residual + (size_t)row * dim) : nullptr;
+    double ss = 0.0;
+    for (int i = tid; i < dim / 4; i += 256) {
+        float4_t v = xr[i];
+        if (RES) {
+            const float4_t r = rr[i];
+            v = float4_t{r.x + v.x, r.y + v.y, r.z + v.z, r.w + v.w};
+            rr[i] = v;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ss += (double)v[j] * (double)v[j];
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) ss += __shfl_xor(ss, d, 64);
+    if ((tid & 63) == 0) s_part[tid >> 6] = ss;
+    __syncthreads();
+    if (tid == 0) {
+        const double total = ((s_part[0] + s_part[1]) + s_part[2]) + s_part[3];
+        s_rmf = (float)(1.0 / sqrt(total / dim + (double)epsilon));
+    }
+    __syncthreads();
+    const float rmf = s_rmf;
+    for (int i = tid; i < dim / 4; i += 256) {
+        const float4_t v = RES ? rr[i] : xr[i];     // RES: this thread wrote these four itself
+        half4_t o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint16_t wb = weight[4 * i + j];
+            const float w = WBF16 ? __builtin_bit_cast(float, (uint32_t)wb << 16)
+                                  : (float)__builtin_bit_cast(_Float16, wb);
+            float t = v[j] * rmf;
+            t = t * (w + constant_bias);
+            t = t * constant_scale;
+            o[j] = (_Float16)t;
+        }
+        *(half4_t*)(y + (size_t)row * dim + 4 * i) = o;
+    }
+}
+
+std::string launch_rms_norm(const void* x, const void* weight, void* y, void* residual, int rows, int dim,
+                            float epsilon, float constant_bias, float constant_scale, int weight_bf16,
+                            hipStream_t stream)
+{
+    const dim3 grid((unsigned)rows), block(256);
+    const float* xf = (const float*)x;
+    const uint16_t* w = (const uint16_t*)weight;
+    _Float16* yh = (_Float16*)y;
+    float* r = (float*)residual;
+    if (residual) {
+        if (weight_bf16) hipLaunchKernelGGL((rms_norm_kernel<true, true>), grid, block, 0, stream, xf, w, yh, r, dim, epsilon, constant_bias, constant_scale);
+        else hipLaunchKernelGGL((rms_norm_kernel<true, false>), grid, block, 0, stream, xf, w, yh, r, dim, epsilon, constant_bias, constant_scale);
+    } else {
+        if (weight_bf16) hipLaunchKernelGGL((rms_norm_kernel<false, true>), grid, block, 0, stream, xf, w, yh, r, dim, epsilon, constant_bias, constant_scale);
+        else hipLaunchKernelGGL((rms_norm_kernel<false, false>), grid, block, 0, stream, xf, w, yh, r, dim, epsilon, constant_bias, constant_scale);
+    }
+    hip_ok(hipGetLastError(), "rms_norm launch");
+    return std::string("rms_norm_kernel<") + (residual ? "2" : "0") + ",float,half," + (weight_bf16 ? "bfloat16" : "half") +
+           ",float> block=256 grid=" + std::to_string(rows);
+}
+
 // crates/berth-exl3/src/signs.rs:25-46: packed su / sv -> fp16 signs.  Little-endian
 // u16 words, bit i of a word is element i of its 16; a set bit is -1.0 (0xBC00),
 // a clear bit +1.0 (0x3C00).  One thread per output pair.

@@ -95,6 +95,10 @@ std::string launch_reconstruct(void* unpacked, const void* packed, int size_k, i
 // per row, per 128 columns: Hadamard with pre- or post-scale
 std::string launch_had_r_128(const void* in, void* out, const void* scale, int pre_scale,
                              int rows, int cols, int fp32, hipStream_t stream);
+std::string launch_add_f32(const void* a, const void* b, void* c, int n, hipStream_t stream);
+std::string launch_rms_norm(const void* x, const void* weight, void* y, void* residual, int rows, int dim,
+                            float epsilon, float constant_bias, float constant_scale, int weight_bf16,
+                            hipStream_t stream);
 std::string launch_unpack_signs(const void* packed, void* out, int64_t words, hipStream_t stream);
 std::string launch_silu_mul(const void* gate, const void* up, void* out, int64_t numel,
                             float act_limit, hipStream_t stream);

@@ -50,6 +50,9 @@ def load() -> C.CDLL:
         L.berth_prefill_reconstruct.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, vp]
         L.berth_prefill_had_r_128.argtypes = [vp, vp, vp, ci, ci, ci, ci, vp]
         L.berth_ops_silu_mul.argtypes = [vp, vp, vp, C.c_int64, C.c_float, vp]
+        L.berth_ops_rms_norm.argtypes = [vp, vp, vp, ci, ci, C.c_float, C.c_float, C.c_float, ci, vp]
+        L.berth_ops_rms_norm_res_in.argtypes = [vp, vp, vp, vp, ci, ci, C.c_float, C.c_float, C.c_float, ci, vp]
+        L.berth_ops_add_f32.argtypes = [vp, vp, vp, ci, vp]
         L.berth_exl3_unpack_signs.argtypes = [vp, vp, C.c_int64, vp]
         L.berth_exl3_unpack_signs.restype = C.c_int
         L.berth_ops_mgemm.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, vp, vp, vp, vp, ci, vp]
@@ -166,6 +169,31 @@ class ops:
         if rc > 0:
             return rc
         raise LaunchError(ops.last_error() or f"exl3_mgemm launch failed ({rc})")
+
+    @staticmethod
+    def rms_norm(x, weight, y, rows: int, dim: int, epsilon: float, constant_bias: float = 1.0,
+                 constant_scale: float = 1.0, weight_bf16: bool = True, stream=None) -> None:
+        """crates/berth-kernels/src/ops.rs:398-425."""
+        rc = load().berth_ops_rms_norm(x, weight, y, rows, dim, epsilon, constant_bias, constant_scale,
+                                       int(weight_bf16), stream)
+        if rc != 0:
+            raise LaunchError(ops.last_error() or f"rms_norm launch failed ({rc})")
+
+    @staticmethod
+    def rms_norm_res_in(x, weight, y, residual, rows: int, dim: int, epsilon: float, constant_bias: float = 1.0,
+                        constant_scale: float = 1.0, weight_bf16: bool = True, stream=None) -> None:
+        """crates/berth-kernels/src/ops.rs:452-486."""
+        rc = load().berth_ops_rms_norm_res_in(x, weight, y, residual, rows, dim, epsilon, constant_bias,
+                                              constant_scale, int(weight_bf16), stream)
+        if rc != 0:
+            raise LaunchError(ops.last_error() or f"rms_norm_res_in launch failed ({rc})")
+
+    @staticmethod
+    def add_f32(a, b, c, n: int, stream=None) -> None:
+        """crates/berth-kernels/src/ops.rs:540-552."""
+        rc = load().berth_ops_add_f32(a, b, c, n, stream)
+        if rc != 0:
+            raise LaunchError(ops.last_error() or f"add_f32 launch failed ({rc})")
 
     @staticmethod
     def silu_mul(gate, up, out, numel: int, act_limit: float = 0.0, stream=None) -> None:

@@ -89,6 +89,18 @@ int berth_exl3_unpack_signs(const void* packed, void* out, int64_t packed_bytes,
  * alias up. */
 int berth_ops_silu_mul(const void* gate, const void* up, void* out, int64_t numel,
                        float act_limit, void* stream);
+/* replaces crates/berth-kernels/src/ops.rs:55-80,398-500 / csrc/ops/norm.cu:128-225: RMS norm
+ * of fp32 rows to fp16, y = rms(x) * (weight + constant_bias) * constant_scale with rms =
+ * 1/sqrt(mean(x^2) + epsilon); weight fp16 (weight_bf16 0) or bf16 (1), dim a multiple of
+ * 4.  _res_in first adds x into the fp32 residual in place and normalises the sum. */
+int berth_ops_rms_norm(const void* x, const void* weight, void* y, int rows, int dim, float epsilon,
+                       float constant_bias, float constant_scale, int weight_bf16, void* stream);
+int berth_ops_rms_norm_res_in(const void* x, const void* weight, void* y, void* residual, int rows, int dim,
+                              float epsilon, float constant_bias, float constant_scale, int weight_bf16,
+                              void* stream);
+/* replaces crates/berth-kernels/src/ops.rs:91-97,522-552 / csrc/ops/add.cu: c = a + b, fp32,
+ * n elements; c may alias a. */
+int berth_ops_add_f32(const void* a, const void* b, void* c, int n, void* stream);
 /* replaces crates/berth-kernels/src/ops.rs:17-38,247-367 / csrc/ops/mgemm.cu:296-340:
  * several EXL3 linears in one launch.  Every list is a DEVICE array.  Sliced
  * mode (all four slice lists given, bszm_in == 1): bszm_out slices sharing the

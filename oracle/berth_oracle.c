@@ -598,3 +598,43 @@ void bo_set_num_threads(int n)
     (void)n;
 #endif
 }
+
+/* ---- glue ops around the MLP (crates/berth-kernels/src/ops.rs:398-552) ------------
+ * rms_norm: y[row] = fp16( (x * rmf) * (w + constant_bias) * constant_scale ), rmf =
+ * 1/sqrt(mean(x^2) + epsilon) rounded to fp32, products in fp32.  With `residual` the
+ * row is first residual += x (fp32, in place) and the norm runs on the sum.  weight
+ * is bf16 (weight_bf16 = 1) or fp16 bits. */
+static float bo_bf16_to_f32(uint16_t h)
+{
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+int bo_rms_norm(const float* x, const uint16_t* weight, uint16_t* y, float* residual, int rows, int dim,
+                float epsilon, float constant_bias, float constant_scale, int weight_bf16)
+{
+    if (!x || !weight || !y || rows < 1 || dim < 1 || dim % 4) return -1;
+    for (int r = 0; r < rows; ++r) {
+        const float* xr = x + (size_t)r * dim;
+        float* rr = residual ? residual + (size_t)r * dim : NULL;
+        double ss = 0.0;
+        for (int i = 0; i < dim; ++i) {
+            float v = xr[i];
+            if (rr) { v = rr[i] + v; rr[i] = v; }
+            ss += (double)v * (double)v;
+        }
+        const float rmf = (float)(1.0 / sqrt(ss / dim + (double)epsilon));
+        for (int i = 0; i < dim; ++i) {
+            const float v = rr ? rr[i] : xr[i];
+            const float w = weight_bf16 ? bo_bf16_to_f32(weight[i]) : bo_f16_to_f32(weight[i]);
+            float t = v * rmf;
+            t = t * (w + constant_bias);
+            t = t * constant_scale;
+            y[(size_t)r * dim + i] = bo_f64_to_f16((double)t);
+        }
+    }
+    return 0;
+}
+

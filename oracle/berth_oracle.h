@@ -146,6 +146,15 @@ int bo_moe_layer(const uint16_t* x, int T, int H, int E, int k, int I, int bits,
                  const bo_lin_t* experts, const bo_lin_t* shared, int shared_I,
                  float* out, int32_t* idx_out, float* w_out);
 
+/* RMS norm with an optional fused residual, crates/berth-kernels/src/ops.rs:398-500:
+ * residual (may be NULL) += x in fp32, then y = fp16((v * rmf) * (w + constant_bias) *
+ * constant_scale) with rmf = fp32(1/sqrt(mean(v^2) + epsilon)); weight bf16 or fp16 bits.
+ * Pinned by the reference's fixtures norm.x / norm_input.y / norm_final.y /
+ * norm_res.* (tests/golden): every output is reproduced bit for bit with the bf16
+ * weight recovered from the fixture itself, and r_out = r + x exactly. */
+int bo_rms_norm(const float* x, const uint16_t* weight, uint16_t* y, float* residual, int rows, int dim,
+                float epsilon, float constant_bias, float constant_scale, int weight_bf16);
+
 /* number of OpenMP threads the library will use */
 int bo_num_threads(void);
 void bo_set_num_threads(int n);

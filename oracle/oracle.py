@@ -45,6 +45,8 @@ def lib():
         L.bo_f16_to_f32.argtypes = [C.c_uint16]
         L.bo_unpack_signs.restype = C.c_long
         L.bo_silu_mul_f16.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_float]
+        L.bo_rms_norm.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float,
+                                  C.c_float, C.c_float, C.c_int]
         _lib = L
     return _lib
 
@@ -271,6 +273,21 @@ def moe_layer(x, wr, experts, k: int, I: int, bits: int, cb: int, bias=None, ren
     if rc:
         raise ValueError("bo_moe_layer failed")
     return out, idx, w
+
+
+def rms_norm(x, weight, epsilon, constant_bias=1.0, constant_scale=1.0, weight_bf16=True, residual=None):
+    """x fp32 [rows][dim]; weight: uint16 bit patterns (bf16 or fp16) [dim].  Returns
+    y fp16 [rows][dim] (and the updated residual when one is given)."""
+    x32 = np.ascontiguousarray(x, dtype=np.float32)
+    rows, dim = (1, x32.size) if x32.ndim == 1 else x32.shape
+    w16 = np.ascontiguousarray(weight).view(np.uint16)
+    y = np.empty((rows, dim), dtype=np.uint16)
+    res = None if residual is None else np.array(residual, dtype=np.float32).reshape(rows, dim).copy()
+    rc = lib().bo_rms_norm(_p(x32), _p(w16), _p(y), _p(res), rows, dim, C.c_float(epsilon), C.c_float(constant_bias),
+                           C.c_float(constant_scale), int(weight_bf16))
+    if rc:
+        raise ValueError("bo_rms_norm failed")
+    return (y.view(np.float16), res) if residual is not None else y.view(np.float16)
 
 
 def num_threads() -> int:

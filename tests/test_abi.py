@@ -106,6 +106,22 @@ def test_unpack_signs_validation():
     K.unpack_signs(None, None, 0)       # empty input: nothing to do
 
 
+def test_glue_op_validation():
+    # crates/berth-kernels/csrc/ops/norm.cu:108-125 and add.cu: refused before any device call
+    with pytest.raises(LaunchError, match="rms_norm: null"):
+        K.ops.rms_norm(None, P, P, 1, 128, 1e-6)
+    with pytest.raises(LaunchError, match="rms_norm: null"):
+        K.ops.rms_norm_res_in(P, P, P, None, 1, 128, 1e-6)
+    with pytest.raises(LaunchError, match="positive"):
+        K.ops.rms_norm(P, P, P, 0, 128, 1e-6)
+    with pytest.raises(LaunchError, match="multiple of 4"):
+        K.ops.rms_norm(P, P, P, 1, 130, 1e-6)
+    with pytest.raises(LaunchError, match="add_f32: null"):
+        K.ops.add_f32(P, None, P, 4)
+    with pytest.raises(LaunchError, match="n must be positive"):
+        K.ops.add_f32(P, P, P, 0)
+
+
 def test_mgemm_validation():
     with pytest.raises(LaunchError, match="null"):
         K.ops.exl3_mgemm(None, P, P, P, P, P, 1, 128, 128, 4, Codebook.MUL1, OutDtype.F16, 1, 2)
