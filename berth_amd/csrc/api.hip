@@ -7,6 +7,7 @@
 
 #include "../../include/berth_kernels_hip.h"
 
+#include <cstdlib>
 #include <mutex>
 
 namespace berth {
@@ -65,9 +66,20 @@ void check_shape(const char* who, const LinearArgs& a)
         throw std::runtime_error(w + ": size_k must be a multiple of 128 (one Hadamard block)");
 }
 
+// rows up to this count take the VALU kernel, more rows the MFMA kernel
+int gemv_max_rows()
+{
+    static const int v = [] {
+        const char* e = std::getenv("BERTH_GEMV_MAX_ROWS");
+        const int x = e ? std::atoi(e) : 8;
+        return x < 1 ? 1 : (x > 8 ? 8 : x);
+    }();
+    return v;
+}
+
 std::string dispatch_linear(const LinearArgs& a)
 {
-    if (a.size_m <= 8) return launch_gemv(a);
+    if (a.size_m <= gemv_max_rows()) return launch_gemv(a);
     return launch_gemm(a);
 }
 
