@@ -242,6 +242,48 @@ def bpw_sweep(gpu, rates, steps: int, nlayers: int = 8):
     return res
 
 
+def lm_head_bench(gpu, steps: int):
+    """The largest single GEMV of the 27B checkpoint: lm_head, K = 5120, N = 248320
+    at 6 bpw with the mul1 codebook and fp16 logits (trellis [320, 15520, 96],
+    953,548,800 bytes: crates/berth-exl3/tests/qwen38_27b.rs:66-76,
+    crates/berth-kernels/csrc/gemm_k6.cu:1-3).  Two device-generated copies are
+    alternated so that no launch finds its weights in a cache."""
+    import torch
+
+    from berth_amd import synth
+    from berth_amd.device import Exl3Linear
+    from berth_amd.kernels import OutDtype
+
+    K, N, bits = 5120, 248320, 6
+    g = torch.Generator(device=gpu.device)
+    g.manual_seed(606)
+    heads = []
+    for li in range(2):
+        tr = torch.randint(0, 65536, (K * N * bits // 16,), generator=g, device=gpu.device,
+                           dtype=torch.int32).to(torch.int16)
+        sc = [((torch.randint(0, 2, (n,), generator=g, device=gpu.device).float() * 2 - 1)
+               * torch.exp(0.1 * torch.randn(n, generator=g, device=gpu.device))).half() for n in (K, N)]
+        heads.append(Exl3Linear.from_device(f"lm_head.{li}", tr, sc[0], sc[1], bits))
+    x = gpu.upload(synth.activations(6, 1, K).view(np.uint16))
+    out = torch.zeros(N, dtype=torch.float16, device=gpu.device)
+    for i in range(4):
+        heads[i % 2].forward(gpu, x, out, OutDtype.F16)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(steps):
+        heads[i % 2].forward(gpu, x, out, OutDtype.F16)
+    e1.record()
+    torch.cuda.synchronize()
+    dt = e0.elapsed_time(e1) * 1e-3 / steps
+    nbytes = linear_bytes(K, N, bits, 1, 2)
+    from berth_amd import kernels as Kn
+    return {"config": "K 5120, N 248320, 6 bpw, mul1, batch 1, fp16 logits", "bytes": nbytes,
+            "us_per_launch": round(dt * 1e6, 1), "GBps": round(nbytes / dt / 1e9, 1),
+            "frac_of_hbm_peak": round(nbytes / dt / 1e9 / HBM_PEAK_GBS, 4),
+            "Gweights_per_s": round(K * N / dt / 1e9, 1), "kernel": Kn.last_launch()}
+
+
 def prefill_bench(gpu, layers, bits: int, rows: int, steps: int):
     """BASELINE.json configs[2]: the same 27B-shaped linears at `rows` = 512 tokens,
     fp16 activations N(0,1), fp16/fp32 outputs with fp32 accumulation, through
@@ -289,6 +331,7 @@ def main():
     ap.add_argument("--no-moe", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--no-lm-head", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only")
     ap.add_argument("--moe-resident-layers", type=int, default=48)
     ap.add_argument("--unfused", action="store_true", help="seven separate launches instead of four")
@@ -428,9 +471,13 @@ def main():
                                           "Gweights_per_s": round(340787200 / ms_per_step / 1e6, 1)}
     if not args.no_prefill:
         line["prefill_gemm"] = prefill_bench(gpu, layers, bits, 512, 10)
-    if not args.no_moe:
+    if not args.no_moe or not args.no_lm_head:
         del layers
         torch.cuda.empty_cache()
+    if not args.no_lm_head:
+        line["lm_head"] = lm_head_bench(gpu, 40)
+        torch.cuda.empty_cache()
+    if not args.no_moe:
         line["moe_layer"] = moe_bench(gpu, max(20, args.steps // 2), max(5, args.warmup // 2))
         torch.cuda.empty_cache()
         line["moe_large_layer"] = moe_large_bench(gpu, 96, args.moe_resident_layers)

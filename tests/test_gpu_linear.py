@@ -264,6 +264,28 @@ def test_full_size_gemv_round_trip_property():
     assert close(y1[256:512], want.reshape(-1))[0] == 0
 
 
+def test_lm_head_shape_6bpw_slices_match_oracle():
+    """The 27B lm_head (K 5120, N 248320, 6 bpw, mul1, fp16 logits: trellis
+    [320, 15520, 96], crates/berth-exl3/tests/qwen38_27b.rs:66-76) at full size;
+    three 256-column windows (first, middle, last) are checked against the oracle."""
+    Kk, N, bits = 5120, 248320, 6
+    tr, suh, svh = synth.linear(66, Kk, N, bits)
+    assert tr.shape == (320, 15520, 96) and tr.nbytes == 953_548_800
+    x = synth.activations(67, 1, Kk)
+    d_tr, d_suh, d_svh, d_x = dev(tr), dev(suh.view(np.uint16)), dev(svh.view(np.uint16)), dev(x.view(np.uint16))
+    a_had = torch.zeros(Kk, dtype=torch.float16, device=DEV)
+    c = torch.zeros(N, dtype=torch.float16, device=DEV)
+    K.exl3_linear(d_x.data_ptr(), d_tr.data_ptr(), c.data_ptr(), d_suh.data_ptr(), a_had.data_ptr(),
+                  d_svh.data_ptr(), 1, Kk, N, bits, Codebook.MUL1, OutDtype.F16)
+    torch.cuda.synchronize()
+    assert "exl3_gemv_kernel<6,2,1>" in K.last_launch()
+    got = host_f16(c)
+    for c0 in (0, 124160, N - 256):
+        sub = np.ascontiguousarray(tr[:, c0 // 16:c0 // 16 + 16, :])
+        want, _ = O.linear(x, sub, suh, svh[c0:c0 + 256], Kk, 256, bits, 2, out_fp32=False)
+        assert close(got[c0:c0 + 256], want.reshape(-1))[0] == 0, c0
+
+
 # ---- multi-linear (exl3_mgemm)
 @pytest.mark.parametrize("rows,fp32", [(1, False), (1, True), (3, False)])
 def test_mgemm_sliced_qkv_bundle(rows, fp32):
