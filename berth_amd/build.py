@@ -55,8 +55,20 @@ def build_all(jobs: int = 8, only: str | None = None) -> list[str]:
             raise RuntimeError(f"link failed for {name}:\n{r.stderr[-4000:]}")
         built.append(out)
     if only is None:
+        built.append(build_reader())
         built.append(build_host_check())
     return built
+
+
+def build_reader() -> str:
+    """The EXL3 checkpoint reader (csrc/host/exl3_reader_capi.cpp): host-only C++."""
+    out = os.path.join(LIB, "libberth_exl3_reader.so")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-shared", "-fPIC", "-Wall",
+           os.path.join(CSRC, "host", "exl3_reader_capi.cpp"), "-o", out]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"checkpoint reader build failed:\n{r.stderr[-4000:]}")
+    return out
 
 
 def build_host_check() -> str:

@@ -6,11 +6,14 @@
 // (device.rs:176-212), MlpLayer (crates/berth-engine/src/mlp.rs:25-334), and a
 // MoeLayer for the Ffn::Moe{router, shared, experts} of
 // crates/berth-plan/src/plan.rs:24-59 with every tensor resident in HBM.
+// Exl3Linear::load, MlpLayer::load and upload_tensor read an EXL3 checkpoint
+// directory through exl3_checkpoint.hpp (device.rs:49-125, mlp.rs:52-112).
 // Header-only; no torch, no HIP headers: everything goes through the C ABIs.
 #pragma once
 
 #include "../../../include/berth_hip.h"
 #include "../../../include/berth_kernels_hip.h"
+#include "exl3_checkpoint.hpp"
 
 #include <cstdint>
 #include <stdexcept>
@@ -23,6 +26,8 @@ namespace berth::engine {
 // crates/berth-engine: Error::Input (caller mistakes), Error::Kernel (launch refused), Error::Device
 struct InputError : std::invalid_argument { using std::invalid_argument::invalid_argument; };
 struct KernelError : std::runtime_error { using std::runtime_error::runtime_error; };
+// Error::Weights: a checkpoint whose tensors do not fit what the engine handles
+struct WeightsError : std::runtime_error { using std::runtime_error::runtime_error; };
 struct DeviceError : std::runtime_error {
     int code;
     DeviceError(int c, const std::string& what) : std::runtime_error(what), code(c) {}
@@ -137,6 +142,22 @@ private:
 
 using Half = uint16_t;      // fp16 bit patterns on the host
 
+// the checkpoint's EXL3 linear with this prefix (device.rs:167-173)
+inline const exl3::LinearExl3& find_linear(const exl3::Checkpoint& ckpt, const std::string& prefix)
+{
+    const exl3::LinearExl3* l = ckpt.find_linear(prefix);
+    if (!l) throw WeightsError(prefix + " is not an EXL3 linear");
+    return *l;
+}
+
+// one checkpoint tensor, as stored, copied to the device (device.rs:65-74)
+inline DeviceBuffer<uint8_t> upload_tensor(const Gpu& gpu, const exl3::Checkpoint& ckpt, const std::string& name)
+{
+    const exl3::TensorInfo* info = ckpt.tensors.get(name);
+    if (!info) throw WeightsError("tensor " + name + " is missing");
+    return DeviceBuffer<uint8_t>::from_host(gpu, exl3::read_tensor(*info));
+}
+
 // scratch shared by every linear of a prefill chunk (device.rs:176-212)
 struct RowScratch {
     RowScratch(const Gpu& gpu, int max_rows_, int max_k_, int max_n_)
@@ -168,6 +189,34 @@ public:
         a_had_ = DeviceBuffer<Half>::zeroed(gpu, (size_t)size_k);
     }
 
+    // <prefix>.trellis, .suh / .svh (or packed .su / .sv, expanded on the device) from a
+    // checkpoint (device.rs:92-125).  Half-integer rates are refused as in the reference;
+    // packed signs, which the reference refuses at this point, are accepted.
+    static Exl3Linear load(const Gpu& gpu, const exl3::Checkpoint& ckpt, const std::string& prefix)
+    {
+        const exl3::LinearExl3& linear = find_linear(ckpt, prefix);
+        if (linear.k.is_half()) throw WeightsError(prefix + ": half-integer rate");
+        Exl3Linear out;
+        out.prefix_ = prefix;
+        out.k_bits_ = linear.k.whole();
+        out.codebook_ = linear.codebook == exl3::Codebook::Mul1  ? Codebook::Mul1
+                        : linear.codebook == exl3::Codebook::Mcg ? Codebook::Mcg
+                                                                 : Codebook::Default;
+        out.suh_ = load_scale(gpu, linear.input_scale, &out.size_k_);
+        out.svh_ = load_scale(gpu, linear.output_scale, &out.size_n_);
+        const auto& shape = linear.trellis.shape;
+        if (out.size_k_ <= 0 || out.size_n_ <= 0 || shape[0] * 16 != (uint64_t)out.size_k_ ||
+            shape[1] * 16 != (uint64_t)out.size_n_)
+            throw WeightsError(prefix + ": trellis " + std::to_string(shape[0]) + "x" + std::to_string(shape[1]) +
+                               " tiles do not match " + std::to_string(out.size_k_) + " x " +
+                               std::to_string(out.size_n_) + " scales");
+        const std::vector<uint8_t> body = exl3::read_tensor(linear.trellis);
+        out.trellis_ = DeviceBuffer<uint16_t>::from_host(gpu, (const uint16_t*)body.data(), body.size() / 2);
+        out.a_had_ = DeviceBuffer<Half>::zeroed(gpu, (size_t)out.size_k_);
+        return out;
+    }
+
+    const std::string& prefix() const { return prefix_; }
     int size_k() const { return size_k_; }
     int size_n() const { return size_n_; }
     int k_bits() const { return k_bits_; }
@@ -219,9 +268,26 @@ public:
     }
 
 private:
+    Exl3Linear() = default;
+    // fp16 vector as stored, or packed sign words expanded to fp16 +-1 on the device
+    static DeviceBuffer<Half> load_scale(const Gpu& gpu, const exl3::HadamardScale& scale, int* channels)
+    {
+        const std::vector<uint8_t> body = exl3::read_tensor(scale.tensor);
+        if (!scale.packed) {
+            *channels = (int)(body.size() / 2);
+            return DeviceBuffer<Half>::from_host(gpu, (const Half*)body.data(), body.size() / 2);
+        }
+        *channels = (int)(body.size() * 8);
+        DeviceBuffer<uint8_t> packed = DeviceBuffer<uint8_t>::from_host(gpu, body);
+        DeviceBuffer<Half> out = DeviceBuffer<Half>::zeroed(gpu, body.size() * 8);
+        if (berth_exl3_unpack_signs(packed.raw(), out.raw(), (int64_t)body.size(), gpu.raw_stream()) != 0)
+            throw KernelError(berth_exl3_last_error());
+        gpu.synchronize();      // `packed` is released on return
+        return out;
+    }
     std::string prefix_;
-    int size_k_, size_n_, k_bits_ = 0;
-    Codebook codebook_;
+    int size_k_ = 0, size_n_ = 0, k_bits_ = 0;
+    Codebook codebook_ = Codebook::Mul1;
     DeviceBuffer<uint16_t> trellis_;
     DeviceBuffer<Half> suh_, svh_, a_had_;
 };
@@ -240,6 +306,32 @@ public:
         g_ = DeviceBuffer<Half>::zeroed(gpu, (size_t)max_rows * intermediate_);
         u_ = DeviceBuffer<Half>::zeroed(gpu, (size_t)max_rows * intermediate_);
     }
+    // layer `layer`'s MLP weights (mlp.rs:52-56)
+    static MlpLayer load(const Gpu& gpu, const exl3::Checkpoint& ckpt, uint32_t layer, int max_rows = 1)
+    {
+        return load_prefixed(gpu, ckpt, "model.language_model.layers." + std::to_string(layer) + ".mlp", max_rows);
+    }
+    // {prefix}.gate_proj, .up_proj and .down_proj (mlp.rs:58-112); a bias is refused because
+    // it would not be applied
+    static MlpLayer load_prefixed(const Gpu& gpu, const exl3::Checkpoint& ckpt, const std::string& prefix,
+                                  int max_rows = 1)
+    {
+        const std::string parts[3] = {prefix + ".gate_proj", prefix + ".up_proj", prefix + ".down_proj"};
+        for (const std::string& part : parts)
+            if (find_linear(ckpt, part).bias) throw WeightsError(part + ": bias is present and is not applied");
+        Exl3Linear gate = Exl3Linear::load(gpu, ckpt, parts[0]);
+        Exl3Linear up = Exl3Linear::load(gpu, ckpt, parts[1]);
+        Exl3Linear down = Exl3Linear::load(gpu, ckpt, parts[2]);
+        auto dims = [](const Exl3Linear& l) { return std::to_string(l.size_k()) + "x" + std::to_string(l.size_n()); };
+        if (gate.size_k() != up.size_k() || gate.size_n() != up.size_n())
+            throw WeightsError(prefix + ": gate is " + dims(gate) + ", up is " + dims(up));
+        if (down.size_k() != gate.size_n() || down.size_n() != gate.size_k())
+            throw WeightsError(prefix + ": down is " + dims(down) + ", gate is " + dims(gate));
+        if (gate.size_n() < 2 || gate.size_n() % 2 != 0)
+            throw WeightsError(prefix + ": intermediate " + std::to_string(gate.size_n()) + " must be positive and even");
+        return MlpLayer(gpu, std::move(gate), std::move(up), std::move(down), max_rows);
+    }
+
     int hidden() const { return hidden_; }
     int intermediate() const { return intermediate_; }
 

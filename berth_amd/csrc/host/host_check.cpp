@@ -3,6 +3,9 @@
 //   host_check linear <dir>   meta.txt: K N rows out_fp32 mode(0 forward/forward_n, 1 forward_rows)
 //   host_check mlp <dir>      meta.txt: hidden intermediate rows
 //   host_check moe <dir>      meta.txt: tokens hidden experts top_k intermediate shared(0/1) has_bias(0/1)
+//   host_check ckpt-info <checkpoint dir>                    (no device) lists the linears the reader found
+//   host_check ckpt-linear <checkpoint dir> <prefix> <dir>   Exl3Linear::load, one row of <dir>/x.bin, fp32 out
+//   host_check ckpt-mlp <checkpoint dir> <layer> <dir>       MlpLayer::load, one row of <dir>/x.bin
 // Tensors are raw little-endian files in <dir>; outputs go to <dir>/y.bin (+ idx.bin).
 #include "engine.hpp"
 
@@ -143,15 +146,58 @@ static int run_moe(const Gpu& gpu, const std::string& dir)
     return 0;
 }
 
+static int run_ckpt_info(const std::string& dir)
+{
+    const berth::exl3::Checkpoint ckpt = berth::exl3::Checkpoint::open(dir);
+    std::printf("arch=%s layers=%u hidden=%u tensors=%zu linears=%zu other=%zu\n", ckpt.config.arch_string.c_str(),
+                ckpt.config.num_hidden_layers, ckpt.config.hidden_size, ckpt.tensors.len(), ckpt.linears().size(),
+                ckpt.other_tensors().size());
+    for (const auto& l : ckpt.linears())
+        std::printf("linear %s k=%s codebook=%d packed=%d/%d bias=%d\n", l.prefix.c_str(), l.k.to_string().c_str(),
+                    (int)l.codebook, (int)l.input_scale.packed, (int)l.output_scale.packed, l.bias ? 1 : 0);
+    return 0;
+}
+
+static int run_ckpt_linear(const Gpu& gpu, const std::string& ckpt_dir, const std::string& prefix, const std::string& dir)
+{
+    const berth::exl3::Checkpoint ckpt = berth::exl3::Checkpoint::open(ckpt_dir);
+    Exl3Linear lin = Exl3Linear::load(gpu, ckpt, prefix);
+    const auto x = DeviceBuffer<Half>::from_host(gpu, read_file<Half>(dir + "/x.bin"));
+    auto y = DeviceBuffer<float>::zeroed(gpu, (size_t)lin.size_n());
+    lin.forward(gpu, x, y.ptr(), y.num_bytes(), OutDtype::F32);
+    gpu.synchronize();
+    write_file(dir + "/y.bin", y.copy_to_host());
+    std::printf("ckpt-linear ok %s K=%d N=%d bits=%d codebook=%d launch=%s\n", lin.prefix().c_str(), lin.size_k(),
+                lin.size_n(), lin.k_bits(), (int)lin.codebook(), berth_exl3_last_launch());
+    return 0;
+}
+
+static int run_ckpt_mlp(const Gpu& gpu, const std::string& ckpt_dir, uint32_t layer, const std::string& dir)
+{
+    const berth::exl3::Checkpoint ckpt = berth::exl3::Checkpoint::open(ckpt_dir);
+    MlpLayer mlp = MlpLayer::load(gpu, ckpt, layer);
+    const auto x = DeviceBuffer<Half>::from_host(gpu, read_file<Half>(dir + "/x.bin"));
+    auto y = DeviceBuffer<float>::zeroed(gpu, (size_t)mlp.hidden());
+    mlp.forward(gpu, x, y);
+    gpu.synchronize();
+    write_file(dir + "/y.bin", y.copy_to_host());
+    std::printf("ckpt-mlp ok layer=%u hidden=%d intermediate=%d\n", layer, mlp.hidden(), mlp.intermediate());
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
     if (argc < 3) {
-        std::fprintf(stderr, "usage: host_check linear|mlp|moe <dir>\n");
+        std::fprintf(stderr, "usage: host_check linear|mlp|moe <dir> | ckpt-info <ckpt> | ckpt-linear <ckpt> <prefix> <dir> "
+                             "| ckpt-mlp <ckpt> <layer> <dir>\n");
         return 2;
     }
     try {
-        Gpu gpu(0);
         const std::string what = argv[1], dir = argv[2];
+        if (what == "ckpt-info") return run_ckpt_info(dir);
+        Gpu gpu(0);
+        if (what == "ckpt-linear" && argc >= 5) return run_ckpt_linear(gpu, dir, argv[3], argv[4]);
+        if (what == "ckpt-mlp" && argc >= 5) return run_ckpt_mlp(gpu, dir, (uint32_t)std::stoul(argv[3]), argv[4]);
         if (what == "linear") return run_linear(gpu, dir);
         if (what == "mlp") return run_mlp(gpu, dir);
         if (what == "moe") return run_moe(gpu, dir);

@@ -1,6 +1,7 @@
 """Host-side owners of device buffers for the EXL3 linear path, mirroring
 crates/berth-engine/src/device.rs:14-367 (`Gpu`, `Exl3Linear`, `RowScratch`) and
-crates/berth-engine/src/mlp.rs:25-334 (`MlpLayer`).  torch is used for device
+crates/berth-engine/src/mlp.rs:25-334 (`MlpLayer`); `load` constructors read an
+EXL3 checkpoint directory through `berth_amd.exl3`.  torch is used for device
 memory and the stream only; every computation goes through the C ABI.
 """
 from __future__ import annotations
@@ -16,6 +17,18 @@ MAX_RECONSTRUCT_N = 32768   # crates/berth-engine/src/device.rs:193
 
 class InputError(ValueError):
     """crates/berth-engine `Error::Input`."""
+
+
+class WeightsError(ValueError):
+    """crates/berth-engine `Error::Weights`: a checkpoint the engine does not handle."""
+
+
+def find_linear(ckpt, prefix: str):
+    """The checkpoint's EXL3 linear with this prefix (device.rs:167-173)."""
+    for lin in ckpt.linears():
+        if lin.prefix == prefix:
+            return lin
+    raise WeightsError(f"{prefix} is not an EXL3 linear")
 
 
 class Gpu:
@@ -118,6 +131,34 @@ class Exl3Linear:
         gpu.synchronize()
         return cls.from_device(prefix, gpu.upload(trellis.view(np.uint16)).reshape(-1), halves[0], halves[1],
                                trellis.shape[2] // 16, codebook)
+
+    @classmethod
+    def load(cls, gpu: Gpu, ckpt, prefix: str) -> "Exl3Linear":
+        """`<prefix>.trellis`, `.suh` / `.svh` (or packed `.su` / `.sv`, expanded on the
+        device) from a `berth_amd.exl3.Checkpoint` (device.rs:92-125).  Half-integer
+        rates are refused as in the reference; packed signs, which the reference
+        refuses at this point, are accepted."""
+        linear = find_linear(ckpt, prefix)
+        if linear.k.is_half():
+            raise WeightsError(f"{prefix}: half-integer rate")
+        halves = []
+        for scale in (linear.input_scale, linear.output_scale):
+            raw = scale.tensor.read_array(np.uint8).ravel()
+            if scale.is_packed():
+                d_raw = torch.from_numpy(raw).to(gpu.device)
+                out = torch.zeros(raw.size * 8, dtype=torch.float16, device=gpu.device)
+                K.unpack_signs(ptr(d_raw), ptr(out), raw.size, gpu.raw_stream())
+                gpu.synchronize()
+            else:
+                out = gpu.upload(raw.view(np.uint16))
+            halves.append(out)
+        tiles_k, tiles_n, _ = linear.trellis.shape
+        if tiles_k * 16 != halves[0].numel() or tiles_n * 16 != halves[1].numel():
+            raise WeightsError(f"{prefix}: trellis {tiles_k}x{tiles_n} tiles do not match "
+                               f"{halves[0].numel()} x {halves[1].numel()} scales")
+        trellis = gpu.upload(linear.trellis.read_array(np.uint16).ravel())
+        return cls.from_device(prefix, trellis, halves[0], halves[1], linear.k.twice // 2,
+                               Codebook(linear.kernel_codebook))
 
     def trellis_bytes(self) -> int:
         return self.trellis.numel() * 2
@@ -235,6 +276,28 @@ class MlpLayer:
             raise InputError("mlp: projection shapes do not chain")
         self.g = torch.zeros(max_rows * self.intermediate, dtype=torch.float16, device=gpu.device)
         self.u = torch.zeros(max_rows * self.intermediate, dtype=torch.float16, device=gpu.device)
+
+    @classmethod
+    def load(cls, gpu: Gpu, ckpt, layer: int, max_rows: int = 1) -> "MlpLayer":
+        """Layer `layer`'s MLP weights (mlp.rs:52-56)."""
+        return cls.load_prefixed(gpu, ckpt, f"model.language_model.layers.{layer}.mlp", max_rows)
+
+    @classmethod
+    def load_prefixed(cls, gpu: Gpu, ckpt, prefix: str, max_rows: int = 1) -> "MlpLayer":
+        """`{prefix}.gate_proj`, `.up_proj`, `.down_proj` (mlp.rs:58-112); a bias is refused
+        because it would not be applied."""
+        parts = [f"{prefix}.gate_proj", f"{prefix}.up_proj", f"{prefix}.down_proj"]
+        for part in parts:
+            if find_linear(ckpt, part).bias is not None:
+                raise WeightsError(f"{part}: bias is present and is not applied")
+        gate, up, down = (Exl3Linear.load(gpu, ckpt, part) for part in parts)
+        if (gate.size_k, gate.size_n) != (up.size_k, up.size_n):
+            raise WeightsError(f"{prefix}: gate is {gate.size_k}x{gate.size_n}, up is {up.size_k}x{up.size_n}")
+        if (down.size_k, down.size_n) != (gate.size_n, gate.size_k):
+            raise WeightsError(f"{prefix}: down is {down.size_k}x{down.size_n}, gate is {gate.size_k}x{gate.size_n}")
+        if gate.size_n < 2 or gate.size_n % 2:
+            raise WeightsError(f"{prefix}: intermediate {gate.size_n} must be positive and even")
+        return cls(gpu, gate, up, down, max_rows)
 
     def forward(self, gpu: Gpu, x: torch.Tensor, y: torch.Tensor) -> None:
         """x fp16 [hidden] -> y fp32 [hidden]."""

@@ -38,6 +38,14 @@ def test_runtime_library_exports_every_declared_symbol():
         assert getattr(lib, name) is not None, name
 
 
+def test_reader_library_exports_every_declared_symbol():
+    lib = C.CDLL(os.path.join(ROOT, "berth_amd", "lib", "libberth_exl3_reader.so"))
+    names = _declared("berth_exl3_reader.h")
+    assert "berth_ckpt_open" in names and len(names) >= 20
+    for name in names:
+        assert getattr(lib, name) is not None, name
+
+
 def test_linear_null_and_bad_sizes_do_not_touch_the_device():
     with pytest.raises(LaunchError, match="null"):
         K.exl3_linear(None, None, None, None, None, None, 1, 128, 256, 4, Codebook.MUL1, OutDtype.F16)
