@@ -284,6 +284,38 @@ def lm_head_bench(gpu, steps: int):
             "Gweights_per_s": round(K * N / dt / 1e9, 1), "kernel": Kn.last_launch()}
 
 
+def mlp_block_bench(gpu, layers, bits: int, steps: int):
+    """One dense MLP block of the 27B shapes (hidden 5120, intermediate 17408) for one
+    token: berth_exl3_mlp (gate and up in one launch, SiLU gating inside the down
+    projection: two launches) beside the reference's four calls
+    (crates/berth-engine/src/mlp.rs:118-150), rotating over the resident layers."""
+    import torch
+
+    from berth_amd import synth
+    from berth_amd.device import MlpLayer
+
+    H, I = synth.SHAPES_27B["gate_proj"]
+    mlps = [MlpLayer(gpu, lin["gate_proj"], lin["up_proj"], lin["down_proj"]) for lin in layers]
+    x = gpu.upload((synth.activations(11, 1, H).astype(np.float32) / np.sqrt(H)).astype(np.float16).view(np.uint16))
+    y = torch.zeros(H, dtype=torch.float32, device=gpu.device)
+    nbytes = 2 * linear_bytes(H, I, bits, 1, 2) + linear_bytes(I, H, bits, 1, 4)
+    res = {"config": f"hidden {H}, intermediate {I}, {bits} bpw, mul1, batch 1", "bytes": nbytes}
+    for name, fused in (("one_call", True), ("four_calls", False)):
+        for i in range(len(mlps)):
+            mlps[i].forward(gpu, x, y, fused=fused)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(steps):
+            mlps[i % len(mlps)].forward(gpu, x, y, fused=fused)
+        e1.record()
+        torch.cuda.synchronize()
+        dt = e0.elapsed_time(e1) * 1e-3 / steps
+        res[name] = {"us_per_block": round(dt * 1e6, 2), "GBps": round(nbytes / dt / 1e9, 1),
+                     "frac_of_hbm_peak": round(nbytes / dt / 1e9 / HBM_PEAK_GBS, 4)}
+    return res
+
+
 def prefill_bench(gpu, layers, bits: int, rows: int, steps: int):
     """BASELINE.json configs[2]: the same 27B-shaped linears at `rows` = 512 tokens,
     fp16 activations N(0,1), fp16/fp32 outputs with fp32 accumulation, through
@@ -332,6 +364,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-lm-head", action="store_true")
+    ap.add_argument("--no-mlp", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only")
     ap.add_argument("--moe-resident-layers", type=int, default=48)
     ap.add_argument("--unfused", action="store_true", help="seven separate launches instead of four")
@@ -469,6 +502,8 @@ def main():
         line["bpw_sweep"][f"{bits}bpw"] = {"GBps": line["value"], "us_per_step": round(ms_per_step * 1e3, 2),
                                           "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
                                           "Gweights_per_s": round(340787200 / ms_per_step / 1e6, 1)}
+    if not args.no_mlp:
+        line["mlp_block"] = mlp_block_bench(gpu, layers, bits, args.steps)
     if not args.no_prefill:
         line["prefill_gemm"] = prefill_bench(gpu, layers, bits, 512, 10)
     if not args.no_moe or not args.no_lm_head:

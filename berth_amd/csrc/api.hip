@@ -232,6 +232,52 @@ extern "C" int berth_prefill_had_r_128(const void* input, void* output, const vo
 extern "C" const char* berth_prefill_last_error(void) { return g_prefill_err.c_str(); }
 extern "C" const char* berth_prefill_last_launch(void) { return g_prefill_launch.c_str(); }
 
+extern "C" int berth_exl3_mlp(const void* x, const berth_exl3_lin* lins, void* gate_out, void* up_out, void* a_had,
+                              void* act_had, void* y, int size_m, int hidden, int intermediate, int k_bits,
+                              int codebook, void* stream)
+{
+    try {
+        g_exl3_err.clear();
+        g_exl3_launch.clear();
+        if (!x || !lins || !gate_out || !up_out || !a_had || !act_had || !y)
+            throw std::runtime_error("exl3 mlp: null device pointer");
+        for (int i = 0; i < 3; ++i)
+            if (!lins[i].trellis || !lins[i].suh || !lins[i].svh) throw std::runtime_error("exl3 mlp: null device pointer");
+        if (size_m < 1 || hidden < 1 || intermediate < 1) throw std::runtime_error("exl3 mlp: sizes must be positive");
+        hipStream_t st = (hipStream_t)stream;
+        LinearArgs down{up_out, lins[2].trellis, y, lins[2].suh, act_had, lins[2].svh, size_m, intermediate, hidden,
+                        k_bits, codebook, 1, st};
+        LinearArgs gate{x, lins[0].trellis, gate_out, lins[0].suh, a_had, lins[0].svh, size_m, hidden, intermediate,
+                        k_bits, codebook, 0, st};
+        check_shape("exl3 mlp", gate);
+        check_shape("exl3 mlp", down);
+        if (size_m <= 8) {
+            PairArgs pair{x, {lins[0].trellis, lins[1].trellis}, {lins[0].suh, lins[1].suh}, {lins[0].svh, lins[1].svh},
+                          {gate_out, up_out}, a_had, size_m, hidden, intermediate, k_bits, codebook, st};
+            std::string desc = launch_gemv_pair(pair);
+            down.a = gate_out;
+            down.a_up = up_out;
+            g_exl3_launch = desc + " ; " + launch_gemv(down);
+            return 0;
+        }
+        LinearArgs up = gate;
+        up.trellis = lins[1].trellis;
+        up.suh = lins[1].suh;
+        up.svh = lins[1].svh;
+        up.c = up_out;
+        std::string desc = launch_gemm(gate);
+        desc += " ; " + launch_gemm(up);
+        desc += " ; " + launch_silu_mul(gate_out, up_out, up_out, (int64_t)size_m * intermediate, 0.0f, st);
+        g_exl3_launch = desc + " ; " + launch_gemm(down);
+        return 0;
+    } catch (const std::exception& err) {
+        g_exl3_err = err.what();
+        g_exl3_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
 extern "C" int berth_exl3_unpack_signs(const void* packed, void* out, int64_t packed_bytes, void* stream)
 {
     try {

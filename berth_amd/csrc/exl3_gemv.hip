@@ -73,6 +73,7 @@ std::string launch_gemv(const LinearArgs& a)
     p.lin.trellis = (const uint32_t*)a.trellis;
     p.lin.suh = (const _Float16*)a.suh;
     p.lin.svh = (const _Float16*)a.svh;
+    p.a_up = (const _Float16*)a.a_up;
     p.rows = a.size_m;
     p.c[0] = a.c;
     p.a_had = (_Float16*)a.a_had;
@@ -89,8 +90,44 @@ std::string launch_gemv(const LinearArgs& a)
     launch_bits(p, a.k_bits, a.codebook, mmax, dim3(grid), a.stream);
     hip_ok(hipGetLastError(), "exl3_gemv_kernel launch");
     return "exl3_gemv_kernel<" + std::to_string(a.k_bits) + "," + std::to_string(a.codebook) + "," +
-           std::to_string(mmax) + "> grid=" + std::to_string(grid) + " block=256 split_k=" +
+           std::to_string(mmax) + (a.a_up ? ",silu" : "") + "> grid=" + std::to_string(grid) + " block=256 split_k=" +
            std::to_string(p.S) + (a.out_fp32 ? " out=f32" : " out=f16");
+}
+
+std::string launch_gemv_pair(const PairArgs& a)
+{
+    if (a.size_m < 1 || a.size_m > 8) throw std::runtime_error("exl3 gemv: rows must be in 1..=8");
+    if (a.size_k % 128 != 0) throw std::runtime_error("exl3 linear: size_k must be a multiple of 128");
+    Workspace& ws = workspace_for_current_device();
+    const int mmax = a.size_m == 1 ? 1 : 8;
+    GemvParams p{};
+    p.a = (const _Float16*)a.a;
+    p.pair = 1;
+    for (int i = 0; i < 2; ++i) {
+        p.shared[i].trellis = (const uint32_t*)a.trellis[i];
+        p.shared[i].suh = (const _Float16*)a.suh[i];
+        p.shared[i].svh = (const _Float16*)a.svh[i];
+        p.c[i] = a.c[i];
+    }
+    p.shared_expert = -1;
+    p.rows = a.size_m;
+    p.a_had = (_Float16*)a.a_had;
+    p.partials = ws.partials;
+    p.counters = ws.counters;
+    p.K = a.size_k;
+    p.N = a.size_n;
+    p.NB = a.size_n / 128;
+    p.KB = a.size_k / 128;
+    p.out_fp32 = 0;
+    const long units = 2L * p.NB;
+    if (units > kCounters) throw std::runtime_error("exl3 gemv: size_n exceeds the split-K counter table");
+    p.S = pick_split(ws, units, p.KB, mmax);
+    dim3 grid((unsigned)(p.NB * p.S), 2);
+    launch_bits(p, a.k_bits, a.codebook, mmax, grid, a.stream);
+    hip_ok(hipGetLastError(), "exl3_gemv_kernel pair launch");
+    return "exl3_gemv_kernel<" + std::to_string(a.k_bits) + "," + std::to_string(a.codebook) + "," +
+           std::to_string(mmax) + "> pair grid=" + std::to_string(grid.x) + "x2 block=256 split_k=" +
+           std::to_string(p.S) + " out=f16";
 }
 
 std::string launch_mgemm(const MgemmArgs& m)

@@ -59,6 +59,7 @@ struct GemvParams {
     int lin_base;
     ExpertLin shared[3];        // an always-on expert passed by value (problem.expert == shared_expert)
     int shared_expert;
+    int pair;                   // dense mode with gridDim.y == 2: linear shared[blockIdx.y] on the same rows
     // multi-linear mode (multi != 0), the argument lists of
     // crates/berth-kernels/src/ops.rs:264-293, all device arrays: one problem per
     // entry of b_list; multi == 2 is the sliced form (per-slice width, row stride
@@ -244,7 +245,7 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
     const int s = local / p.NB;
     const int which = blockIdx.y;
 
-    ExpertLin lin = p.lin;
+    ExpertLin lin = p.pair ? p.shared[which] : p.lin;
     int row0 = 0, rows = p.rows;
     if (p.problems) {
         if (prob >= *p.num_problems) return;
@@ -303,7 +304,7 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
         w.kb0 = s * 4 + wave;
         w.step = wc;
         w.rows = rows;
-        if (p.a_had && nb == 0) gemv_accumulate<BITS, CB, MMAX, SILU, true>(w, src, xs[wave], acc);
+        if (p.a_had && nb == 0 && which == 0) gemv_accumulate<BITS, CB, MMAX, SILU, true>(w, src, xs[wave], acc);
         else gemv_accumulate<BITS, CB, MMAX, SILU, false>(w, src, xs[wave], acc);
     }
 

@@ -305,6 +305,11 @@ public:
             throw InputError("mlp: projection shapes do not chain");
         g_ = DeviceBuffer<Half>::zeroed(gpu, (size_t)max_rows * intermediate_);
         u_ = DeviceBuffer<Half>::zeroed(gpu, (size_t)max_rows * intermediate_);
+        x_had_ = DeviceBuffer<Half>::zeroed(gpu, (size_t)max_rows * hidden_);
+        act_had_ = DeviceBuffer<Half>::zeroed(gpu, (size_t)max_rows * intermediate_);
+        // the one-call path takes one bit rate and codebook for the three linears
+        uniform_ = gate_.k_bits() == up_.k_bits() && gate_.k_bits() == down_.k_bits() &&
+                   gate_.codebook() == up_.codebook() && gate_.codebook() == down_.codebook();
     }
     // layer `layer`'s MLP weights (mlp.rs:52-56)
     static MlpLayer load(const Gpu& gpu, const exl3::Checkpoint& ckpt, uint32_t layer, int max_rows = 1)
@@ -335,9 +340,23 @@ public:
     int hidden() const { return hidden_; }
     int intermediate() const { return intermediate_; }
 
-    // x fp16 [hidden] -> y fp32 [hidden]
+    // x fp16 [rows][hidden] -> y fp32 [rows][hidden] through berth_exl3_mlp: gate and up in one
+    // launch, silu(g) * u evaluated inside the down projection (two launches up to 8 rows)
+    void forward_fused(const Gpu& gpu, const DeviceBuffer<Half>& x, DeviceBuffer<float>& y, int rows = 1) const
+    {
+        if (!uniform_) throw InputError("mlp: the one-call path needs one bit rate and codebook");
+        if (rows < 1 || rows > max_rows_) throw InputError("mlp: rows exceed the layer scratch");
+        if (x.len() < (size_t)rows * hidden_ || y.len() < (size_t)rows * hidden_)
+            throw InputError(gate_.prefix() + ": buffer too small");
+        const berth_exl3_lin lins[3] = {gate_.table_entry(), up_.table_entry(), down_.table_entry()};
+        if (berth_exl3_mlp(x.raw(), lins, g_.raw(), u_.raw(), x_had_.raw(), act_had_.raw(), y.raw(), rows, hidden_,
+                           intermediate_, gate_.k_bits(), (int)gate_.codebook(), gpu.raw_stream()) != 0)
+            throw KernelError(berth_exl3_last_error());
+    }
+    // x fp16 [hidden] -> y fp32 [hidden], the reference's four calls (mlp.rs:118-150)
     void forward(const Gpu& gpu, const DeviceBuffer<Half>& x, DeviceBuffer<float>& y) const
     {
+        if (x.len() < (size_t)hidden_ || y.len() < (size_t)hidden_) throw InputError(gate_.prefix() + ": buffer too small");
         gate_.forward(gpu, x, g_.ptr(), g_.num_bytes(), OutDtype::F16);
         up_.forward(gpu, x, u_.ptr(), u_.num_bytes(), OutDtype::F16);
         silu(gpu, intermediate_);
@@ -363,7 +382,8 @@ private:
     }
     Exl3Linear gate_, up_, down_;
     int hidden_ = 0, intermediate_ = 0, max_rows_;
-    DeviceBuffer<Half> g_, u_;
+    bool uniform_ = false;
+    DeviceBuffer<Half> g_, u_, x_had_, act_had_;
 };
 
 // router + E routed experts of three linears + optional always-on shared expert

@@ -1,7 +1,7 @@
 // Runs the C++ host layer (engine.hpp) on case files written by the test suite and
 // writes the results back, so that the tests can compare them with the CPU oracle:
 //   host_check linear <dir>   meta.txt: K N rows out_fp32 mode(0 forward/forward_n, 1 forward_rows)
-//   host_check mlp <dir>      meta.txt: hidden intermediate rows
+//   host_check mlp <dir>      meta.txt: hidden intermediate rows [fused(0/1)]
 //   host_check moe <dir>      meta.txt: tokens hidden experts top_k intermediate shared(0/1) has_bias(0/1)
 //   host_check ckpt-info <checkpoint dir>                    (no device) lists the linears the reader found
 //   host_check ckpt-linear <checkpoint dir> <prefix> <dir>   Exl3Linear::load, one row of <dir>/x.bin, fp32 out
@@ -105,7 +105,10 @@ static int run_mlp(const Gpu& gpu, const std::string& dir)
                  load_linear(gpu, dir, "down", I, H), rows);
     const auto x = DeviceBuffer<Half>::from_host(gpu, read_file<Half>(dir + "/x.bin"));
     auto y = DeviceBuffer<float>::zeroed(gpu, (size_t)rows * H);
-    if (rows == 1) {
+    const bool fused = m.size() > 3 && m[3] != 0;
+    if (fused) {
+        mlp.forward_fused(gpu, x, y, rows);
+    } else if (rows == 1) {
         mlp.forward(gpu, x, y);
     } else {
         RowScratch scratch(gpu, rows, H > I ? H : I, H > I ? H : I);
@@ -113,7 +116,7 @@ static int run_mlp(const Gpu& gpu, const std::string& dir)
     }
     gpu.synchronize();
     write_file(dir + "/y.bin", y.copy_to_host());
-    std::printf("mlp ok rows=%d\n", rows);
+    std::printf("mlp ok rows=%d fused=%d launch=%s\n", rows, fused ? 1 : 0, fused ? berth_exl3_last_launch() : "");
     return 0;
 }
 

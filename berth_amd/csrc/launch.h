@@ -38,7 +38,21 @@ struct LinearArgs {
     const void* svh;
     int size_m, size_k, size_n, k_bits, codebook, out_fp32;
     hipStream_t stream;
+    const void* a_up = nullptr;   // VALU kernel only: the input is silu(a) * a_up, element by element
 };
+
+// two linears of one shape on the same input rows in one launch (gate and up of an MLP)
+struct PairArgs {
+    const void* a;
+    const void* trellis[2];
+    const void* suh[2];
+    const void* svh[2];
+    void* c[2];                 // fp16 [size_m][size_n] each
+    void* a_had;                // [size_m][size_k]
+    int size_m, size_k, size_n, k_bits, codebook;
+    hipStream_t stream;
+};
+std::string launch_gemv_pair(const PairArgs& args);
 
 // grouped (MoE) launches: problems, experts and num_problems are device memory
 struct GroupedArgs {

@@ -276,6 +276,9 @@ class MlpLayer:
             raise InputError("mlp: projection shapes do not chain")
         self.g = torch.zeros(max_rows * self.intermediate, dtype=torch.float16, device=gpu.device)
         self.u = torch.zeros(max_rows * self.intermediate, dtype=torch.float16, device=gpu.device)
+        self.x_had = self.act_had = None      # rotated inputs of the fused call, allocated on first use
+        # the one-call path takes one bit rate and codebook for the three linears
+        self.uniform = gate.k_bits == up.k_bits == down.k_bits and gate.codebook == up.codebook == down.codebook
 
     @classmethod
     def load(cls, gpu: Gpu, ckpt, layer: int, max_rows: int = 1) -> "MlpLayer":
@@ -299,8 +302,20 @@ class MlpLayer:
             raise WeightsError(f"{prefix}: intermediate {gate.size_n} must be positive and even")
         return cls(gpu, gate, up, down, max_rows)
 
-    def forward(self, gpu: Gpu, x: torch.Tensor, y: torch.Tensor) -> None:
-        """x fp16 [hidden] -> y fp32 [hidden]."""
+    def forward(self, gpu: Gpu, x: torch.Tensor, y: torch.Tensor, fused: bool = True, rows: int = 1) -> None:
+        """x fp16 [rows][hidden] -> y fp32 [rows][hidden].  fused: one `berth_exl3_mlp` call (two
+        launches up to 8 rows); otherwise the reference's four calls for one row (mlp.rs:118-150)."""
+        if fused and self.uniform:
+            if rows * self.intermediate > self.g.numel() or x.numel() < rows * self.hidden or \
+               y.numel() < rows * self.hidden:
+                raise InputError(f"{self.gate.prefix}: buffer too small")
+            if self.x_had is None or self.x_had.numel() < rows * self.hidden:
+                self.x_had = torch.zeros(rows * self.hidden, dtype=torch.float16, device=x.device)
+                self.act_had = torch.zeros(self.g.numel(), dtype=torch.float16, device=x.device)
+            lins = [(ptr(l.trellis), ptr(l.suh), ptr(l.svh)) for l in (self.gate, self.up, self.down)]
+            K.exl3_mlp(ptr(x), lins, ptr(self.g), ptr(self.u), ptr(self.x_had), ptr(self.act_had), ptr(y), rows,
+                       self.hidden, self.intermediate, self.gate.k_bits, self.gate.codebook, gpu.raw_stream())
+            return
         self.gate.forward(gpu, x, self.g, OutDtype.F16)
         self.up.forward(gpu, x, self.u, OutDtype.F16)
         K.ops.silu_mul(ptr(self.g), ptr(self.u), ptr(self.u), self.intermediate, 0.0, gpu.raw_stream())

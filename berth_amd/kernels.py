@@ -54,6 +54,7 @@ def load() -> C.CDLL:
         L.berth_ops_rms_norm_res_in.argtypes = [vp, vp, vp, vp, ci, ci, C.c_float, C.c_float, C.c_float, ci, vp]
         L.berth_ops_add_f32.argtypes = [vp, vp, vp, ci, vp]
         L.berth_exl3_unpack_signs.argtypes = [vp, vp, C.c_int64, vp]
+        L.berth_exl3_mlp.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         L.berth_exl3_unpack_signs.restype = C.c_int
         L.berth_ops_mgemm.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, vp, vp, vp, vp, ci, vp]
         for name in ("berth_exl3_last_error", "berth_exl3_last_launch", "berth_prefill_last_error",
@@ -88,6 +89,22 @@ def exl3_linear(a, trellis, c, suh, a_had, svh, size_m, size_k, size_n, k_bits,
                              int(codebook), int(out), stream)
     if rc != 0:
         raise LaunchError(last_error() or f"exl3 linear launch failed ({rc})")
+
+
+class Exl3Lin(C.Structure):
+    """`berth_exl3_lin`: device addresses of one linear's trellis, suh and svh."""
+    _fields_ = [("trellis", C.c_void_p), ("suh", C.c_void_p), ("svh", C.c_void_p)]
+
+
+def exl3_mlp(x, lins, gate_out, up_out, a_had, act_had, y, size_m, hidden, intermediate, k_bits,
+             codebook: Codebook, stream=None) -> None:
+    """y = down(silu(gate(x)) * up(x)): the four calls of crates/berth-engine/src/mlp.rs:118-150
+    in one entry (two launches up to 8 rows).  lins: three (trellis, suh, svh) address triples."""
+    table = (Exl3Lin * 3)(*[Exl3Lin(*t) for t in lins])
+    rc = load().berth_exl3_mlp(x, table, gate_out, up_out, a_had, act_had, y, size_m, hidden, intermediate, k_bits,
+                               int(codebook), stream)
+    if rc != 0:
+        raise LaunchError(last_error() or f"exl3 mlp launch failed ({rc})")
 
 
 def unpack_signs(packed, out, packed_bytes: int, stream=None) -> None:

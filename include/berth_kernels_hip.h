@@ -142,6 +142,25 @@ typedef struct {
     const void* svh;        /* fp16 [N] */
 } berth_exl3_lin;
 
+/* ---- one dense MLP block ----------------------------------------------------
+ * y = down(silu(gate(x)) * up(x)), the four calls of MlpLayer::forward
+ * (crates/berth-engine/src/mlp.rs:118-150: two berth_exl3_linear with fp16
+ * output, berth_ops_silu_mul with act_limit 0, berth_exl3_linear with fp32
+ * output) in one entry.  Up to 8 rows run as two launches: gate and up share one
+ * launch and the rotated input, and the down projection evaluates silu(g) * u
+ * while it rotates its input (same fp16 steps as berth_ops_silu_mul, so the
+ * activation is bit-identical to the unfused sequence).  More rows run the
+ * unfused sequence on the MFMA kernel.
+ * lins: HOST array {gate, up, down} of device pointers.  x fp16 [m][hidden];
+ * gate_out, up_out fp16 [m][intermediate] (written; above 8 rows up_out ends up
+ * holding the activation); a_had fp16 [m][hidden] and act_had fp16
+ * [m][intermediate] (written: the rotated inputs); y fp32 [m][hidden].
+ * hidden % 128 == 0, intermediate % 128 == 0.  Errors and launch text go to
+ * berth_exl3_last_error / berth_exl3_last_launch. */
+int berth_exl3_mlp(const void* x, const berth_exl3_lin* lins, void* gate_out, void* up_out,
+                   void* a_had, void* act_had, void* y, int size_m, int hidden, int intermediate,
+                   int k_bits, int codebook, void* stream);
+
 /* x fp16 [T][H]; wr fp16 [H][E] (the unquantised router, mlp.gate.weight laid out
  * input-major); bias fp32 [E] or NULL; idx int32 [T][k]; w fp32 [T][k]; logits fp32
  * [T][E] or NULL; parts_scratch fp32 [T][ceil(H/64)][E]. */

@@ -139,3 +139,19 @@ def test_mgemm_validation():
         K.ops.exl3_mgemm(P, P, P, P, P, P, 1, 128, 128, 4, Codebook.MUL1, OutDtype.F16, 2, 2, P, P, P, P, 1)
     with pytest.raises(LaunchError, match="num_had_src requires"):
         K.ops.exl3_mgemm(P, P, P, P, P, P, 1, 128, 128, 4, Codebook.MUL1, OutDtype.F16, 1, 2, num_had_src=1)
+
+
+def test_fused_mlp_validation():
+    P = 0x1000
+    lins = [(P, P, P)] * 3
+    with pytest.raises(LaunchError, match="null"):
+        K.exl3_mlp(None, lins, P, P, P, P, P, 1, 256, 384, 4, Codebook.MUL1)
+    with pytest.raises(LaunchError, match="null"):
+        K.exl3_mlp(P, [(P, P, P), (P, None, P), (P, P, P)], P, P, P, P, P, 1, 256, 384, 4, Codebook.MUL1)
+    with pytest.raises(LaunchError, match="positive"):
+        K.exl3_mlp(P, lins, P, P, P, P, P, 0, 256, 384, 4, Codebook.MUL1)
+    with pytest.raises(LaunchError, match="multiple of 128"):
+        K.exl3_mlp(P, lins, P, P, P, P, P, 1, 256, 200, 4, Codebook.MUL1)
+    with pytest.raises(LaunchError, match="1..=8"):
+        K.exl3_mlp(P, lins, P, P, P, P, P, 1, 256, 384, 9, Codebook.MUL1)
+    assert K.last_launch() == ""

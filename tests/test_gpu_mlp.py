@@ -1,0 +1,96 @@
+"""The dense MLP block in one call (berth_exl3_mlp: gate and up in one launch, SiLU
+gating inside the down projection) against the CPU oracle, stage by stage, and
+against the reference's four-call sequence (crates/berth-engine/src/mlp.rs:118-150)."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+import torch
+
+from berth_amd import kernels as K
+from berth_amd import synth
+from berth_amd.device import Exl3Linear, Gpu, MlpLayer
+from oracle import oracle as O
+from tests.gpu_util import close, host_f16, host_u16
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EXE = os.path.join(ROOT, "berth_amd", "lib", "berth_host_check")
+
+
+def _layer(gpu, H, I, bits, seed, rows):
+    lins = [synth.linear(seed, H, I, bits), synth.linear(seed + 3, H, I, bits), synth.linear(seed + 6, I, H, bits)]
+    mlp = MlpLayer(gpu, *(Exl3Linear(gpu, n, *l) for n, l in zip(("gate", "up", "down"), lins)), max_rows=rows)
+    return lins, mlp
+
+
+@pytest.mark.parametrize("rows,H,I,bits", [(1, 256, 384, 4), (3, 256, 384, 3), (8, 256, 384, 4), (1, 1024, 2816, 4),
+                                           (2, 2048, 768, 2), (20, 256, 384, 4), (40, 512, 256, 5)])
+def test_fused_mlp_stage_by_stage(rows, H, I, bits):
+    gpu = Gpu(0)
+    (gate, up, down), mlp = _layer(gpu, H, I, bits, 9000 + rows, rows)
+    x = (synth.activations(9100 + rows, rows, H).astype(np.float32) / np.sqrt(H)).astype(np.float16)
+    y = torch.zeros((rows, H), dtype=torch.float32, device=gpu.device)
+    mlp.forward(gpu, gpu.upload(x.view(np.uint16)), y, rows=rows)
+    gpu.synchronize()
+    launch = K.last_launch()
+    if rows <= 8:
+        assert launch.count("exl3_gemv_kernel") == 2 and "pair" in launch and ",silu>" in launch
+    else:
+        assert launch.count("exl3_gemm_kernel") == 3 and "silu_mul" in launch
+
+    g_want, xh_want = O.linear(x, *gate, H, I, bits, 2)
+    u_want, _ = O.linear(x, *up, H, I, bits, 2)
+    g_got = host_f16(mlp.g)[:rows * I].reshape(rows, I)
+    assert close(g_got, g_want.reshape(rows, I))[0] == 0
+    if rows <= 8:
+        # the rotated input is the gate's (its suh); above 8 rows the up projection rewrites it with its own
+        assert np.array_equal(host_u16(mlp.x_had)[:rows * H], xh_want.view(np.uint16).ravel())
+        u_got = host_f16(mlp.u)[:rows * I].reshape(rows, I)
+        assert close(u_got, u_want.reshape(rows, I))[0] == 0
+        act = O.silu_mul(g_got, u_got).reshape(rows, I)            # from the GPU's own gate / up outputs
+        # the activation the down projection formed, seen through its rotated copy: bit-exact
+        assert np.array_equal(host_u16(mlp.act_had)[:rows * I],
+                              O.had_rows_f16(act, down[1], True).view(np.uint16).ravel())
+    else:
+        act = host_f16(mlp.u)[:rows * I].reshape(rows, I)          # up_out holds the activation
+        assert close(act, O.silu_mul(g_want, u_want).reshape(rows, I), rtol=4e-3, atol=2e-3)[0] == 0
+    y_want, _ = O.linear(act, *down, I, H, bits, 2, out_fp32=True)
+    assert close(y.cpu().numpy(), y_want.reshape(rows, H))[0] == 0
+
+
+def test_fused_mlp_equals_the_four_call_sequence_up_to_summation_order():
+    gpu = Gpu(0)
+    H, I = 1024, 2816
+    _, mlp = _layer(gpu, H, I, 4, 9500, 1)
+    x = (synth.activations(9501, 1, H).astype(np.float32) / np.sqrt(H)).astype(np.float16)
+    dx = gpu.upload(x.view(np.uint16))
+    y_fused = torch.zeros(H, dtype=torch.float32, device=gpu.device)
+    y_calls = torch.zeros(H, dtype=torch.float32, device=gpu.device)
+    mlp.forward(gpu, dx, y_fused)
+    mlp.forward(gpu, dx, y_calls, fused=False)
+    gpu.synchronize()
+    a, b = y_fused.cpu().numpy(), y_calls.cpu().numpy()
+    assert np.abs(a - b).max() <= 2e-3 * np.abs(b).max()
+
+
+@pytest.mark.parametrize("rows", [1, 5])
+def test_cpp_mlp_forward_fused(tmp_path, rows):
+    H, I, bits = 256, 384, 3
+    trio = dict(gate=synth.linear(5000, H, I, bits), up=synth.linear(5003, H, I, bits), down=synth.linear(5006, I, H, bits))
+    x = (synth.activations(5100 + rows, rows, H).astype(np.float32) / np.sqrt(H)).astype(np.float16)
+    for name, (tr, suh, svh) in trio.items():
+        tr.tofile(tmp_path / f"{name}.trellis.bin")
+        suh.view(np.uint16).tofile(tmp_path / f"{name}.suh.bin")
+        svh.view(np.uint16).tofile(tmp_path / f"{name}.svh.bin")
+    x.view(np.uint16).tofile(tmp_path / "x.bin")
+    (tmp_path / "meta.txt").write_text(f"{H} {I} {rows} 1\n")
+    r = subprocess.run([EXE, "mlp", str(tmp_path)], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "fused=1" in r.stdout and "pair" in r.stdout, r.stdout + r.stderr
+    y = np.fromfile(tmp_path / "y.bin", dtype=np.float32).reshape(rows, H)
+    g, _ = O.linear(x, *trio["gate"], H, I, bits, 2)
+    u, _ = O.linear(x, *trio["up"], H, I, bits, 2)
+    want, _ = O.linear(O.silu_mul(g, u).reshape(rows, I), *trio["down"], I, H, bits, 2, out_fp32=True)
+    assert np.abs(y - want.reshape(rows, H)).max() <= 2e-3 * np.abs(want).max()
