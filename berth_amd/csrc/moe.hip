@@ -955,10 +955,22 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
             LinearArgs la{a, lin.trellis, c, lin.suh, wsb + L.s_ahad, lin.svh, T, kk, nn, k_bits, codebook, fp32, stream};
             return T <= 8 ? launch_gemv(la) : launch_gemm(la);
         };
-        dense(x, shared[0], wsb + L.sg, H, shared_I, 0);
-        dense(x, shared[1], wsb + L.su, H, shared_I, 0);
-        launch_silu_mul(wsb + L.sg, wsb + L.su, wsb + L.su, (int64_t)T * shared_I, 0.0f, stream);
-        dense(wsb + L.su, shared[2], wsb + L.shared_out, shared_I, H, 1);
+        if (T <= 8) {
+            // gate and up in one launch, silu(g) * u formed inside the down projection
+            PairArgs pa{x, {shared[0].trellis, shared[1].trellis}, {shared[0].suh, shared[1].suh},
+                        {shared[0].svh, shared[1].svh}, {wsb + L.sg, wsb + L.su}, wsb + L.s_ahad, T, H, shared_I,
+                        k_bits, codebook, stream};
+            launch_gemv_pair(pa);
+            LinearArgs down{wsb + L.sg, shared[2].trellis, wsb + L.shared_out, shared[2].suh, wsb + L.s_ahad,
+                            shared[2].svh, T, shared_I, H, k_bits, codebook, 1, stream};
+            down.a_up = wsb + L.su;
+            launch_gemv(down);
+        } else {
+            dense(x, shared[0], wsb + L.sg, H, shared_I, 0);
+            dense(x, shared[1], wsb + L.su, H, shared_I, 0);
+            launch_silu_mul(wsb + L.sg, wsb + L.su, wsb + L.su, (int64_t)T * shared_I, 0.0f, stream);
+            dense(wsb + L.su, shared[2], wsb + L.shared_out, shared_I, H, 1);
+        }
         shared_out = (const float*)(wsb + L.shared_out);
         desc += " + shared expert";
     }
