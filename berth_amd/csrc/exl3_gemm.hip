@@ -9,6 +9,8 @@
 
 namespace berth {
 
+static_assert(kGemmWrittenBase * 2 == kCounters, "the GEMM keeps two counters per tile");
+
 // one translation unit per codebook (exl3_gemm_cb{0,1,2}.hip) keeps the build parallel
 void launch_gemm_cb0(const GemmParams& p, int bits, int mb, hipStream_t stream, std::string& desc, dim3 grid);
 void launch_gemm_cb1(const GemmParams& p, int bits, int mb, hipStream_t stream, std::string& desc, dim3 grid);
@@ -23,21 +25,22 @@ static void gemm_bits(const GemmParams& p, int bits, int cb, int mb, hipStream_t
     }
 }
 
-// split-K factor for `tiles` output tiles of MB*32 x 256: fill the chip about twice,
-// keep at least two k-blocks per workgroup, stay inside the workspace
+// split-K factor for `tiles` output tiles of MB*32 x 256: one workgroup per compute unit
+// (a second resident workgroup adds nothing once the whole chip is busy, and fewer
+// workgroups share a tile), at least two k-blocks per workgroup, inside the workspace
 static int gemm_split(const Workspace& ws, long tiles, int KB, int mb)
 {
     static const int per_cu = [] {
         const char* e = std::getenv("BERTH_GEMM_WG_PER_CU");
         int v = e ? std::atoi(e) : 0;
-        return v > 0 ? v : 2;
+        return v > 0 ? v : 1;
     }();
     long S = ((long)ws.cu_count * per_cu + tiles - 1) / tiles;
     if (S > KB / 2) S = KB / 2;
     if (S < 1) S = 1;
     const size_t per_wg = (size_t)4 * mb * 2 * 16 * 64 * sizeof(float);
     while (S > 1 && (size_t)tiles * S * per_wg > kPartialBytes) --S;
-    if (tiles > kCounters) S = 1;
+    if (tiles > kCounters / 2) S = 1;          // two counters per tile
     return (int)S;
 }
 
@@ -68,8 +71,33 @@ std::string launch_gemm(const LinearArgs& a)
     p.tiles_y = mtiles;
     std::string desc;
     p.tile0 = 0;
-    p.S = gemm_split(ws, tiles, KB, mb);
-    gemm_bits(p, a.k_bits, a.codebook, mb, a.stream, desc, dim3((unsigned)(tiles * p.S), 1, 1));
+    static const int balance = [] {
+        const char* e = std::getenv("BERTH_GEMM_BALANCED");
+        return e ? std::atoi(e) : 1;
+    }();
+    // 128-row tiles rarely divide over the compute units (272 tiles on 256 units leave most of
+    // the chip idle for the second half of the launch): deal the (tile, k-block) units out evenly
+    const long units = tiles * KB;
+    // one workgroup per compute unit, two when a workgroup still gets 16 k-blocks or more
+    // (measured on the 27B shapes at 512 rows: gate/up and down are fastest with two, q and o
+    // with one, where fewer workgroups share a tile)
+    long slots = units >= 32L * ws.cu_count ? 2L * ws.cu_count : ws.cu_count;
+    if (balance > 1) slots = balance;
+    const long G = units < slots ? units : slots;
+    const long per_wg = units / G;                                   // >= 1
+    const long parts = (KB + per_wg - 1) / per_wg + 1;               // workgroups that can share a tile
+    const size_t part_bytes = (size_t)4 * mb * 2 * 16 * 64 * sizeof(float);
+    if (balance && mb == 4 && tiles <= kCounters / 2 && per_wg < KB && units < (1L << 30) && (size_t)tiles * parts * part_bytes <= kPartialBytes) {
+        p.S = 1;
+        p.units = (int)units;
+        p.unit_q = (int)(units / G);
+        p.unit_r = (int)(units % G);
+        p.max_parts = (int)parts;
+        gemm_bits(p, a.k_bits, a.codebook, mb, a.stream, desc, dim3((unsigned)G, 1, 1));
+    } else {
+        p.S = gemm_split(ws, tiles, KB, mb);
+        gemm_bits(p, a.k_bits, a.codebook, mb, a.stream, desc, dim3((unsigned)(tiles * p.S), 1, 1));
+    }
     hip_ok(hipGetLastError(), "exl3_gemm_kernel launch");
     return d0 + " + " + desc + (a.out_fp32 ? " out=f32" : " out=f16");
 }

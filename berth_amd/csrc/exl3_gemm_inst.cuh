@@ -1,6 +1,6 @@
 // Per-codebook instantiations of the MFMA GEMM kernel (included by
 // exl3_gemm_cb{0,1,2}.hip with BERTH_GEMM_CB defined): 32-row and 128-row tiles for
-// every bit rate.
+// every bit rate, and the balanced variant of the 128-row kernel.
 #include "exl3_gemm_kernel.cuh"
 #include "launch.h"
 
@@ -17,6 +17,20 @@ static void gemm_launch_mb(const GemmParams& p, hipStream_t stream, std::string&
         static const hipError_t attr = hipFuncSetAttribute((const void*)exl3_gemm_kernel<BITS, CB, MB>,
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         hip_ok(attr, "exl3_gemm_kernel shared-memory attribute");
+    }
+    if (p.units > 0) {
+        // balanced dense launch (128-row tiles only): two workgroups per compute unit
+        if constexpr (MB == 4) {
+            static const hipError_t attr2 = hipFuncSetAttribute((const void*)exl3_gemm_balanced_kernel<BITS, CB, MB>,
+                                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            hip_ok(attr2, "exl3_gemm_balanced_kernel shared-memory attribute");
+            hipLaunchKernelGGL((exl3_gemm_balanced_kernel<BITS, CB, MB>), grid, dim3(256), smem, stream, p);
+            desc = "exl3_gemm_balanced_kernel<" + std::to_string(BITS) + "," + std::to_string(CB) + "," +
+                   std::to_string(BM) + "x256> grid=" + std::to_string(grid.x) + " units=" + std::to_string(p.units) +
+                   " max_parts=" + std::to_string(p.max_parts) + " smem=" + std::to_string(smem);
+            return;
+        }
+        throw std::runtime_error("exl3 gemm: balanced launches use 128-row tiles");
     }
     hipLaunchKernelGGL((exl3_gemm_kernel<BITS, CB, MB>), grid, dim3(256), smem, stream, p);
     desc = "exl3_gemm_kernel<" + std::to_string(BITS) + "," + std::to_string(CB) + "," + std::to_string(BM) +

@@ -20,9 +20,10 @@
 // tile in LDS for the output Hadamard.
 //
 // K can be split over S workgroups (few rows, or few columns: not enough tiles to
-// fill the chip).  Partial accumulators go to the library workspace in register
-// layout; the last workgroup to arrive (self-resetting counter) adds them in split
-// order and runs the epilogue, so the result does not depend on timing.
+// fill the chip).  The last workgroup to arrive at a tile (self-resetting counters)
+// finishes it: the others leave their partial accumulators in the library workspace
+// in register layout, and the finisher adds all parts in k order, so the result does
+// not depend on timing.
 #pragma once
 
 #include "exl3_gemv_kernel.cuh"
@@ -48,13 +49,29 @@ struct GemmParams {
     int S;
     float* partials;            // [unit][S][4 waves][MB][2][16][64]
     unsigned* counters;         // [unit]
+    // balanced dense launches (exl3_gemm_balanced_kernel): the launch's (tile, k-block) units,
+    // tile-major, are dealt out evenly to gridDim.x workgroups
+    int units;                  // tiles * K/128; 0: not a balanced launch
+    int unit_q, unit_r;         // units = unit_q * gridDim.x + unit_r
+    int max_parts;              // upper bound of workgroups that share one tile
 };
+
+// the k-blocks of one tile that a workgroup accumulates, and its place among the
+// workgroups that share the tile
+struct KRange {
+    int kb0, kb1, step;         // k-blocks kb0, kb0 + step, ... < kb1
+    int part, parts;            // this workgroup's position (k order) and the number of sharers
+    size_t slot0;               // first partial-sum slot of the tile
+    size_t counter;             // arrival counter of the tile
+};
+
+constexpr int kGemmWrittenBase = 32768;   // second half of the counter table: "partial sums written" per tile
 
 constexpr int kAStride = 128 + 8;   // halves per LDS row of the A tile (272 B: conflict-free b128 reads)
 
 // one output tile: rows of problem / row block `tile_y`, 256 columns
-template <int BITS, int CB, int MB>  // MB = 32-row blocks per workgroup
-__device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y, const int nblk, const int split,
+template <int BITS, int CB, int MB, bool DENSE>  // MB = 32-row blocks per workgroup; DENSE: never a problem list
+__device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y, const int nblk, const KRange kr,
                                           const int which, unsigned char* smem)
 {
     constexpr int BM = MB * 32;
@@ -71,16 +88,20 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
     int m0 = tile_y * BM;
     int m_end = p.M;
     ExpertLin lin = p.lin;
-    if (p.problems) {
+    const _Float16* a_had = p.a_had[0];
+    void* cout = p.c[0];
+    if constexpr (!DENSE) {
+        // (dynamic indexing of the parameter block: kept out of the dense instantiations, where
+        // it would force the whole block into private memory)
         const GroupProblem gp = p.problems[tile_y];
         lin = gp.expert == p.shared_expert ? p.shared[p.lin_base + which]
                                            : p.experts[gp.expert * p.lins_per_expert + p.lin_base + which];
         m0 = gp.row0;
         m_end = gp.row0 + gp.nrows;
+        a_had = p.a_had[which];
+        cout = p.c[which];
     }
     const int rows_here = min(BM, m_end - m0);          // >= 1
-    const _Float16* a_had = p.a_had[which];
-    void* cout = p.c[which];
     const int nw = n0 + wave * 64;                      // first column of this wave
     const bool active = nw < p.N;
     const int tn = p.N >> 4;
@@ -103,7 +124,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
         // reloaded for the wave's next k-block as soon as a step has consumed them
         // (rolling prefetch, one k-block ahead); on the last k-block the reload reads
         // the same addresses again and is ignored, which keeps the loop free of branches.
-        if (active && split < KB) {
+        if (active && kr.kb0 < kr.kb1) {
             const global_ptr<const uint32_t> tb = as_global(lin.trellis) + (size_t)half_id * row_dw +
                                                  (size_t)((nw >> 4) + (slot >> 3)) * tile_dw + (slot & 7) * BITS;
             const int arow = m0 + min(slot, rows_here - 1);         // rows past the problem repeat its last row
@@ -112,8 +133,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
             uint32_t cur[4][BITS];
             half8_t av[4][2];
             {
-                const global_ptr<const uint32_t> t0 = tb + (size_t)(split * 8) * row_dw;
-                const global_ptr<const half8_t> a0 = ab + split * 16;
+                const global_ptr<const uint32_t> t0 = tb + (size_t)(kr.kb0 * 8) * row_dw;
+                const global_ptr<const half8_t> a0 = ab + kr.kb0 * 16;
 #pragma unroll
                 for (int st = 0; st < 4; ++st) {
                     load_tile_dwords<BITS>(t0 + (size_t)(2 * st) * row_dw, cur[st]);
@@ -122,8 +143,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
-            for (int kb = split; kb < KB; kb += p.S) {
-                const int nkb = kb + p.S < KB ? kb + p.S : kb;
+            for (int kb = kr.kb0; kb < kr.kb1; kb += kr.step) {
+                const int nkb = kb + kr.step < kr.kb1 ? kb + kr.step : kb;
                 const global_ptr<const uint32_t> tnx = tb + (size_t)(nkb * 8) * row_dw;
                 const global_ptr<const half8_t> anx = ab + nkb * 16;
 #pragma unroll
@@ -185,13 +206,13 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
     #pragma unroll
                 for (int j = 0; j < BITS; ++j) nxt[st][j] = nb[(size_t)(2 * st) * row_dw + j];
         };
-        if (split < KB) {
-            load_a(split);
-            if (active) load_b(split);
+        if (kr.kb0 < kr.kb1) {
+            load_a(kr.kb0);
+            if (active) load_b(kr.kb0);
         }
 
         int buf = 0;
-        for (int kb = split; kb < KB; kb += p.S, buf ^= 1) {
+        for (int kb = kr.kb0; kb < kr.kb1; kb += kr.step, buf ^= 1) {
             uint32_t cur[4][BITS];
     #pragma unroll
             for (int st = 0; st < 4; ++st)
@@ -206,9 +227,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
                 dst[0] = a_nxt[ps][0];
                 dst[1] = a_nxt[ps][1];
             }
-            if (kb + p.S < KB) {
-                load_a(kb + p.S);
-                if (active) load_b(kb + p.S);
+            if (kb + kr.step < kr.kb1) {
+                load_a(kb + kr.step);
+                if (active) load_b(kb + kr.step);
             }
             __syncthreads();
 
@@ -246,66 +267,90 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
 
     // ---- split-K handoff.  Register r of a lane holds tile row 8*(r/4) + 4*half_id + r%4,
     // so only registers with 8*(r/4) < rows matter.
-    if (p.S > 1) {
-        const int nblocks = (p.N + 255) >> 8;
-        // dense: tiles of this launch count from 0; grouped: (linear, problem, column block)
-        const size_t unit = p.problems ? ((size_t)which * p.tiles_y + tile_y) * nblocks + nblk
-                                       : (size_t)tile_y * nblocks + nblk - p.tile0;
+    if (kr.parts > 1) {
+        // Arrive first.  The last workgroup to arrive finishes the tile: it waits until the
+        // others have written their partial sums (they bump the tile's second counter after
+        // their stores; a workgroup that has arrived is running and depends on nothing, so
+        // the wait is short and cannot block) and adds the parts in k order.  If it holds
+        // part 0 itself it starts from its registers and never writes them out.
         constexpr size_t kPerWg = (size_t)4 * MB * 2 * 16 * 64;
-        float* mine = p.partials + (unit * p.S + split) * kPerWg + (size_t)wave * MB * 2 * 16 * 64;
-        if (active) {
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                for (int f = 0; f < 2; ++f)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        if (mb * 32 + 8 * (r >> 2) < rows_here)
-                            __hip_atomic_store(mine + ((mb * 2 + f) * 16 + r) * 64 + lane, acc[mb][f][r],
-                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __syncthreads();
+        unsigned* arrived = p.counters + kr.counter;
+        unsigned* written = p.counters + kGemmWrittenBase + kr.counter;
         if (threadIdx.x == 0) {
-            unsigned old = __hip_atomic_fetch_add(p.counters + unit, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            s_last = (old == (unsigned)(p.S - 1)) ? 1u : 0u;
+            unsigned old = __hip_atomic_fetch_add(arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = (old == (unsigned)(kr.parts - 1)) ? 1u : 0u;
         }
         __syncthreads();
-        if (!s_last) return;
+        const bool finisher = s_last != 0;
+        const float* all = p.partials + kr.slot0 * kPerWg + (size_t)wave * MB * 2 * 16 * 64;
+        if (!(finisher && kr.part == 0)) {
+            float* mine = p.partials + (kr.slot0 + kr.part) * kPerWg + (size_t)wave * MB * 2 * 16 * 64;
+            if (active) {
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int f = 0; f < 2; ++f)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                            if (mb * 32 + 8 * (r >> 2) < rows_here)
+                                __hip_atomic_store(mine + ((mb * 2 + f) * 16 + r) * 64 + lane, acc[mb][f][r],
+                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        if (!finisher) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __syncthreads();
+            if (threadIdx.x == 0) __hip_atomic_fetch_add(written, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+        if (threadIdx.x == 0) {
+            while (__hip_atomic_load(written, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != (unsigned)(kr.parts - 1))
+                __builtin_amdgcn_s_sleep(2);
+            __hip_atomic_store(written, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        if (threadIdx.x == 0) __hip_atomic_store(p.counters + unit, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (active) {
-            const float* all = p.partials + unit * p.S * kPerWg + (size_t)wave * MB * 2 * 16 * 64;
+            // part 0 first (from memory unless it is this workgroup's own), then parts 1, 2, ...
+            // added in order.  64 (128-row tiles) or 128 (32-row tiles) loads a lane are in
+            // flight at a time: half of a part's register blocks, or four whole parts.
+            constexpr int kGroup = MB == 1 ? 2 : 4;             // (mb, f) register blocks per batch
+            constexpr int kParts = MB == 1 ? 4 : 1;             // parts per batch
+            const int first = kr.part == 0 ? 1 : 0;
+            for (int j0 = first; j0 < kr.parts; j0 += kParts) {
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
+                for (int g0 = 0; g0 < MB * 2; g0 += kGroup) {
+                    float tmp[kParts][kGroup][16];
 #pragma unroll
-                for (int f = 0; f < 2; ++f) {
-                    if (mb * 32 >= rows_here) continue;
-                    // sixteen registers x four splits in flight together; adds in split order
-                    float sum[16];
+                    for (int jj = 0; jj < kParts; ++jj) {
+                        const int j = j0 + jj < kr.parts ? j0 + jj : kr.parts - 1;      // past the end: ignored
+                        const float* src = all + (size_t)j * kPerWg;
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) sum[r] = 0.0f;
-                    for (int ss = 0; ss < p.S; ss += 4) {
-                        float part[4][16];
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const int sj = ss + j < p.S ? ss + j : p.S - 1;      // past the end: re-read, ignored
+                        for (int b = 0; b < kGroup; ++b) {
+                            const int blk = g0 + b;             // = mb * 2 + f
+                            if ((blk >> 1) * 32 >= rows_here) continue;                 // workgroup-uniform
 #pragma unroll
                             for (int r = 0; r < 16; ++r)
-                                part[j][r] = __hip_atomic_load(all + (size_t)sj * kPerWg + ((mb * 2 + f) * 16 + r) * 64 + lane,
-                                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                tmp[jj][b][r] = __hip_atomic_load(src + (blk * 16 + r) * 64 + lane, __ATOMIC_RELAXED,
+                                                                  __HIP_MEMORY_SCOPE_AGENT);
                         }
-#pragma unroll
-                        for (int j = 0; j < 4; ++j)
-#pragma unroll
-                            for (int r = 0; r < 16; ++r) {
-                                const float nv = sum[r] + part[j][r];
-                                sum[r] = ss + j < p.S ? nv : sum[r];
-                            }
                     }
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[mb][f][r] = sum[r];
+                    for (int jj = 0; jj < kParts; ++jj) {
+                        if (j0 + jj >= kr.parts) break;
+#pragma unroll
+                        for (int b = 0; b < kGroup; ++b) {
+                            const int blk = g0 + b;
+                            if ((blk >> 1) * 32 >= rows_here) continue;
+#pragma unroll
+                            for (int r = 0; r < 16; ++r)
+                                acc[blk >> 1][blk & 1][r] =
+                                    j0 + jj == 0 ? tmp[jj][b][r] : acc[blk >> 1][blk & 1][r] + tmp[jj][b][r];
+                        }
+                    }
                 }
+            }
         }
     }
 
@@ -377,14 +422,81 @@ __global__ __launch_bounds__(256, 2) void exl3_gemm_kernel(GemmParams p)
     extern __shared__ __align__(16) unsigned char smem[];
     const int unit = blockIdx.x / p.S;
     const int split = blockIdx.x - unit * p.S;
+    const int nblocks = (p.N + 255) >> 8;
+    KRange kr;
+    kr.kb0 = split;
+    kr.kb1 = p.K >> 7;
+    kr.step = p.S;
+    kr.part = split;
+    kr.parts = p.S;
     if (!p.problems) {
-        const int nblocks = (p.N + 255) >> 8;
         const int tile = p.tile0 + unit;
-        gemm_tile<BITS, CB, MB>(p, tile / nblocks, tile % nblocks, split, 0, smem);
+        kr.counter = (size_t)unit;
+        kr.slot0 = kr.counter * p.S;
+        gemm_tile<BITS, CB, MB, true>(p, tile / nblocks, tile % nblocks, kr, 0, smem);
         return;
     }
     if ((int)blockIdx.z >= *p.num_problems) return;
-    gemm_tile<BITS, CB, MB>(p, blockIdx.z, unit, split, blockIdx.y, smem);
+    // grouped: (linear, problem, column block)
+    kr.counter = ((size_t)blockIdx.y * p.tiles_y + blockIdx.z) * nblocks + unit;
+    kr.slot0 = kr.counter * p.S;
+    gemm_tile<BITS, CB, MB, false>(p, blockIdx.z, unit, kr, blockIdx.y, smem);
+}
+
+// Dense launches whose tile count does not divide over the compute units: the
+// (tile, k-block) units of the launch, tile-major, are cut into gridDim.x equal
+// contiguous ranges, one per workgroup (two workgroups per compute unit), so every
+// workgroup does the same amount of decode and MFMA work.  A range covers the end
+// of one tile, possibly whole tiles, and the start of another; a tile shared by
+// several workgroups is finished by the last of them to arrive, which adds the
+// partial sums in k order, so the result does not depend on timing.
+// Workgroup w owns unit_q + 1 units if w < unit_r, else unit_q (units = unit_q * G + unit_r),
+// starting at w * unit_q + min(w, unit_r).  32-bit arithmetic on workgroup-uniform values
+// only, so the k loop and its addresses stay in scalar registers as in the plain kernel.
+__device__ __forceinline__ int range_start(const GemmParams& p, int w) { return w * p.unit_q + min(w, p.unit_r); }
+__device__ __forceinline__ int range_owner(const GemmParams& p, int x)
+{
+    const int big = p.unit_r * (p.unit_q + 1);      // units held by the workgroups with one extra
+    return x < big ? x / (p.unit_q + 1) : p.unit_r + (x - big) / p.unit_q;
+}
+
+template <int BITS, int CB, int MB>
+__device__ __forceinline__ void gemm_segment(const GemmParams& p, const int u, const int stop, unsigned char* smem)
+{
+    const int nblocks = (p.N + 255) >> 8;
+    const int KB = p.K >> 7;
+    const int tile = u / KB;
+    const int t0 = tile * KB;                                   // the tile's first unit
+    const int w_first = range_owner(p, t0);
+    const int w_last = range_owner(p, t0 + KB - 1);
+    KRange kr;
+    kr.kb0 = u - t0;
+    kr.kb1 = stop - t0;
+    kr.step = 1;
+    kr.part = (int)blockIdx.x - w_first;
+    kr.parts = w_last - w_first + 1;
+    kr.counter = (size_t)tile;
+    kr.slot0 = (size_t)tile * p.max_parts;
+    const int t = p.tile0 + tile;
+    gemm_tile<BITS, CB, MB, true>(p, t / nblocks, t % nblocks, kr, 0, smem);
+}
+
+// The launcher uses this kernel when a range is at most one tile long, so a range has at
+// most two segments: the end of one tile and the start of the next.
+template <int BITS, int CB, int MB>
+__global__ __launch_bounds__(256, 2) void exl3_gemm_balanced_kernel(GemmParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int KB = p.K >> 7;
+    const int u = range_start(p, (int)blockIdx.x);
+    const int u_end = range_start(p, (int)blockIdx.x + 1);
+    const int t1 = (u / KB + 1) * KB;
+    const int stop = min(u_end, t1);
+    gemm_segment<BITS, CB, MB>(p, u, stop, smem);
+    if (stop < u_end) {
+        __syncthreads();                                        // the epilogue's LDS tile is the next A tile
+        gemm_segment<BITS, CB, MB>(p, stop, u_end, smem);
+    }
 }
 
 }  // namespace berth

@@ -25,7 +25,7 @@ struct Workspace {
     int device = -1;
     int cu_count = 0;
 };
-constexpr size_t kPartialBytes = 32u << 20;
+constexpr size_t kPartialBytes = (size_t)256 << 20;
 constexpr int kCounters = 65536;
 Workspace& workspace_for_current_device();
 

@@ -14,7 +14,7 @@
  *     ran and is empty after a failure;
  *   - argument validation happens before any device call; C++ exceptions never
  *     cross this boundary; bias is not applied;
- *   - the library owns lazily allocated per-device internals (a 32 MiB split-K
+ *   - the library owns lazily allocated per-device internals (a 256 MiB split-K
  *     workspace and its counters) that are never freed or grown; concurrent
  *     launches on one device are not serialised and share that workspace.
  */

@@ -206,6 +206,38 @@ def test_gemm_split_k(m, Kk, N):
     assert np.array_equal(got.view(np.uint32), got2.view(np.uint32))
 
 
+@pytest.mark.parametrize("m,Kk,N,fp32", [(512, 1024, 4096, True), (384, 640, 5632, False), (200, 768, 8320, True),
+                                         (130, 256, 16384, False)])
+def test_gemm_128_row_tiles_dealt_out_evenly(m, Kk, N, fp32):
+    """Enough 128 x 256 tiles to use them: the (tile, k-block) units are cut into one equal
+    range per compute unit, tiles shared by several workgroups are summed in k order."""
+    got, want, ah, want_ah, launch = _run_linear(m, Kk, N, 4, 2, fp32, 700 + m, prefill=True)
+    assert "exl3_gemm_balanced_kernel<4,2,128x256>" in launch, launch
+    assert np.array_equal(ah, want_ah)
+    bad, worst = close(got, want)
+    assert bad == 0, (bad, worst, launch)
+    got2, _, _, _, _ = _run_linear(m, Kk, N, 4, 2, fp32, 700 + m, prefill=True)
+    assert np.array_equal(got.view(np.uint16), got2.view(np.uint16))
+
+
+def test_gemm_128_row_tiles_one_workgroup_per_tile_and_split():
+    """The same tiles without the even deal (BERTH_GEMM_BALANCED=0, read once per process)."""
+    import os
+    import subprocess
+    import sys
+    code = (
+        "import numpy as np, tests.test_gpu_linear as T\n"
+        "for m, K, N in ((512, 1024, 4096), (200, 768, 8320)):\n"
+        "    got, want, ah, want_ah, launch = T._run_linear(m, K, N, 4, 2, True, 700 + m, prefill=True)\n"
+        "    assert 'exl3_gemm_kernel<4,2,128x256>' in launch, launch\n"
+        "    assert np.array_equal(ah, want_ah) and T.close(got, want)[0] == 0, launch\n"
+        "print('ok')\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=600, cwd=root,
+                       env=dict(os.environ, BERTH_GEMM_BALANCED="0"))
+    assert r.returncode == 0 and "ok" in r.stdout, r.stdout + r.stderr
+
+
 def test_linear_through_decode_entry_with_many_rows():
     """forward_n passes rows 2..144 of a K = 6 linear to the m = 1 entry
     (crates/berth-engine/src/device.rs:338-352)."""
