@@ -460,8 +460,19 @@ __device__ __forceinline__ int range_owner(const GemmParams& p, int x)
     return x < big ? x / (p.unit_q + 1) : p.unit_r + (x - big) / p.unit_q;
 }
 
+// Workgroups are handed to the eight compute dies round-robin (workgroup i runs on die
+// i % 8), and every die has its own L2.  Renumbering them so that a die gets a contiguous
+// eighth of the ranges makes the tiles of one die share their rows of the activation
+// (one 128-row block, 1.3 MB at K = 5120, instead of all of them): a quarter less traffic
+// behind the L2 on the 27B gate projection at 512 rows.
+__device__ __forceinline__ int die_major_index(int i, int n)
+{
+    return (n & 7) == 0 ? (i & 7) * (n >> 3) + (i >> 3) : i;
+}
+
 template <int BITS, int CB, int MB>
-__device__ __forceinline__ void gemm_segment(const GemmParams& p, const int u, const int stop, unsigned char* smem)
+__device__ __forceinline__ void gemm_segment(const GemmParams& p, const int w, const int u, const int stop,
+                                             unsigned char* smem)
 {
     const int nblocks = (p.N + 255) >> 8;
     const int KB = p.K >> 7;
@@ -473,7 +484,7 @@ __device__ __forceinline__ void gemm_segment(const GemmParams& p, const int u, c
     kr.kb0 = u - t0;
     kr.kb1 = stop - t0;
     kr.step = 1;
-    kr.part = (int)blockIdx.x - w_first;
+    kr.part = w - w_first;
     kr.parts = w_last - w_first + 1;
     kr.counter = (size_t)tile;
     kr.slot0 = (size_t)tile * p.max_parts;
@@ -488,14 +499,15 @@ __global__ __launch_bounds__(256, 2) void exl3_gemm_balanced_kernel(GemmParams p
 {
     extern __shared__ __align__(16) unsigned char smem[];
     const int KB = p.K >> 7;
-    const int u = range_start(p, (int)blockIdx.x);
-    const int u_end = range_start(p, (int)blockIdx.x + 1);
+    const int w = die_major_index((int)blockIdx.x, (int)gridDim.x);
+    const int u = range_start(p, w);
+    const int u_end = range_start(p, w + 1);
     const int t1 = (u / KB + 1) * KB;
     const int stop = min(u_end, t1);
-    gemm_segment<BITS, CB, MB>(p, u, stop, smem);
+    gemm_segment<BITS, CB, MB>(p, w, u, stop, smem);
     if (stop < u_end) {
         __syncthreads();                                        // the epilogue's LDS tile is the next A tile
-        gemm_segment<BITS, CB, MB>(p, stop, u_end, smem);
+        gemm_segment<BITS, CB, MB>(p, w, stop, u_end, smem);
     }
 }
 
