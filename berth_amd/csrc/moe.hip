@@ -68,38 +68,64 @@ struct RouteParams {
 // over the selected k (renorm) or over all experts.
 constexpr int kRoutePer = kMaxExperts / 64;
 
-__device__ __forceinline__ int route_topk(const float (&lg)[kRoutePer], int lane, const RouteParams& p, int t)
+__device__ __forceinline__ float lane_value(float v, int lane_index)
 {
-    constexpr int PER = kRoutePer;
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane_index));
+}
+
+// the same value in every lane: butterflies over lane distances 1 .. 32
+__device__ __forceinline__ float wave_max(float v)
+{
+    v = fmaxf(v, lane_xor_dpp<1>(v));
+    v = fmaxf(v, lane_xor_dpp<2>(v));
+    v = fmaxf(v, lane_xor_dpp<4>(v));
+    v = fmaxf(v, lane_xor_dpp<8>(v));
+    v = fmaxf(v, lane_xor_swap16(v));
+    return fmaxf(v, lane_xor_swap32(v));
+}
+__device__ __forceinline__ int wave_min(int v)
+{
+    auto x = [](int a) { return __builtin_bit_cast(float, a); };
+    auto y = [](float a) { return __builtin_bit_cast(int, a); };
+    v = min(v, y(lane_xor_dpp<1>(x(v))));
+    v = min(v, y(lane_xor_dpp<2>(x(v))));
+    v = min(v, y(lane_xor_dpp<4>(x(v))));
+    v = min(v, y(lane_xor_dpp<8>(x(v))));
+    v = min(v, y(lane_xor_swap16(x(v))));
+    return min(v, y(lane_xor_swap32(x(v))));
+}
+
+// PER: how many of the lane's registers can hold experts (ceil(E / 64) rounded up to 2, 8 or 16)
+template <int PER>
+__device__ __forceinline__ int route_topk_n(const float (&lg)[kRoutePer], int lane, const RouteParams& p, int t)
+{
     unsigned taken = 0;
     float sel_logit = 0.0f;         // lane j keeps the logit of slot j
     int sel_idx = 0;
+    // One slot per round: the largest remaining logit of the wave (max butterflies), then the
+    // lowest expert index among the registers that hold it (min butterflies).  Two short
+    // reductions of one value each instead of one reduction of (value, index) pairs with a
+    // tie rule: the dependent instruction chain of a round is about a third as long.
     for (int j = 0; j < p.k; ++j) {
-        float bv = -INFINITY;
-        int bi = 0x7fffffff;
+        float lv = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < PER; ++i) {
-            const int e = lane + 64 * i;
-            if (e < p.E && !((taken >> i) & 1u) && (bi == 0x7fffffff || lg[i] > bv)) { bv = lg[i]; bi = e; }
-        }
-        auto merge = [&](float ov, int oi) {
-            const bool take = (oi != 0x7fffffff) && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi));
-            if (take) { bv = ov; bi = oi; }
-        };
-        merge(lane_xor_dpp<1>(bv), __builtin_bit_cast(int, lane_xor_dpp<1>(__builtin_bit_cast(float, bi))));
-        merge(lane_xor_dpp<2>(bv), __builtin_bit_cast(int, lane_xor_dpp<2>(__builtin_bit_cast(float, bi))));
-        merge(lane_xor_dpp<4>(bv), __builtin_bit_cast(int, lane_xor_dpp<4>(__builtin_bit_cast(float, bi))));
-        merge(lane_xor_dpp<8>(bv), __builtin_bit_cast(int, lane_xor_dpp<8>(__builtin_bit_cast(float, bi))));
-        merge(lane_xor_swap16(bv), __builtin_bit_cast(int, lane_xor_swap16(__builtin_bit_cast(float, bi))));
-        merge(lane_xor_swap32(bv), __builtin_bit_cast(int, lane_xor_swap32(__builtin_bit_cast(float, bi))));
+        for (int i = 0; i < PER; ++i)
+            if (lane + 64 * i < p.E && !((taken >> i) & 1u)) lv = fmaxf(lv, lg[i]);
+        const float bv = wave_max(lv);
+        int ci = 0x7fffffff;
+#pragma unroll
+        for (int i = PER - 1; i >= 0; --i)
+            if (lane + 64 * i < p.E && !((taken >> i) & 1u) && lg[i] == bv) ci = lane + 64 * i;
+        const int bi = wave_min(ci);
         if ((bi & 63) == lane) taken |= 1u << (bi >> 6);
         if (lane == j) { sel_logit = bv; sel_idx = bi; }
     }
-    const float mx = __shfl(sel_logit, 0, 64);
+    // lane j is wave-uniform here: v_readlane instead of a round trip through the LDS crossbar
+    const float mx = lane_value(sel_logit, 0);
     float ev = (lane < p.k) ? expf(sel_logit - mx) : 0.0f;
     float denom = 0.0f;
     if (p.renorm) {
-        for (int j = 0; j < p.k; ++j) denom += __shfl(ev, j, 64);       // slot order
+        for (int j = 0; j < p.k; ++j) denom += lane_value(ev, j);       // slot order
     } else {
         float loc = 0.0f;
 #pragma unroll
@@ -116,6 +142,13 @@ __device__ __forceinline__ int route_topk(const float (&lg)[kRoutePer], int lane
     return sel_idx;     // lane j < k: expert of slot j
 }
 
+__device__ __forceinline__ int route_topk(const float (&lg)[kRoutePer], int lane, const RouteParams& p, int t)
+{
+    if (p.E <= 128) return route_topk_n<2>(lg, lane, p, t);         // workgroup-uniform
+    if (p.E <= 512) return route_topk_n<8>(lg, lane, p, t);
+    return route_topk_n<kRoutePer>(lg, lane, p, t);
+}
+
 // One token: what moe_permute_kernel writes, by the wave that holds the selection
 // (lane j < k has the expert of slot j; the k experts are distinct).  Sorted position
 // of slot j = number of selected experts with a smaller index; every expert is one
@@ -125,7 +158,7 @@ __device__ __forceinline__ void route_sort_one_token(const PermuteParams& q, int
     const int k = q.k;
     int rank = 0;
     for (int j = 0; j < k; ++j) {
-        const int other = __shfl(sel_idx, j, 64);
+        const int other = __builtin_amdgcn_readlane(sel_idx, j);
         rank += (lane < k && other < sel_idx) ? 1 : 0;
     }
     if (lane < k) {
@@ -138,7 +171,7 @@ __device__ __forceinline__ void route_sort_one_token(const PermuteParams& q, int
     for (int e0 = 0; e0 <= q.E; e0 += 64) {         // wave-uniform loop: every lane takes part in the exchanges
         const int e = e0 + lane;
         int below = 0;
-        for (int j = 0; j < k; ++j) below += (__shfl(sel_idx, j, 64) < e) ? 1 : 0;
+        for (int j = 0; j < k; ++j) below += (__builtin_amdgcn_readlane(sel_idx, j) < e) ? 1 : 0;
         if (e <= q.E) q.offsets[e] = below;
     }
     if (lane == 0) {
@@ -237,6 +270,87 @@ __global__ __launch_bounds__(256) void moe_route_kernel(RouteParams p)
     }
     const int sel = route_topk(lg, lane, p, t);
     if (p.sort.perm) route_sort_one_token(p.sort, lane, sel);
+}
+
+// One token and a small router (at most 128 experts, an even number; at most 4096 rows):
+// a single workgroup of sixteen waves streams the whole router weight, so the segment sums
+// meet in LDS instead of travelling through memory and a counter.  Wave w takes segments w,
+// w + 16, ...; a lane holds two neighbouring experts (one 4-byte load per row) and the
+// segment's activations come from the lanes of one coalesced load (v_readlane: the row index
+// is the same for the whole wave).  Same arithmetic as moe_route_kernel: fma chains in row
+// order per 64-row segment, segments added in order, bias, top-k, sort.
+constexpr int kRouteOneMaxSeg = 64;
+constexpr int kRouteOneMaxE = 128;
+
+__global__ __launch_bounds__(1024) void moe_route_one_token_kernel(RouteParams p)
+{
+    __shared__ float part_s[kRouteOneMaxSeg][kRouteOneMaxE];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#ifdef BERTH_ROUTE_TRACE
+    long long q0 = wall_clock64();
+#endif
+    const int pairs = p.E >> 1;                         // lanes with work
+    const int col = min(lane, pairs - 1);               // idle lanes repeat the last pair and store nothing
+    const global_ptr<const uint32_t> wr = (global_ptr<const uint32_t>)as_global((const uint32_t*)p.wr);
+
+    for (int seg = wave; seg < p.nseg; seg += 16) {
+        const int h0 = seg * kRouteSeg;
+        const int hn = min(kRouteSeg, p.H - h0);
+        // one activation per lane (zero past the end of the input), broadcast row by row with
+        // v_readlane; rows past the end of a partial segment re-read its last row and meet zeros
+        const float xv = lane < hn ? (float)p.x[h0 + lane] : 0.0f;
+        uint32_t wv[kRouteSeg];
+#pragma unroll
+        for (int i = 0; i < kRouteSeg; ++i) wv[i] = wr[(size_t)(h0 + min(i, hn - 1)) * pairs + col];
+        float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kRouteSeg; ++i) {
+            const float xi = lane_value(xv, i);
+            const half2_t w2 = as_half2(wv[i]);
+            a0 = __builtin_fmaf(xi, (float)w2.x, a0);
+            a1 = __builtin_fmaf(xi, (float)w2.y, a1);
+        }
+        if (lane < pairs) {
+            part_s[seg][2 * lane] = a0;
+            part_s[seg][2 * lane + 1] = a1;
+        }
+    }
+#ifdef BERTH_ROUTE_TRACE
+    long long q1 = wall_clock64();
+#endif
+    __syncthreads();
+    if (wave != 0) return;
+#ifdef BERTH_ROUTE_TRACE
+    long long q2 = wall_clock64();
+#endif
+
+    constexpr int PER = kRoutePer;
+    float lg[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int e = lane + 64 * i;
+        float v = -INFINITY;
+        if (i < kRouteOneMaxE / 64 && e < p.E) {
+            v = 0.0f;
+            for (int sg = 0; sg < p.nseg; ++sg) v += part_s[sg][e];
+            if (p.bias) v += p.bias[e];
+            if (p.logits) p.logits[e] = v;
+        }
+        lg[i] = v;
+    }
+#ifdef BERTH_ROUTE_TRACE
+    long long q3 = wall_clock64();
+#endif
+    const int sel = route_topk(lg, lane, p, 0);
+#ifdef BERTH_ROUTE_TRACE
+    long long q4 = wall_clock64();
+#endif
+    if (p.sort.perm) route_sort_one_token(p.sort, lane, sel);
+#ifdef BERTH_ROUTE_TRACE
+    long long q5 = wall_clock64();
+    if (lane == 0) printf("route: stream %lld barrier %lld sum %lld topk %lld sort %lld (10 ns ticks)\n", q1 - q0, q2 - q1, q3 - q2, q4 - q3, q5 - q4);
+#endif
 }
 
 // Many tokens: the same arithmetic in two launches, so that the segment sums of a
@@ -672,6 +786,11 @@ std::string run_route(const void* x, const void* wr, const float* bias, int32_t*
         hip_ok(hipGetLastError(), "moe_route_finish_kernel launch");
         return "moe_route_partial_kernel grid=" + std::to_string(grid.x) + "x" + std::to_string(grid.y) +
                " + moe_route_finish_kernel grid=" + std::to_string(T);
+    }
+    if (T == 1 && E % 2 == 0 && E <= kRouteOneMaxE && p.nseg <= kRouteOneMaxSeg) {
+        hipLaunchKernelGGL(moe_route_one_token_kernel, dim3(1), dim3(1024), 0, stream, p);
+        hip_ok(hipGetLastError(), "moe_route_one_token_kernel launch");
+        return std::string("moe_route_one_token_kernel grid=1") + (p.sort.perm ? " (with the sort of the one token)" : "");
     }
     dim3 grid(p.nseg, groups);
     hipLaunchKernelGGL(moe_route_kernel, grid, dim3(256), 0, stream, p);
