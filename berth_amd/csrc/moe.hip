@@ -287,9 +287,6 @@ __global__ __launch_bounds__(1024) void moe_route_one_token_kernel(RouteParams p
     __shared__ float part_s[kRouteOneMaxSeg][kRouteOneMaxE];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-#ifdef BERTH_ROUTE_TRACE
-    long long q0 = wall_clock64();
-#endif
     const int pairs = p.E >> 1;                         // lanes with work
     const int col = min(lane, pairs - 1);               // idle lanes repeat the last pair and store nothing
     const global_ptr<const uint32_t> wr = (global_ptr<const uint32_t>)as_global((const uint32_t*)p.wr);
@@ -316,14 +313,8 @@ __global__ __launch_bounds__(1024) void moe_route_one_token_kernel(RouteParams p
             part_s[seg][2 * lane + 1] = a1;
         }
     }
-#ifdef BERTH_ROUTE_TRACE
-    long long q1 = wall_clock64();
-#endif
     __syncthreads();
     if (wave != 0) return;
-#ifdef BERTH_ROUTE_TRACE
-    long long q2 = wall_clock64();
-#endif
 
     constexpr int PER = kRoutePer;
     float lg[PER];
@@ -339,18 +330,8 @@ __global__ __launch_bounds__(1024) void moe_route_one_token_kernel(RouteParams p
         }
         lg[i] = v;
     }
-#ifdef BERTH_ROUTE_TRACE
-    long long q3 = wall_clock64();
-#endif
     const int sel = route_topk(lg, lane, p, 0);
-#ifdef BERTH_ROUTE_TRACE
-    long long q4 = wall_clock64();
-#endif
     if (p.sort.perm) route_sort_one_token(p.sort, lane, sel);
-#ifdef BERTH_ROUTE_TRACE
-    long long q5 = wall_clock64();
-    if (lane == 0) printf("route: stream %lld barrier %lld sum %lld topk %lld sort %lld (10 ns ticks)\n", q1 - q0, q2 - q1, q3 - q2, q4 - q3, q5 - q4);
-#endif
 }
 
 // Many tokens: the same arithmetic in two launches, so that the segment sums of a
