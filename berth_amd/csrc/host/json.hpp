@@ -5,6 +5,7 @@
 //   * a number is an unsigned integer, a negative integer or a float, decided by
 //     its spelling ("6" is an integer, "6.0" and "6e0" are floats), and integers
 //     that do not fit 64 bits become floats;
+//   * strings must be valid UTF-8;
 //   * nesting is limited to 128 levels;
 //   * errors carry "<reason> at line L column C".
 // Header-only, no dependencies beyond the standard library.
@@ -224,6 +225,24 @@ private:
             const unsigned char c = (unsigned char)*p_++;
             if (c == '"') return out;
             if (c < 0x20) fail("control character (\\u0000-\\u001F) found while parsing a string");
+            if (c >= 0x80) {
+                // a string is UTF-8: check the sequence (no overlong forms, no surrogates, <= U+10FFFF)
+                int more = c >= 0xF0 ? 3 : c >= 0xE0 ? 2 : c >= 0xC2 ? 1 : -1;
+                if (c > 0xF4) more = -1;
+                if (more < 0 || end_ - p_ < more) fail("invalid unicode code point");
+                const unsigned char c1 = (unsigned char)p_[0];
+                bool okay = (c1 & 0xC0) == 0x80;
+                if (c == 0xE0) okay = okay && c1 >= 0xA0;
+                if (c == 0xED) okay = okay && c1 < 0xA0;
+                if (c == 0xF0) okay = okay && c1 >= 0x90;
+                if (c == 0xF4) okay = okay && c1 < 0x90;
+                for (int k = 1; k < more; ++k) okay = okay && ((unsigned char)p_[k] & 0xC0) == 0x80;
+                if (!okay) fail("invalid unicode code point");
+                out += (char)c;
+                out.append(p_, (size_t)more);
+                p_ += more;
+                continue;
+            }
             if (c != '\\') { out += (char)c; continue; }
             if (p_ == end_) fail("EOF while parsing a string");
             const char e = *p_++;

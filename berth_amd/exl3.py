@@ -124,7 +124,7 @@ class TensorInfo:
         `dtype`, shaped like the tensor when the element sizes agree."""
         raw = np.empty(self.length, dtype=np.uint8)
         shape = (C.c_uint64 * max(1, len(self.shape)))(*self.shape)
-        t = _Tensor(self.name.encode(), self.shard.encode(), int(self.dtype), len(self.shape), shape, self.offset,
+        t = _Tensor(self.name.encode(), os.fsencode(self.shard), int(self.dtype), len(self.shape), shape, self.offset,
                     self.length)
         _check(_load().berth_ckpt_read_tensor(C.byref(t), raw.ctypes.data_as(C.c_void_p), self.length))
         out = raw.view(dtype)
@@ -288,7 +288,7 @@ def _str(b) -> Optional[str]:
 
 
 def _tensor(t: _Tensor) -> TensorInfo:
-    return TensorInfo(t.name.decode(), t.shard.decode(), DType(t.dtype), tuple(int(t.shape[i]) for i in range(t.rank)),
+    return TensorInfo(t.name.decode("utf-8", "replace"), os.fsdecode(t.shard), DType(t.dtype), tuple(int(t.shape[i]) for i in range(t.rank)),
                       int(t.offset), int(t.length))
 
 
@@ -304,7 +304,8 @@ def _config(handle) -> ModelConfig:
         version=_str(c.version), vision_bits=opt("vision_bits"), mtp_bits=opt("mtp_bits"),
         out_scales=_str(c.out_scales),
         calibration=Calibration(int(c.calibration_rows), int(c.calibration_cols)) if c.has_calibration else None)
-    layers = tuple((LayerType(c.layer_type_kinds[i]), c.layer_type_names[i].decode()) for i in range(c.num_layer_types))
+    layers = tuple((LayerType(c.layer_type_kinds[i]), c.layer_type_names[i].decode("utf-8", "replace"))
+                   for i in range(c.num_layer_types))
     return ModelConfig(
         arch_string=_str(c.arch_string), num_hidden_layers=int(c.num_hidden_layers), hidden_size=int(c.hidden_size),
         intermediate_size=opt("intermediate_size"), head_dim=int(c.head_dim),
@@ -324,7 +325,7 @@ class LinearExl3:
     def __init__(self, owner: "Checkpoint", index: int, rec: _Linear):
         self._owner = owner
         self._index = index
-        self.prefix = rec.prefix.decode()
+        self.prefix = rec.prefix.decode("utf-8", "replace")
         self.trellis = _tensor(rec.trellis)
         self.input_scale = HadamardScale(_tensor(rec.input_scale), bool(rec.input_packed))
         self.output_scale = HadamardScale(_tensor(rec.output_scale), bool(rec.output_packed))
@@ -383,7 +384,7 @@ class Checkpoint:
     def __init__(self, handle):
         self._handle = handle
         L = _load()
-        self.directory = L.berth_ckpt_directory(handle).decode()
+        self.directory = os.fsdecode(L.berth_ckpt_directory(handle))
         self.config = _config(L.berth_ckpt_config_of(handle))
         self.tensors = TensorIndex(self)
         self._linears = []

@@ -571,6 +571,14 @@ def test_json_reader_details():
     assert ModelConfig.from_slice(text.encode()).arch_string == "Lasté😀"
     value["quantization_config"]["bits"] = 18446744073709551616        # 2^64: a float, fine for `bits`
     assert parse(value).quantization.bits == 2.0 ** 64
+    # strings are UTF-8: a stray continuation byte, an overlong form and a surrogate are refused
+    for bad in (b"\x80", b"\xc0\xaf", b"\xed\xa0\x80", b"\xf5\x80\x80\x80", b"\xe2\x82"):
+        blob = json.dumps(sample()).encode().replace(b"Qwen3_5ForConditionalGeneration", b"Q" + bad + b"x")
+        with pytest.raises(Error) as e:
+            ModelConfig.from_slice(blob)
+        assert e.value.kind == ErrorKind.PARSE and "invalid unicode code point" in str(e.value)
+    ok = json.dumps(sample()).encode().replace(b"Qwen3_5ForConditionalGeneration", "Qé€😀".encode())
+    assert ModelConfig.from_slice(ok).arch_string == "Qé€😀"
     deep = b"[" * 200 + b"]" * 200
     with pytest.raises(Error, match="recursion limit"):
         ModelConfig.from_slice(deep)
@@ -618,3 +626,47 @@ def test_cpp_host_layer_lists_a_checkpoint_without_a_device(tmp_path):
     assert "linear block.0.v k=4 codebook=2 packed=0/0 bias=0" in r.stdout
     r = subprocess.run([exe, "ckpt-info", str(tmp_path / "nope")], capture_output=True, text=True, timeout=60)
     assert r.returncode == 1 and "not a checkpoint directory" in r.stderr
+
+
+def test_mutated_headers_and_configs_only_ever_raise_reader_errors(tmp_path):
+    """Truncations and single-byte edits of a valid header / config either parse or fail with
+    the reader's own error: never a crash, never another exception type."""
+    rng = np.random.default_rng(11)
+    write_config(tmp_path)
+    shard = tmp_path / "model.safetensors"
+    write_tensors(shard, demo_tensors())
+    good = shard.read_bytes()
+    header_len = struct.unpack("<Q", good[:8])[0]
+    outcomes = {"ok": 0, "error": 0}
+
+    def attempt():
+        try:
+            Checkpoint.open(tmp_path)
+            outcomes["ok"] += 1
+        except Error as e:
+            assert e.kind in (ErrorKind.MISSING_FIELD, ErrorKind.BAD_FIELD, ErrorKind.READ, ErrorKind.PARSE)
+            assert str(e)
+            outcomes["error"] += 1
+
+    for cut in list(range(0, 24)) + [int(v) for v in rng.integers(24, len(good), size=40)]:
+        shard.write_bytes(good[:cut])
+        attempt()
+    for _ in range(200):
+        pos = int(rng.integers(0, 8 + header_len))
+        b = bytearray(good)
+        b[pos] = int(rng.integers(0, 256))
+        shard.write_bytes(bytes(b))
+        attempt()
+    shard.write_bytes(good)
+    cfg = json.dumps(CONFIG).encode()
+    for _ in range(200):
+        b = bytearray(cfg)
+        for _ in range(int(rng.integers(1, 4))):
+            b[int(rng.integers(0, len(b)))] = int(rng.integers(0, 256))
+        (tmp_path / "config.json").write_bytes(bytes(b))
+        attempt()
+        try:
+            ModelConfig.from_slice(bytes(b[:int(rng.integers(0, len(b)))]))
+        except Error:
+            pass
+    assert outcomes["error"] > 100 and outcomes["ok"] > 10, outcomes
