@@ -199,13 +199,25 @@ std::string launch_gemv_grouped(const GroupedArgs& g)
     const long units = (long)g.max_problems * g.num_lins * p.NB;
     if (units > kCounters) throw std::runtime_error("moe grouped linear: too many (problem, column block) units");
     const int mmax = g.single_row ? 1 : 8;
+    if (g.comb_out) {
+        if (!g.single_row || g.num_lins != 1 || !g.out_fp32 || !g.a_up || !g.comb_w || !g.comb_inv || g.comb_k < 1)
+            throw std::runtime_error("moe grouped linear: the folded combine needs one-row problems of a silu-input fp32 linear");
+        if (units + p.NB > kCounters) throw std::runtime_error("moe grouped linear: too many units for the folded combine");
+        p.comb_w = g.comb_w;
+        p.comb_inv = g.comb_inv;
+        p.comb_shared = g.comb_shared;
+        p.comb_out = g.comb_out;
+        p.comb_counters = ws.counters + units;
+        p.comb_k = g.comb_k;
+    }
     p.S = pick_split(ws, units, p.KB, mmax);
     dim3 grid((unsigned)(g.max_problems * p.NB * p.S), (unsigned)g.num_lins);
     launch_bits(p, g.k_bits, g.codebook, mmax, grid, g.stream);
     hip_ok(hipGetLastError(), "exl3_gemv_kernel grouped launch");
     return "exl3_gemv_kernel<" + std::to_string(g.k_bits) + "," + std::to_string(g.codebook) + "," +
            std::to_string(mmax) + "> grouped grid=" +
-           std::to_string(grid.x) + "x" + std::to_string(grid.y) + " split_k=" + std::to_string(p.S);
+           std::to_string(grid.x) + "x" + std::to_string(grid.y) + " split_k=" + std::to_string(p.S) +
+           (g.comb_out ? " +combine" : "");
 }
 
 }  // namespace berth

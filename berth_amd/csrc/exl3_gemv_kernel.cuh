@@ -78,6 +78,17 @@ struct GemvParams {
     float* partials;            // [problem][lin][NB][S][MMAX][128]
     unsigned* counters;         // [problem][lin][NB]
     int K, N, NB, KB, S, out_fp32;
+    // one-token expert combine folded into the down projection (grouped mode, one
+    // row per problem, fp32 rows in c[0]): the last problem to finish a column
+    // block writes comb_out[h] = fma chain over j of comb_w[j] * c[0][comb_inv[j]][h]
+    // starting from comb_shared[h] (or 0), the arithmetic of the separate combine
+    // kernel.  comb_out == nullptr: off.
+    const float* comb_w;
+    const int32_t* comb_inv;
+    const float* comb_shared;
+    float* comb_out;
+    unsigned* comb_counters;    // [NB], zero between launches
+    int comb_k;
 };
 
 // silu(g) * u with every step rounded to fp16: e = exp(-g); s = 1 + e; r = 1 / s;
@@ -389,6 +400,58 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
         v0 = (v0 * kRsqrt128) * (float)sv.x;
         v1 = (v1 * kRsqrt128) * (float)sv.y;
         size_t at = (size_t)(row0 + m) * n_stride + nb * 128 + 2 * lane;
+        if constexpr (SILU && MMAX == 1) {
+            if (p.comb_out) {
+                // m == 0, wave 0.  The row goes out as agent-scope atomic stores so
+                // that whichever workgroup arrives last can read every row of this
+                // column block without a cache write-back; the stores have to be
+                // complete before the arrival is counted.
+                union Pair { unsigned long long u; float f[2]; };
+                Pair mine;
+                mine.f[0] = v0;
+                mine.f[1] = v1;
+                __hip_atomic_store((unsigned long long*)((float*)cout + at), mine.u, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                unsigned old = 0;
+                if (lane == 0)
+                    old = __hip_atomic_fetch_add(p.comb_counters + nb, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                old = (unsigned)__builtin_amdgcn_readfirstlane((int)old);
+                if (old + 1 != (unsigned)*p.num_problems) return;
+                if (lane == 0) __hip_atomic_store(p.comb_counters + nb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                const int h = nb * 128 + 2 * lane;
+                Pair acc2;
+                acc2.u = 0ull;
+                if (p.comb_shared)
+                    acc2.u = __hip_atomic_load((const unsigned long long*)(p.comb_shared + h), __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+                float a0 = acc2.f[0], a1 = acc2.f[1];
+                // eight rows in flight at a time; the fma chain stays in slot order
+                for (int j0 = 0; j0 < p.comb_k; j0 += 8) {
+                    Pair part[8];
+                    float wj[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        const int j = j0 + u < p.comb_k ? j0 + u : p.comb_k - 1;
+                        wj[u] = p.comb_w[j];
+                        const float* row = (const float*)cout + (size_t)p.comb_inv[j] * n_stride + h;
+                        part[u].u = __hip_atomic_load((const unsigned long long*)row, __ATOMIC_RELAXED,
+                                                      __HIP_MEMORY_SCOPE_AGENT);
+                    }
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        if (j0 + u < p.comb_k) {
+                            a0 = __builtin_fmaf(wj[u], part[u].f[0], a0);
+                            a1 = __builtin_fmaf(wj[u], part[u].f[1], a1);
+                        }
+                }
+                float2_t o2 = {a0, a1};
+                *(float2_t*)(p.comb_out + h) = o2;
+                return;
+            }
+        }
         if (p.out_fp32) {
             float2_t o = {v0, v1};
             *(float2_t*)((float*)cout + at) = o;

@@ -75,6 +75,14 @@ struct GroupedArgs {
     const void* a_had2;         // ... and of the second linear of the launch
     int size_k, size_n, k_bits, codebook, out_fp32;
     hipStream_t stream;
+    // VALU path, single_row, one linear, fp32 out, silu input: also combine the
+    // problems' rows into comb_out[size_n] (weights comb_w[comb_k], rows
+    // comb_inv[comb_k] of c0, start value comb_shared[size_n] or zero)
+    const float* comb_w = nullptr;
+    const int32_t* comb_inv = nullptr;
+    const float* comb_shared = nullptr;
+    float* comb_out = nullptr;
+    int comb_k = 0;
 };
 std::string launch_gemv_grouped(const GroupedArgs& args);
 std::string launch_gemm_grouped(const GroupedArgs& args);

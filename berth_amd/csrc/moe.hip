@@ -680,6 +680,17 @@ int moe_big_min()
     return v;
 }
 
+// One token: the down projection's last arrival per column block also combines the
+// block (BERTH_MOE_FOLD_COMBINE=0 keeps the separate combine launch).
+bool fold_combine_enabled()
+{
+    static const bool v = [] {
+        const char* e = std::getenv("BERTH_MOE_FOLD_COMBINE");
+        return !e || std::atoi(e) != 0;
+    }();
+    return v;
+}
+
 // The always-on expert runs as one more expert of the grouped launches (rows P ..
 // P + T - 1, token order) when it has the routed experts' intermediate size.
 bool shared_is_folded(int I, int shared_I) { return shared_I > 0 && shared_I == I; }
@@ -994,6 +1005,37 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
         desc += " + " + launch_gemm_grouped(g);
     }
 
+    // shared expert: three dense linears on every token (ahead of the routed down
+    // projection, which may finish the layer)
+    const float* shared_out = nullptr;
+    if (fold) {
+        shared_out = (const float*)(wsb + L.shared_out);
+        desc += " (shared expert in the grouped launches)";
+    } else if (shared) {
+        auto dense = [&](const void* a, const berth_exl3_lin& lin, void* c, int kk, int nn, int fp32) {
+            LinearArgs la{a, lin.trellis, c, lin.suh, wsb + L.s_ahad, lin.svh, T, kk, nn, k_bits, codebook, fp32, stream};
+            return T <= 8 ? launch_gemv(la) : launch_gemm(la);
+        };
+        if (T <= 8) {
+            // gate and up in one launch, silu(g) * u formed inside the down projection
+            PairArgs pa{x, {shared[0].trellis, shared[1].trellis}, {shared[0].suh, shared[1].suh},
+                        {shared[0].svh, shared[1].svh}, {wsb + L.sg, wsb + L.su}, wsb + L.s_ahad, T, H, shared_I,
+                        k_bits, codebook, stream};
+            launch_gemv_pair(pa);
+            LinearArgs down{wsb + L.sg, shared[2].trellis, wsb + L.shared_out, shared[2].suh, wsb + L.s_ahad,
+                            shared[2].svh, T, shared_I, H, k_bits, codebook, 1, stream};
+            down.a_up = wsb + L.su;
+            launch_gemv(down);
+        } else {
+            dense(x, shared[0], wsb + L.sg, H, shared_I, 0);
+            dense(x, shared[1], wsb + L.su, H, shared_I, 0);
+            launch_silu_mul(wsb + L.sg, wsb + L.su, wsb + L.su, (int64_t)T * shared_I, 0.0f, stream);
+            dense(wsb + L.su, shared[2], wsb + L.shared_out, shared_I, H, 1);
+        }
+        shared_out = (const float*)(wsb + L.shared_out);
+        desc += " + shared expert";
+    }
+
     // down: input silu(g) * u evaluated while the activation is rotated, fp32 out
     g.a = wsb + L.g;
     g.a_up = wsb + L.u;
@@ -1006,6 +1048,16 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
     g.size_k = I;
     g.size_n = H;
     g.out_fp32 = 1;
+    // one token: the last expert to finish a column block of the down projection
+    // also combines that block, so no combine launch follows
+    const bool fold_combine = T == 1 && L.max_v > 0 && L.max_m == 0 && fold_combine_enabled();
+    if (fold_combine) {
+        g.comb_w = (const float*)w;
+        g.comb_inv = (const int32_t*)(wsb + L.inv);
+        g.comb_shared = shared_out;
+        g.comb_out = (float*)out;
+        g.comb_k = k;
+    }
     if (L.max_v > 0) {
         g.problems = wsb + L.vprob;
         g.num_problems = (const int*)(wsb + L.counts);
@@ -1045,42 +1097,14 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
         desc += " + " + launch_gemm_grouped(g);
     }
 
-    // shared expert: three dense linears on every token
-    const float* shared_out = nullptr;
-    if (fold) {
-        shared_out = (const float*)(wsb + L.shared_out);
-        desc += " (shared expert in the grouped launches)";
-    } else if (shared) {
-        auto dense = [&](const void* a, const berth_exl3_lin& lin, void* c, int kk, int nn, int fp32) {
-            LinearArgs la{a, lin.trellis, c, lin.suh, wsb + L.s_ahad, lin.svh, T, kk, nn, k_bits, codebook, fp32, stream};
-            return T <= 8 ? launch_gemv(la) : launch_gemm(la);
-        };
-        if (T <= 8) {
-            // gate and up in one launch, silu(g) * u formed inside the down projection
-            PairArgs pa{x, {shared[0].trellis, shared[1].trellis}, {shared[0].suh, shared[1].suh},
-                        {shared[0].svh, shared[1].svh}, {wsb + L.sg, wsb + L.su}, wsb + L.s_ahad, T, H, shared_I,
-                        k_bits, codebook, stream};
-            launch_gemv_pair(pa);
-            LinearArgs down{wsb + L.sg, shared[2].trellis, wsb + L.shared_out, shared[2].suh, wsb + L.s_ahad,
-                            shared[2].svh, T, shared_I, H, k_bits, codebook, 1, stream};
-            down.a_up = wsb + L.su;
-            launch_gemv(down);
-        } else {
-            dense(x, shared[0], wsb + L.sg, H, shared_I, 0);
-            dense(x, shared[1], wsb + L.su, H, shared_I, 0);
-            launch_silu_mul(wsb + L.sg, wsb + L.su, wsb + L.su, (int64_t)T * shared_I, 0.0f, stream);
-            dense(wsb + L.su, shared[2], wsb + L.shared_out, shared_I, H, 1);
-        }
-        shared_out = (const float*)(wsb + L.shared_out);
-        desc += " + shared expert";
+    if (!fold_combine) {
+        const size_t total = (size_t)T * H;
+        hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                           (const float*)(wsb + L.slot_out), shared_out, (const float*)w,
+                           (const int32_t*)(wsb + L.inv), (float*)out, T, H, k);
+        hip_ok(hipGetLastError(), "moe_combine_kernel launch");
+        desc += " + moe_combine_kernel";
     }
-
-    const size_t total = (size_t)T * H;
-    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
-                       (const float*)(wsb + L.slot_out), shared_out, (const float*)w,
-                       (const int32_t*)(wsb + L.inv), (float*)out, T, H, k);
-    hip_ok(hipGetLastError(), "moe_combine_kernel launch");
-    desc += " + moe_combine_kernel";
     if (idx_out) hip_ok(hipMemcpyAsync(idx_out, idx, (size_t)P * 4, hipMemcpyDeviceToDevice, stream), "idx copy");
     if (w_out) hip_ok(hipMemcpyAsync(w_out, w, (size_t)P * 4, hipMemcpyDeviceToDevice, stream), "w copy");
     g_moe_launch = desc;

@@ -140,6 +140,8 @@ def _check_stages(layer, x, experts_np, shared_np, idx, w, out, T, H, E, k, I, b
 
 @pytest.mark.parametrize("T,H,E,k,I,bits,shared_I,scale", [
     (1, 256, 8, 2, 128, 4, 0, 1.0),
+    (1, 256, 8, 2, 128, 4, 128, 1.0),       # one token, shared expert inside the grouped launches
+    (1, 384, 8, 3, 128, 4, 256, 1.0),       # one token, shared expert as dense launches
     (4, 256, 8, 3, 256, 4, 128, 1.0),
     (40, 256, 4, 2, 128, 4, 0, 1.0),        # about 20 rows per expert
     (70, 256, 6, 2, 128, 3, 128, 30.0),     # skewed routing: one expert with several 32-row chunks
@@ -223,6 +225,54 @@ def test_moe_config4_shape_zipf_shared():
     assert np.allclose(w.cpu().numpy(), ow, rtol=1e-5, atol=1e-7)
     _check_stages(layer, x, experts_np, shared_np, oi, w.cpu().numpy(), out.cpu().numpy(), T, H, E, k, I, bits, I)
     assert np.abs(out.cpu().numpy() - want).max() <= 2e-3 * np.abs(want).max()
+
+
+def _one_token_outputs():
+    """One token through three layers (no shared expert, shared expert of the routed
+    size, shared expert of another size), twice each: output bits and launch text."""
+    gpu = Gpu(0)
+    res = {}
+    for name, (H, E, k, I, bits, shared_I) in {"plain": (2048, 128, 8, 768, 4, 0), "folded": (512, 16, 4, 256, 3, 256),
+                                               "dense": (512, 16, 4, 256, 4, 384)}.items():
+        wr, _, experts, _, shared = _make_layer(gpu, 8100 + H + shared_I, H, E, I, bits, shared_I)
+        layer = MoeLayer(gpu, wr, experts, k, shared=shared)
+        outs = []
+        for rep in range(2):
+            x = (synth.activations(77 + rep, 1, H).astype(np.float32) / np.sqrt(H)).astype(np.float16)
+            out = torch.zeros((1, H), dtype=torch.float32, device=DEV)
+            layer.forward(gpu, dev(x.view(np.uint16)), out, 1)
+            torch.cuda.synchronize()
+            outs.append(out.cpu().numpy().view(np.uint32))
+        res[name] = np.stack(outs)
+        res[name + "_launch"] = np.array(K.moe.last_launch())
+    return res
+
+
+def test_moe_one_token_combine_inside_down_projection(tmp_path):
+    """With one token the last expert to finish a column block of the down projection
+    combines it; the result has the bits of the separate combine launch
+    (BERTH_MOE_FOLD_COMBINE=0, read once per process, so in a process of its own)."""
+    import os
+    import subprocess
+    import sys
+
+    here = _one_token_outputs()
+    for name in ("plain", "folded", "dense"):
+        launch = str(here[name + "_launch"])
+        assert "+combine" in launch and "moe_combine_kernel" not in launch, launch
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    path = str(tmp_path / "separate.npz")
+    code = ("import numpy as np, tests.test_gpu_moe as T\n"
+            f"np.savez({path!r}, **T._one_token_outputs())\nprint('ok')\n")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=600, cwd=root,
+                       env=dict(os.environ, BERTH_MOE_FOLD_COMBINE="0"))
+    assert r.returncode == 0 and "ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+    there = np.load(path)
+    for name in ("plain", "folded", "dense"):
+        launch = str(there[name + "_launch"])
+        assert "moe_combine_kernel" in launch and "+combine" not in launch, launch
+        assert np.array_equal(here[name], there[name]), name
+        assert here[name].any()
 
 
 def test_moe_layer_with_128_row_problems():
