@@ -64,39 +64,58 @@ std::string launch_gemm(const LinearArgs& a)
     // over the chip; narrow outputs (few column tiles) run as 32-row tiles instead
     const int nblocks = (a.size_n + 255) / 256;
     const long tiles128 = (long)nblocks * ((a.size_m + 127) / 128);
-    const int mb = (a.size_m <= 32 || tiles128 * 4 < ws.cu_count) ? 1 : 4;
-    const int mtiles = (a.size_m + mb * 32 - 1) / (mb * 32);
-    const long tiles = (long)nblocks * mtiles;
+    const int mb_plain = (a.size_m <= 32 || tiles128 * 4 < ws.cu_count) ? 1 : 4;
     const int KB = a.size_k / 128;
-    p.tiles_y = mtiles;
     std::string desc;
     p.tile0 = 0;
     static const int balance = [] {
         const char* e = std::getenv("BERTH_GEMM_BALANCED");
         return e ? std::atoi(e) : 1;
     }();
+    static const bool rows256 = [] {
+        const char* e = std::getenv("BERTH_GEMM_ROWS256");
+        return !e || std::atoi(e) != 0;
+    }();
     // 128-row tiles rarely divide over the compute units (272 tiles on 256 units leave most of
-    // the chip idle for the second half of the launch): deal the (tile, k-block) units out evenly
-    const long units = tiles * KB;
-    // one workgroup per compute unit, two when a workgroup still gets 16 k-blocks or more
-    // (measured on the 27B shapes at 512 rows: gate/up and down are fastest with two, q and o
-    // with one, where fewer workgroups share a tile)
-    long slots = units >= 32L * ws.cu_count ? 2L * ws.cu_count : ws.cu_count;
-    if (balance > 1) slots = balance;
-    const long G = units < slots ? units : slots;
-    const long per_wg = units / G;                                   // >= 1
-    const long parts = (KB + per_wg - 1) / per_wg + 1;               // workgroups that can share a tile
-    const size_t part_bytes = (size_t)4 * mb * 2 * 16 * 64 * sizeof(float);
-    if (balance && mb == 4 && tiles <= kCounters / 2 && per_wg < KB && units < (1L << 30) && (size_t)tiles * parts * part_bytes <= kPartialBytes) {
+    // the chip idle for the second half of the launch): deal the (tile, k-block) units out evenly.
+    // 128-row tiles: one workgroup per compute unit, two when a workgroup still gets 16 k-blocks
+    // or more (measured on the 27B shapes at 512 rows: gate/up and down are fastest with two, q
+    // and o with one, where fewer workgroups share a tile).  256-row tiles (more than 128 rows):
+    // a weight is decoded once per 256 rows; one workgroup of eight waves fills a compute unit.
+    auto balanced = [&](int mb) {
+        const int mtiles = (a.size_m + mb * 32 - 1) / (mb * 32);
+        const long tiles = (long)nblocks * mtiles;
+        const long units = tiles * KB;
+        long slots = (mb == 4 && units >= 32L * ws.cu_count) ? 2L * ws.cu_count : ws.cu_count;
+        if (balance > 1) slots = balance;
+        const long G = units < slots ? units : slots;
+        const long per_wg = units / G;                                   // >= 1
+        const long parts = (KB + per_wg - 1) / per_wg + 1;               // workgroups that can share a tile
+        const size_t part_bytes = (size_t)4 * mb * 2 * 16 * 64 * sizeof(float);
+        if (!(tiles <= kCounters / 2 && per_wg < KB && units < (1L << 30) &&
+              (size_t)tiles * parts * part_bytes <= kPartialBytes))
+            return false;
+        p.tiles_y = mtiles;
         p.S = 1;
         p.units = (int)units;
         p.unit_q = (int)(units / G);
         p.unit_r = (int)(units % G);
         p.max_parts = (int)parts;
         gemm_bits(p, a.k_bits, a.codebook, mb, a.stream, desc, dim3((unsigned)G, 1, 1));
-    } else {
-        p.S = gemm_split(ws, tiles, KB, mb);
-        gemm_bits(p, a.k_bits, a.codebook, mb, a.stream, desc, dim3((unsigned)(tiles * p.S), 1, 1));
+        return true;
+    };
+    bool done = false;
+    if (balance && mb_plain == 4) {
+        if (rows256 && a.size_m > 128) done = balanced(8);
+        if (!done) done = balanced(4);
+    }
+    if (!done) {
+        const int mtiles = (a.size_m + mb_plain * 32 - 1) / (mb_plain * 32);
+        const long tiles = (long)nblocks * mtiles;
+        p.tiles_y = mtiles;
+        p.units = 0;
+        p.S = gemm_split(ws, tiles, KB, mb_plain);
+        gemm_bits(p, a.k_bits, a.codebook, mb_plain, a.stream, desc, dim3((unsigned)(tiles * p.S), 1, 1));
     }
     hip_ok(hipGetLastError(), "exl3_gemm_kernel launch");
     return d0 + " + " + desc + (a.out_fp32 ? " out=f32" : " out=f16");

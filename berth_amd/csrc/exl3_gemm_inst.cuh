@@ -1,7 +1,8 @@
 // Per-codebook instantiations of the MFMA GEMM kernel (included by
 // exl3_gemm_cb{0,1,2}.hip with BERTH_GEMM_CB defined): 32-row and 128-row tiles for
-// every bit rate, and the balanced variant of the 128-row kernel.
+// every bit rate, the balanced variant of the 128-row kernel, and the 256-row kernel.
 #include "exl3_gemm_kernel.cuh"
+#include "exl3_gemm_wide_kernel.cuh"
 #include "launch.h"
 
 namespace berth {
@@ -38,10 +39,25 @@ static void gemm_launch_mb(const GemmParams& p, hipStream_t stream, std::string&
            " split_k=" + std::to_string(p.S) + " smem=" + std::to_string(smem);
 }
 
+// 256-row tiles (balanced dense launches only): eight waves, decoded weights shared through LDS
+template <int BITS, int CB>
+static void gemm_launch_wide(const GemmParams& p, hipStream_t stream, std::string& desc, dim3 grid)
+{
+    if (p.units <= 0) throw std::runtime_error("exl3 gemm: 256-row tiles exist only as balanced launches");
+    static const hipError_t attr = hipFuncSetAttribute((const void*)exl3_gemm_wide_kernel<BITS, CB>,
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kWideSmem);
+    hip_ok(attr, "exl3_gemm_wide_kernel shared-memory attribute");
+    hipLaunchKernelGGL((exl3_gemm_wide_kernel<BITS, CB>), grid, dim3(512), kWideSmem, stream, p);
+    desc = "exl3_gemm_wide_kernel<" + std::to_string(BITS) + "," + std::to_string(CB) + ",256x256> grid=" +
+           std::to_string(grid.x) + " units=" + std::to_string(p.units) + " max_parts=" + std::to_string(p.max_parts) +
+           " smem=" + std::to_string(kWideSmem);
+}
+
 template <int BITS, int CB>
 static void gemm_launch(const GemmParams& p, int mb, hipStream_t stream, std::string& desc, dim3 grid)
 {
     if (mb == 1) gemm_launch_mb<BITS, CB, 1>(p, stream, desc, grid);
+    else if (mb == 8) gemm_launch_wide<BITS, CB>(p, stream, desc, grid);
     else gemm_launch_mb<BITS, CB, 4>(p, stream, desc, grid);
 }
 

@@ -206,18 +206,49 @@ def test_gemm_split_k(m, Kk, N):
     assert np.array_equal(got.view(np.uint32), got2.view(np.uint32))
 
 
-@pytest.mark.parametrize("m,Kk,N,fp32", [(512, 1024, 4096, True), (384, 640, 5632, False), (200, 768, 8320, True),
-                                         (130, 256, 16384, False)])
-def test_gemm_128_row_tiles_dealt_out_evenly(m, Kk, N, fp32):
-    """Enough 128 x 256 tiles to use them: the (tile, k-block) units are cut into one equal
-    range per compute unit, tiles shared by several workgroups are summed in k order."""
-    got, want, ah, want_ah, launch = _run_linear(m, Kk, N, 4, 2, fp32, 700 + m, prefill=True)
-    assert "exl3_gemm_balanced_kernel<4,2,128x256>" in launch, launch
+def _check_balanced(m, Kk, N, fp32, tile, bits=4):
+    got, want, ah, want_ah, launch = _run_linear(m, Kk, N, bits, 2, fp32, 700 + m, prefill=True)
+    name = "exl3_gemm_wide_kernel" if tile == 256 else "exl3_gemm_balanced_kernel"
+    assert f"{name}<{bits},2,{tile}x256>" in launch, launch
     assert np.array_equal(ah, want_ah)
     bad, worst = close(got, want)
     assert bad == 0, (bad, worst, launch)
-    got2, _, _, _, _ = _run_linear(m, Kk, N, 4, 2, fp32, 700 + m, prefill=True)
+    got2, _, _, _, _ = _run_linear(m, Kk, N, bits, 2, fp32, 700 + m, prefill=True)
     assert np.array_equal(got.view(np.uint16), got2.view(np.uint16))
+
+
+@pytest.mark.parametrize("m,Kk,N,fp32", [(128, 1024, 16384, True), (100, 640, 16640, False), (65, 256, 17408, True)])
+def test_gemm_128_row_tiles_dealt_out_evenly(m, Kk, N, fp32):
+    """Enough 128 x 256 tiles to use them: the (tile, k-block) units are cut into one equal
+    range per compute unit, tiles shared by several workgroups are summed in k order."""
+    _check_balanced(m, Kk, N, fp32, 128)
+
+
+@pytest.mark.parametrize("m,Kk,N,fp32,bits", [(512, 1024, 4096, True, 4), (384, 640, 5632, False, 4),
+                                              (200, 768, 8320, True, 4), (130, 256, 16384, False, 4),
+                                              (300, 1024, 5632, True, 3), (640, 512, 4352, False, 5)])
+def test_gemm_256_row_tiles_dealt_out_evenly(m, Kk, N, fp32, bits):
+    """More than 128 rows: 256 x 256 tiles of eight waves; every weight is decoded once per
+    tile and reaches the MFMA waves through LDS.  Dealt out the same way.  The last tile may be
+    short (second row half with 72, 2 or no rows at all) or the only one; 8320 and 4352
+    columns leave half of the last column tile empty."""
+    _check_balanced(m, Kk, N, fp32, 256, bits)
+
+
+def test_gemm_128_row_tiles_for_more_than_128_rows():
+    """BERTH_GEMM_ROWS256=0 (read once per process) keeps 128-row tiles at any row count."""
+    import os
+    import subprocess
+    import sys
+    code = (
+        "import tests.test_gpu_linear as T\n"
+        "for m, K, N, f in ((512, 1024, 4096, True), (200, 768, 8320, False)):\n"
+        "    T._check_balanced(m, K, N, f, 128)\n"
+        "print('ok')\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=600, cwd=root,
+                       env=dict(os.environ, BERTH_GEMM_ROWS256="0"))
+    assert r.returncode == 0 and "ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
 
 
 def test_gemm_128_row_tiles_one_workgroup_per_tile_and_split():
