@@ -346,9 +346,35 @@ def prefill_bench(gpu, layers, bits: int, rows: int, steps: int):
         step(i)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
+
+    # Beside it: the vendor library's dense fp16 GEMM (torch.matmul) on already
+    # decoded fp16 weights of the same seven shapes.  It reads 4x the weight bytes
+    # and decodes nothing; it shows what a plain MFMA GEMM reaches at 512 rows of
+    # these shapes on this device, i.e. the practical ceiling for the fused kernel.
+    dense_us = 0.0
+    for n in ORDER:
+        Kk, N = synth.SHAPES_27B[n]
+        a = torch.randn((rows, Kk), device=gpu.device, dtype=torch.float16)
+        ws = [torch.randn((Kk, N), device=gpu.device, dtype=torch.float16) for _ in range(3)]
+        c = torch.empty((rows, N), device=gpu.device, dtype=torch.float16)
+        for i in range(3):
+            torch.matmul(a, ws[i], out=c)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(12):
+            torch.matmul(a, ws[i % 3], out=c)
+        e1.record()
+        torch.cuda.synchronize()
+        dense_us += e0.elapsed_time(e1) / 12 * 1e3
+        del a, ws, c
+    torch.cuda.empty_cache()
     return {"rows": rows, "ms_per_layer_set": round(dt * 1e3, 3), "tflops": round(flops / dt / 1e12, 1),
             "mfma_peak_tflops": 2500.0, "frac_of_fp16_mfma_peak": round(flops / dt / 2.5e15, 4),
-            "tokens_per_s": round(rows / dt, 0)}
+            "tokens_per_s": round(rows / dt, 0),
+            "vendor_dense_fp16_gemm": {"what": "torch.matmul on decoded fp16 weights, same shapes and rows",
+                                       "ms_per_layer_set": round(dense_us * 1e-3, 3),
+                                       "tflops": round(flops / dense_us / 1e6, 1)}}
 
 
 def main():

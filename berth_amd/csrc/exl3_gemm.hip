@@ -72,16 +72,18 @@ std::string launch_gemm(const LinearArgs& a)
         const char* e = std::getenv("BERTH_GEMM_BALANCED");
         return e ? std::atoi(e) : 1;
     }();
-    static const bool rows256 = [] {
+    // 0: never 256-row tiles; 1 (default): where they are faster; 2: wherever they are possible
+    static const int rows256 = [] {
         const char* e = std::getenv("BERTH_GEMM_ROWS256");
-        return !e || std::atoi(e) != 0;
+        return e ? std::atoi(e) : 1;
     }();
     // 128-row tiles rarely divide over the compute units (272 tiles on 256 units leave most of
     // the chip idle for the second half of the launch): deal the (tile, k-block) units out evenly.
     // 128-row tiles: one workgroup per compute unit, two when a workgroup still gets 16 k-blocks
     // or more (measured on the 27B shapes at 512 rows: gate/up and down are fastest with two, q
-    // and o with one, where fewer workgroups share a tile).  256-row tiles (more than 128 rows):
-    // a weight is decoded once per 256 rows; one workgroup of eight waves fills a compute unit.
+    // and o with one, where fewer workgroups share a tile).  256-row tiles (more than 128 rows,
+    // wide outputs): a weight is decoded once per 256 rows; one workgroup of eight waves fills a
+    // compute unit.
     auto balanced = [&](int mb) {
         const int mtiles = (a.size_m + mb * 32 - 1) / (mb * 32);
         const long tiles = (long)nblocks * mtiles;
@@ -106,7 +108,11 @@ std::string launch_gemm(const LinearArgs& a)
     };
     bool done = false;
     if (balance && mb_plain == 4) {
-        if (rows256 && a.size_m > 128) done = balanced(8);
+        // 256-row tiles pay when there are enough of them that few workgroups share a tile
+        // (measured at 512 rows: gate/up 5120x17408, 136 tiles, 148 -> 139 us; q, o and down
+        // with 40..48 tiles are 5 % slower than with 128-row tiles)
+        const long tiles256 = (long)nblocks * ((a.size_m + 255) / 256);
+        if (a.size_m > 128 && (rows256 >= 2 || (rows256 == 1 && tiles256 * 2 >= ws.cu_count))) done = balanced(8);
         if (!done) done = balanced(4);
     }
     if (!done) {

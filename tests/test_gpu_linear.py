@@ -224,15 +224,32 @@ def test_gemm_128_row_tiles_dealt_out_evenly(m, Kk, N, fp32):
     _check_balanced(m, Kk, N, fp32, 128)
 
 
-@pytest.mark.parametrize("m,Kk,N,fp32,bits", [(512, 1024, 4096, True, 4), (384, 640, 5632, False, 4),
-                                              (200, 768, 8320, True, 4), (130, 256, 16384, False, 4),
-                                              (300, 1024, 5632, True, 3), (640, 512, 4352, False, 5)])
+@pytest.mark.parametrize("m,Kk,N,fp32,bits", [(512, 512, 16384, True, 4), (300, 256, 16640, False, 4),
+                                              (640, 256, 11008, True, 3)])
 def test_gemm_256_row_tiles_dealt_out_evenly(m, Kk, N, fp32, bits):
-    """More than 128 rows: 256 x 256 tiles of eight waves; every weight is decoded once per
-    tile and reaches the MFMA waves through LDS.  Dealt out the same way.  The last tile may be
-    short (second row half with 72, 2 or no rows at all) or the only one; 8320 and 4352
-    columns leave half of the last column tile empty."""
+    """More than 128 rows and at least half as many 256 x 256 tiles as compute units: tiles
+    of eight waves; every weight is decoded once per tile and reaches the MFMA waves through
+    LDS.  Dealt out the same way.  The last row tile may be short (44 or 128 rows)."""
     _check_balanced(m, Kk, N, fp32, 256, bits)
+
+
+def test_gemm_256_row_tiles_on_narrow_outputs():
+    """BERTH_GEMM_ROWS256=2 (read once per process) takes 256-row tiles wherever they are
+    possible: short last tiles (second row half with 72, 2 or no rows at all), a single tile
+    row, 8320 and 4352 columns (half of the last column tile empty), 3 and 5 bpw."""
+    import os
+    import subprocess
+    import sys
+    code = (
+        "import tests.test_gpu_linear as T\n"
+        "for m, K, N, f, b in ((512, 1024, 4096, True, 4), (384, 640, 5632, False, 4), (200, 768, 8320, True, 4),\n"
+        "                      (130, 256, 16384, False, 4), (300, 1024, 5632, True, 3), (640, 512, 4352, False, 5)):\n"
+        "    T._check_balanced(m, K, N, f, 256, b)\n"
+        "print('ok')\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=600, cwd=root,
+                       env=dict(os.environ, BERTH_GEMM_ROWS256="2"))
+    assert r.returncode == 0 and "ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
 
 
 def test_gemm_128_row_tiles_for_more_than_128_rows():
