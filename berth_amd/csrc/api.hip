@@ -208,6 +208,37 @@ extern "C" int berth_prefill_reconstruct(void* unpacked, const void* packed, int
     }
 }
 
+extern "C" int berth_prefill_reconstruct_had(void* unpacked, const void* packed, const void* suh,
+                                             const void* svh, int size_k, int slice_n, int full_n,
+                                             int n_offset, int k_bits, int codebook, void* stream)
+{
+    try {
+        g_prefill_err.clear();
+        g_prefill_launch.clear();
+        if (!unpacked || !packed || !suh || !svh)
+            throw std::runtime_error("prefill reconstruct_had: null device pointer");
+        if (size_k < 128 || slice_n < 128 || full_n < 128)
+            throw std::runtime_error("prefill reconstruct_had: sizes must be positive");
+        if (k_bits < 1 || k_bits > 8) throw std::runtime_error("prefill reconstruct_had: K must be in 1..=8");
+        if (codebook < 0 || codebook > 2)
+            throw std::runtime_error("prefill reconstruct_had: codebook must be 0, 1, or 2");
+        if (size_k % 128) throw std::runtime_error("prefill reconstruct_had: K must be a multiple of 128");
+        if (slice_n % 128) throw std::runtime_error("prefill reconstruct_had: slice N must be a multiple of 128");
+        if (full_n % 16) throw std::runtime_error("prefill reconstruct_had: full N must be a multiple of 16");
+        if (n_offset % 128) throw std::runtime_error("prefill reconstruct_had: n_offset must be a multiple of 128");
+        if (n_offset < 0 || n_offset + slice_n > full_n)
+            throw std::runtime_error("prefill reconstruct_had: slice exceeds the trellis");
+        g_prefill_launch = launch_reconstruct_had(unpacked, packed, suh, svh, size_k, slice_n, full_n, n_offset,
+                                                  k_bits, codebook, (hipStream_t)stream);
+        return 0;
+    } catch (const std::exception& err) {
+        g_prefill_err = err.what();
+        g_prefill_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
 extern "C" int berth_prefill_had_r_128(const void* input, void* output, const void* scale,
                                        int pre_scale, int rows, int cols, int fp32, void* stream)
 {

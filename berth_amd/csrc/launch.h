@@ -114,6 +114,10 @@ std::string launch_gemm(const LinearArgs& args);
 std::string launch_reconstruct(void* unpacked, const void* packed, int size_k, int slice_n,
                                int full_n, int n_offset, int k_bits, int codebook,
                                hipStream_t stream);
+// trellis -> fp16 effective weight (both Hadamards and sign scales folded in)
+std::string launch_reconstruct_had(void* unpacked, const void* packed, const void* suh, const void* svh,
+                                   int size_k, int slice_n, int full_n, int n_offset, int k_bits, int codebook,
+                                   hipStream_t stream);
 // per row, per 128 columns: Hadamard with pre- or post-scale
 std::string launch_had_r_128(const void* in, void* out, const void* scale, int pre_scale,
                              int rows, int cols, int fp32, hipStream_t stream);

@@ -48,6 +48,7 @@ def load() -> C.CDLL:
         L.berth_prefill_exl3_linear.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
         L.berth_prefill_hgemm.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, vp]
         L.berth_prefill_reconstruct.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, vp]
+        L.berth_prefill_reconstruct_had.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
         L.berth_prefill_had_r_128.argtypes = [vp, vp, vp, ci, ci, ci, ci, vp]
         L.berth_ops_silu_mul.argtypes = [vp, vp, vp, C.c_int64, C.c_float, vp]
         L.berth_ops_rms_norm.argtypes = [vp, vp, vp, ci, ci, C.c_float, C.c_float, C.c_float, ci, vp]
@@ -156,6 +157,16 @@ class prefill_lin:
                                               k_bits, int(codebook), stream)
         if rc != 0:
             raise LaunchError(prefill_lin.last_error() or f"prefill reconstruct launch failed ({rc})")
+
+    @staticmethod
+    def reconstruct_had(unpacked, packed, suh, svh, size_k, slice_n, full_n, n_offset, k_bits,
+                        codebook: Codebook, stream=None) -> None:
+        """Columns n_offset.. of the effective weight diag(suh) Hh W Hh diag(svh) as fp16
+        [size_k][slice_n] (crates/berth-kernels/csrc/prefill_lin/reconstruct.cu:96-123)."""
+        rc = load().berth_prefill_reconstruct_had(unpacked, packed, suh, svh, size_k, slice_n, full_n, n_offset,
+                                                  k_bits, int(codebook), stream)
+        if rc != 0:
+            raise LaunchError(prefill_lin.last_error() or f"prefill reconstruct_had launch failed ({rc})")
 
     @staticmethod
     def had_r_128(inp, out, scale, pre_scale: bool, rows, cols, fp32: bool, stream=None) -> None:

@@ -63,15 +63,22 @@ int berth_prefill_hgemm(const void* a, const void* b, void* c, int size_m, int s
 const char* berth_prefill_last_error(void);
 const char* berth_prefill_last_launch(void);
 
-/* The reference keeps these two internal (C++ linkage,
- * crates/berth-kernels/csrc/prefill_lin/api.h, reconstruct.cu:31-93); they are
+/* The reference keeps these three internal (C++ linkage,
+ * crates/berth-kernels/csrc/prefill_lin/api.h, reconstruct.cu:31-123); they are
  * exported here because the dequantised weight is a parity target of its own.
  * reconstruct: unpacked fp16 [size_k][slice_n] = columns n_offset.. of the
- * decoded [size_k][full_n] inner weight.  had_r_128: per row and 128 columns,
- * out = Hh(in*scale) when pre_scale, else Hh(in)*scale; fp32 selects float
- * tensors. */
+ * decoded [size_k][full_n] inner weight.  reconstruct_had (reconstruct.cu:96-123,
+ * the reference's weight for 1024 rows and more): the same slice of the
+ * EFFECTIVE weight diag(suh) * Hh * W * Hh * diag(svh) per 128 x 128 block, so
+ * that a plain GEMM a @ unpacked is the operator's output; suh fp16 [size_k],
+ * svh fp16 [full_n] (the slice's part is taken at n_offset); size_k % 128 == 0.
+ * had_r_128: per row and 128 columns, out = Hh(in*scale) when pre_scale, else
+ * Hh(in)*scale; fp32 selects float tensors. */
 int berth_prefill_reconstruct(void* unpacked, const void* packed, int size_k, int slice_n,
                               int full_n, int n_offset, int k_bits, int codebook, void* stream);
+int berth_prefill_reconstruct_had(void* unpacked, const void* packed, const void* suh, const void* svh,
+                                  int size_k, int slice_n, int full_n, int n_offset, int k_bits,
+                                  int codebook, void* stream);
 int berth_prefill_had_r_128(const void* input, void* output, const void* scale, int pre_scale,
                             int rows, int cols, int fp32, void* stream);
 

@@ -239,6 +239,51 @@ int bo_had_rows_f32(const float* in, float* out, const uint16_t* scale,
     return 0;
 }
 
+/* Effective weight: both 128-block Hadamards and both sign scales folded into the decoded
+ * weight, per 128 x 128 block W_eff = diag(suh) Hh W Hh diag(svh)
+ * (crates/berth-kernels/csrc/prefill_lin/reconstruct.cu:96-123; the kernel body is in the
+ * absent fork, so the rounding contract is this build's: fp32 butterflies down the columns,
+ * then along the rows, ((v / sqrt(128)) / sqrt(128)) * suh[k] * svh[n], one rounding to
+ * fp16).  Pinned by the operator identity a @ W_eff == bo_linear(a). */
+int bo_reconstruct_had(const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh,
+                       int size_k, int size_n, int bits, int cb, uint16_t* w_out)
+{
+    if (size_k < 128 || size_n < 128 || size_k % 128 || size_n % 128) return -1;
+    uint16_t* w = (uint16_t*)malloc((size_t)size_k * size_n * 2);
+    if (!w) return -2;
+    int rc = bo_dequant(trellis, size_k, size_n, bits, cb, w);
+    if (rc) { free(w); return rc; }
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int kb = 0; kb < size_k / 128; ++kb) {
+        for (int nb = 0; nb < size_n / 128; ++nb) {
+            float* blk = (float*)malloc(128 * 128 * sizeof(float));
+            float v[128];
+            for (int k = 0; k < 128; ++k)
+                for (int n = 0; n < 128; ++n)
+                    blk[k * 128 + n] = bo_f16_to_f32(w[(size_t)(kb * 128 + k) * size_n + nb * 128 + n]);
+            for (int n = 0; n < 128; ++n) {
+                for (int k = 0; k < 128; ++k) v[k] = blk[k * 128 + n];
+                bo_had128(v);
+                for (int k = 0; k < 128; ++k) blk[k * 128 + n] = v[k];
+            }
+            for (int k = 0; k < 128; ++k) {
+                bo_had128(blk + k * 128);
+                float su = bo_f16_to_f32(suh[kb * 128 + k]);
+                for (int n = 0; n < 128; ++n) {
+                    float o = blk[k * 128 + n] * BO_RSQRT128;
+                    o = o * BO_RSQRT128;
+                    o = o * su;
+                    o = o * bo_f16_to_f32(svh[nb * 128 + n]);
+                    w_out[(size_t)(kb * 128 + k) * size_n + nb * 128 + n] = bo_f32_to_f16(o);
+                }
+            }
+            free(blk);
+        }
+    }
+    free(w);
+    return 0;
+}
+
 /* ---------------------------------------------------------------- linear */
 
 static void finish_rows(const float* z, void* c_out, const uint16_t* svh,

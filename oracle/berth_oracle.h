@@ -35,6 +35,10 @@
  *                        crates/berth-kernels/csrc/prefill_lin/reconstruct.cu:31-67;
  *                        Sylvester ordering [A]; pinned mathematically
  *                        (H*H = I, equals scipy.linalg.hadamard)
+ *   bo_reconstruct_had   launch contract [P] crates/berth-kernels/csrc/prefill_lin/
+ *                        reconstruct.cu:96-123 (kernel body in the absent fork);
+ *                        pinned by the operator identity a @ W_eff == bo_linear(a);
+ *                        rounding order [D] — parity unpinned
  *   bo_linear            [P] operator order crates/berth-kernels/csrc/prefill_lin/
  *                        linear.cu:198-220; pinned by the closed form
  *                        y = x @ diag(suh) Hh W Hh diag(svh)
@@ -69,6 +73,8 @@ uint16_t bo_decode_state(uint32_t state, int cb);
 /* trellis [K/16][N/16][16*bits] -> fp16 bits W[K][N] (the inner weight) */
 int bo_dequant(const uint16_t* trellis, int size_k, int size_n, int bits, int cb,
                uint16_t* w_out);
+int bo_reconstruct_had(const uint16_t* trellis, const uint16_t* suh, const uint16_t* svh,
+                       int size_k, int size_n, int bits, int cb, uint16_t* w_out);
 /* packed su/sv -> fp16 +-1 bit patterns; returns number of signs or -1 */
 long bo_unpack_signs(const uint8_t* packed_le, size_t nbytes, uint16_t* out);
 

@@ -93,6 +93,17 @@ def dequant(trellis, size_k: int, size_n: int, bits: int, cb: int) -> np.ndarray
     return out.view(np.float16)
 
 
+def reconstruct_had(trellis, suh, svh, size_k: int, size_n: int, bits: int, cb: int) -> np.ndarray:
+    """fp16 [size_k][size_n] effective weight diag(suh) Hh W Hh diag(svh)."""
+    tr = _u16(trellis)
+    assert tr.size == (size_k // 16) * (size_n // 16) * 16 * bits
+    out = np.empty((size_k, size_n), dtype=np.uint16)
+    rc = lib().bo_reconstruct_had(_p(tr), _p(_u16(suh)), _p(_u16(svh)), size_k, size_n, bits, cb, _p(out))
+    if rc:
+        raise ValueError("bo_reconstruct_had: bad shape")
+    return out.view(np.float16)
+
+
 def unpack_signs(packed: bytes) -> np.ndarray:
     buf = np.frombuffer(packed, dtype=np.uint8).copy()
     out = np.empty(max(1, len(packed) // 2 * 16), dtype=np.uint16)

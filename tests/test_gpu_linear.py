@@ -71,6 +71,45 @@ def test_dequant_full_size_config0_is_bit_exact():
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("Kk,N,bits,cb,n_offset,slice_n", [(256, 384, 4, 2, 0, None), (128, 128, 3, 2, 0, None),
+                                                          (384, 512, 4, 2, 128, 256), (256, 256, 5, 0, 0, None),
+                                                          (1024, 1280, 4, 2, 256, 1024), (128, 256, 2, 1, 128, 128)])
+def test_reconstruct_had_bit_exact(Kk, N, bits, cb, n_offset, slice_n):
+    """The effective weight diag(suh) Hh W Hh diag(svh) (the reference's weight for 1024 rows and
+    more, crates/berth-kernels/csrc/prefill_lin/reconstruct.cu:96-123), whole and as a column
+    slice, against the oracle: same butterfly order, one rounding, so the same bits."""
+    tr, suh, svh = synth.linear(77 + Kk + bits, Kk, N, bits)
+    slice_n = slice_n or N
+    d_tr, d_suh, d_svh = dev(tr), dev(suh.view(np.uint16)), dev(svh.view(np.uint16))
+    out = torch.zeros((Kk, slice_n), dtype=torch.float16, device=DEV)
+    K.prefill_lin.reconstruct_had(out.data_ptr(), d_tr.data_ptr(), d_suh.data_ptr(), d_svh.data_ptr(), Kk, slice_n, N,
+                                  n_offset, bits, Codebook(cb))
+    torch.cuda.synchronize()
+    assert "exl3_reconstruct_had_kernel" in K.prefill_lin.last_launch()
+    want = O.reconstruct_had(tr, suh, svh, Kk, N, bits, cb).view(np.uint16)
+    assert np.array_equal(host_u16(out), want[:, n_offset:n_offset + slice_n])
+
+
+def test_reconstruct_had_then_plain_gemm_is_the_operator():
+    """a @ W_eff through berth_prefill_hgemm against the fused linear of the same rows: the two
+    routes round in different places (W_eff to fp16 here, the rotated activation there), so the
+    bar is a relative one over the whole output."""
+    m, Kk, N, bits = 48, 512, 768, 4
+    tr, suh, svh = synth.linear(901, Kk, N, bits)
+    x = synth.activations(902, m, Kk)
+    d_tr, d_suh, d_svh, d_x = dev(tr), dev(suh.view(np.uint16)), dev(svh.view(np.uint16)), dev(x.view(np.uint16))
+    w_eff = torch.zeros((Kk, N), dtype=torch.float16, device=DEV)
+    K.prefill_lin.reconstruct_had(w_eff.data_ptr(), d_tr.data_ptr(), d_suh.data_ptr(), d_svh.data_ptr(), Kk, N, N, 0,
+                                  bits, Codebook.MUL1)
+    c = torch.zeros((m, N), dtype=torch.float32, device=DEV)
+    K.prefill_lin.hgemm(d_x.data_ptr(), w_eff.data_ptr(), c.data_ptr(), m, Kk, N, N, OutDtype.F32)
+    torch.cuda.synchronize()
+    want, _ = O.linear(x, tr, suh, svh, Kk, N, bits, 2, out_fp32=True)
+    got = c.cpu().numpy().astype(np.float64)
+    rel = np.linalg.norm(got - want) / np.linalg.norm(want)
+    assert rel < 5e-4, rel
+
+
 @pytest.mark.parametrize("pre", [True, False])
 @pytest.mark.parametrize("fp32", [False, True])
 def test_had_r_128_bit_exact(pre, fp32):
