@@ -63,9 +63,41 @@ def cpu_baseline(bits: int, seconds: float):
         if dt >= seconds:
             break
     nbytes = linear_bytes(K, N, bits, 1, 2) * reps
-    return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": O.num_threads(), "kind": "port",
-            "sample": f"{reps} x q_proj {K}x{N} {bits} bpw batch-1 decode-on-the-fly GEMV in {dt:.1f} s "
-                      f"({K * N * reps / dt / 1e6:.0f} M weights/s)"}
+    res = {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": O.num_threads(), "kind": "port",
+           "sample": f"{reps} x q_proj {K}x{N} {bits} bpw batch-1 decode-on-the-fly GEMV in {dt:.1f} s "
+                     f"({K * N * reps / dt / 1e6:.0f} M weights/s)"}
+
+    def timed(fn, budget):
+        fn()
+        n, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            n += 1
+            el = time.perf_counter() - t0
+            if el >= budget:
+                return el / n, n
+
+    # the other CPU figures of the same port, a few seconds each: BASELINE configs[0]
+    # (4096 x 4096, 4 bpw) as a GEMV and as a dequantisation, configs[3] at one token
+    k0 = 4096
+    tr0, suh0, svh0 = synth.linear(13, k0, k0, 4)
+    x0 = synth.activations(14, 1, k0)
+    t_gemv0, n_gemv0 = timed(lambda: O.gemv_fused(x0, tr0, suh0, svh0, k0, k0, 4, 2, out_fp32=False), 2.0)
+    t_deq, n_deq = timed(lambda: O.dequant(tr0, k0, k0, 4, 2), 2.0)
+    H, E, topk, I = 2048, 128, 8, 768
+    distinct = [tuple(synth.linear(2000 + 10 * e + 3 * j, *shape, 4) for j, shape in enumerate(((H, I), (H, I), (I, H))))
+                for e in range(8)]
+    experts = [distinct[e % 8] for e in range(E)]       # 8 distinct synthetic experts repeated: timing only
+    wr = synth.router_weight(15, H, E)
+    xm = synth.activations(16, 1, H)
+    t_moe, n_moe = timed(lambda: O.moe_layer(xm, wr, experts, topk, I, 4, 2), 3.0)
+    res["also"] = {
+        "config0_gemv_ms": round(t_gemv0 * 1e3, 3), "config0_gemv_GBps": round(linear_bytes(k0, k0, 4, 1, 2) / t_gemv0 / 1e9, 3),
+        "config0_dequant_Gweights_per_s": round(k0 * k0 / t_deq / 1e9, 3),
+        "moe_config3_one_token_us_per_token": round(t_moe * 1e6, 1),
+        "sample": f"{n_gemv0} GEMVs and {n_deq} dequantisations of 4096x4096 at 4 bpw, {n_moe} one-token MoE layers "
+                  f"(128 experts, top-8; 8 distinct synthetic experts repeated)"}
+    return res
 
 
 def moe_bench(gpu, steps: int, warmup: int):
