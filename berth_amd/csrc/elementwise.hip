@@ -6,31 +6,50 @@
 namespace berth {
 
 // crates/berth-kernels/csrc/prefill_lin/reconstruct.cu:31-67: per row and per
-// 128 columns, out = Hh(in * scale) (pre) or Hh(in) * scale (post).  One wave per
-// 128 block, four blocks per workgroup.
+// 128 columns, out = Hh(in * scale) (pre) or Hh(in) * scale (post).
 template <typename T, bool PRE>
 __global__ __launch_bounds__(256) void had_r_128_kernel(const T* __restrict__ in, T* __restrict__ out,
                                                         const _Float16* __restrict__ scale,
                                                         long blocks, int col_blocks)
 {
+    // sixteen lanes per 128 block, eight consecutive elements per lane (one or two 16-byte
+    // accesses): a wave takes four neighbouring blocks at a time and strides over the tensor
+    typedef T vec8_t __attribute__((ext_vector_type(8)));
     const int lane = threadIdx.x & 63;
-    const long blk = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (blk >= blocks) return;
-    const int cb = (int)(blk % col_blocks);
-    const size_t at = (size_t)blk * 128 + 2 * lane;
-    float v0 = (float)in[at], v1 = (float)in[at + 1];
-    float s0 = 1.0f, s1 = 1.0f;
-    if (scale) {
-        s0 = (float)scale[cb * 128 + 2 * lane];
-        s1 = (float)scale[cb * 128 + 2 * lane + 1];
+    const int l16 = lane & 15;
+    const long waves = (long)gridDim.x * 4;
+    const long groups = (blocks + 3) / 4;
+    for (long g = (long)blockIdx.x * 4 + (threadIdx.x >> 6); g < groups; g += waves) {
+        const long blk = g * 4 + (lane >> 4);
+        const bool live = blk < blocks;
+        const long b = live ? blk : blocks - 1;             // lanes past the end redo the last block and store nothing
+        const int cb = (int)(b % col_blocks);
+        const size_t at = (size_t)b * 128 + 8 * l16;
+        const vec8_t x = *(const vec8_t*)(in + at);
+        float v[8], sc[8];
+        if (scale) {
+            const half8_t s8 = *(const half8_t*)(scale + cb * 128 + 8 * l16);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sc[i] = (float)s8[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sc[i] = 1.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            v[i] = (float)x[i];
+            if (PRE) v[i] *= sc[i];
+        }
+        had128_row16(v, lane);
+        vec8_t o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float r = v[i] * kRsqrt128;
+            if (!PRE) r *= sc[i];
+            o[i] = (T)r;
+        }
+        if (live) *(vec8_t*)(out + at) = o;
     }
-    if (PRE) { v0 *= s0; v1 *= s1; }
-    had128_wave(v0, v1, lane);
-    v0 *= kRsqrt128;
-    v1 *= kRsqrt128;
-    if (!PRE) { v0 *= s0; v1 *= s1; }
-    out[at] = (T)v0;
-    out[at + 1] = (T)v1;
 }
 
 std::string launch_had_r_128(const void* in, void* out, const void* scale, int pre_scale,
@@ -38,7 +57,8 @@ std::string launch_had_r_128(const void* in, void* out, const void* scale, int p
 {
     const int col_blocks = cols / 128;
     const long blocks = (long)rows * col_blocks;
-    const dim3 grid((unsigned)((blocks + 3) / 4));
+    const long wgs = (blocks + 15) / 16;                    // four blocks per wave, four waves per workgroup
+    const dim3 grid((unsigned)(wgs < 4096 ? wgs : 4096));
     const _Float16* sc = (const _Float16*)scale;
     if (fp32) {
         if (pre_scale) hipLaunchKernelGGL((had_r_128_kernel<float, true>), grid, dim3(256), 0, stream, (const float*)in, (float*)out, sc, blocks, col_blocks);
