@@ -339,15 +339,27 @@ __global__ __launch_bounds__(1024) void moe_route_one_token_kernel(RouteParams p
 // token group.  First launch: partial sums of kRouteBigTT tokens x one 64-row
 // segment; second launch: one workgroup per token adds the segments in order,
 // adds the bias and selects.
-constexpr int kRouteBigTT = 16;
+constexpr int kRouteBigTT = 4;      // tokens per thread of the first launch
 constexpr int kRouteBigT = 32;      // calls with at least this many tokens take the two-launch path
+
+// How the 256 threads of a first-launch workgroup are used: `lanes` threads cover the expert
+// pairs (64, 128 or 256: a router of up to 128 experts needs one wave), and 256 / lanes token
+// subgroups of kRouteBigTT tokens sit side by side, so a small router does not leave three
+// waves of four idle.  More than 512 experts: a thread walks pairs tid, tid + 256, ...
+inline __host__ __device__ int route_big_lanes(int E)
+{
+    const int pairs = (E + 1) >> 1;
+    return pairs <= 64 ? 64 : (pairs <= 128 ? 128 : 256);
+}
+inline __host__ __device__ int route_big_group(int E) { return kRouteBigTT * (256 / route_big_lanes(E)); }
 
 // partial sums of kRouteBigTT tokens x two neighbouring experts over one segment.
 // EVEN: the expert count is even, so the pair is one aligned 4-byte load per row.
 // Eight rows of the router weight are loaded back to back (no branch in between:
 // the loads are what the loop waits for); the fma chains stay in row order.
+// xs: this thread's tokens, [row][kRouteBigTT] with row stride `xs_stride` floats.
 template <bool EVEN>
-__device__ __forceinline__ void route_pair_segment(const RouteParams& p, const float (*xs)[kRouteBigTT], int e0,
+__device__ __forceinline__ void route_pair_segment(const RouteParams& p, const float* xs, int xs_stride, int e0,
                                                    int h0, int hn, float (&part)[2][kRouteBigTT])
 {
     const bool two = e0 + 1 < p.E;
@@ -382,7 +394,7 @@ __device__ __forceinline__ void route_pair_segment(const RouteParams& p, const f
         for (int i = 0; i < 8; ++i) {
             // rows past the segment hold zeros in xs: they add +-0 to the partial sum, and
             // the sign of a zero partial sum never reaches a logit (0 + partial comes first)
-            const float4_t* xrow = (const float4_t*)&xs[hb + i][0];
+            const float4_t* xrow = (const float4_t*)(xs + (size_t)(hb + i) * xs_stride);
 #pragma unroll
             for (int q = 0; q < kRouteBigTT / 4; ++q) {
                 const float4_t xv = xrow[q];
@@ -398,13 +410,16 @@ __device__ __forceinline__ void route_pair_segment(const RouteParams& p, const f
 
 __global__ __launch_bounds__(256) void moe_route_partial_kernel(RouteParams p)
 {
-    __shared__ __align__(16) float xs[kRouteSeg][kRouteBigTT];      // [row][token]: one b128 read per 4 tokens
+    constexpr int kMaxGroup = kRouteBigTT * 4;
+    __shared__ __align__(16) float xs[kRouteSeg][kMaxGroup];        // [row][token]: one b128 read per 4 tokens
+    const int lanes = route_big_lanes(p.E);
+    const int group = kRouteBigTT * (256 / lanes);                  // tokens of this workgroup
     const int seg = blockIdx.x, grp = blockIdx.y;
-    const int t0 = grp * kRouteBigTT;
+    const int t0 = grp * group;
     const int h0 = seg * kRouteSeg;
     const int hn = min(kRouteSeg, p.H - h0);
     const int tid = threadIdx.x;
-    for (int i = tid; i < kRouteBigTT * kRouteSeg; i += 256) {
+    for (int i = tid; i < group * kRouteSeg; i += 256) {
         const int tt = i / kRouteSeg, h = i % kRouteSeg;
         float v = 0.0f;
         if (t0 + tt < p.T && h < hn) v = (float)p.x[(size_t)(t0 + tt) * p.H + h0 + h];
@@ -412,17 +427,19 @@ __global__ __launch_bounds__(256) void moe_route_partial_kernel(RouteParams p)
     }
     __syncthreads();
     const bool even = (p.E & 1) == 0;
-    for (int e0 = 2 * tid; e0 < p.E; e0 += 512) {
+    const int sub = tid / lanes;                                    // token subgroup of this thread
+    const int ts = t0 + sub * kRouteBigTT;
+    for (int e0 = 2 * (tid % lanes); e0 < p.E; e0 += 2 * lanes) {
         float part[2][kRouteBigTT];
 #pragma unroll
         for (int tt = 0; tt < kRouteBigTT; ++tt) part[0][tt] = part[1][tt] = 0.0f;
-        if (even) route_pair_segment<true>(p, xs, e0, h0, hn, part);
-        else route_pair_segment<false>(p, xs, e0, h0, hn, part);
+        if (even) route_pair_segment<true>(p, &xs[0][sub * kRouteBigTT], kMaxGroup, e0, h0, hn, part);
+        else route_pair_segment<false>(p, &xs[0][sub * kRouteBigTT], kMaxGroup, e0, h0, hn, part);
         const bool two = e0 + 1 < p.E;
 #pragma unroll
         for (int tt = 0; tt < kRouteBigTT; ++tt) {
-            if (t0 + tt < p.T) {
-                float* dst = p.parts + ((size_t)(t0 + tt) * p.nseg + seg) * p.E + e0;
+            if (ts + tt < p.T) {
+                float* dst = p.parts + ((size_t)(ts + tt) * p.nseg + seg) * p.E + e0;
                 dst[0] = part[0][tt];
                 if (two) dst[1] = part[1][tt];
             }
@@ -611,25 +628,33 @@ __global__ __launch_bounds__(256) void moe_had_rows_kernel(HadRowsParams p)
     const ExpertLin lin = ex == p.shared_expert ? p.shared[p.lin_base + which]
                                                 : p.experts[ex * p.lins_per_expert + p.lin_base + which];
     const int src = p.gather ? p.gather[r] / p.gather_div : r;
-    const half2_t* xrow = (const half2_t*)(p.a + (size_t)src * p.K);
-    const half2_t* urow = p.a_up ? (const half2_t*)(p.a_up + (size_t)src * p.K) : nullptr;
-    const half2_t* srow = (const half2_t*)lin.suh;
-    half2_t* orow = (half2_t*)(p.out[which] + (size_t)r * p.K);
-    for (int kb = wave; kb * 128 < p.K; kb += 4) {
-        half2_t x = xrow[kb * 64 + lane];
+    const _Float16* xrow = p.a + (size_t)src * p.K;
+    const _Float16* urow = p.a_up ? p.a_up + (size_t)src * p.K : nullptr;
+    const _Float16* srow = lin.suh;
+    _Float16* orow = p.out[which] + (size_t)r * p.K;
+    // sixteen lanes per 128 block, eight consecutive elements per lane (16-byte accesses): the
+    // workgroup rotates sixteen blocks at a time
+    const int l16 = lane & 15;
+    const int nkb = p.K >> 7;
+    for (int kb0 = 0; kb0 < nkb; kb0 += 16) {
+        const int kb = kb0 + wave * 4 + (lane >> 4);
+        const bool live = kb < nkb;
+        const int at = (live ? kb : nkb - 1) * 128 + 8 * l16;   // lanes past the end redo the last block, store nothing
+        half8_t x = *(const half8_t*)(xrow + at);
         if (urow) {
-            const half2_t u = urow[kb * 64 + lane];
-            x.x = silu_mul_h(x.x, u.x);
-            x.y = silu_mul_h(x.y, u.y);
+            const half8_t u = *(const half8_t*)(urow + at);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[i] = silu_mul_h(x[i], u[i]);
         }
-        const half2_t sc = srow[kb * 64 + lane];
-        float v0 = (float)x.x * (float)sc.x;
-        float v1 = (float)x.y * (float)sc.y;
-        had128_wave(v0, v1, lane);
-        half2_t o;
-        o.x = (_Float16)(v0 * kRsqrt128);
-        o.y = (_Float16)(v1 * kRsqrt128);
-        orow[kb * 64 + lane] = o;
+        const half8_t sc = *(const half8_t*)(srow + at);
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (float)x[i] * (float)sc[i];
+        had128_row16(v, lane);
+        half8_t o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = (_Float16)(v[i] * kRsqrt128);
+        if (live) *(half8_t*)(orow + at) = o;
     }
 }
 
@@ -771,7 +796,8 @@ std::string run_route(const void* x, const void* wr, const float* bias, int32_t*
     const int groups = (T + kRouteTT - 1) / kRouteTT;
     if (groups > kCounters) throw std::runtime_error("moe route: too many tokens for the counter table");
     if (T >= kRouteBigT) {
-        dim3 grid(p.nseg, (T + kRouteBigTT - 1) / kRouteBigTT);
+        const int group = route_big_group(E);
+        dim3 grid(p.nseg, (T + group - 1) / group);
         hipLaunchKernelGGL(moe_route_partial_kernel, grid, dim3(256), 0, stream, p);
         hip_ok(hipGetLastError(), "moe_route_partial_kernel launch");
         hipLaunchKernelGGL(moe_route_finish_kernel, dim3(T), dim3(256), 0, stream, p);
