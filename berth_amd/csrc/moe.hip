@@ -336,31 +336,34 @@ __global__ __launch_bounds__(1024) void moe_route_one_token_kernel(RouteParams p
 
 // Many tokens: the same arithmetic in two launches, so that the segment sums of a
 // token are added by a workgroup of its own instead of the last workgroup of a
-// token group.  First launch: partial sums of kRouteBigTT tokens x one 64-row
+// token group.  First launch: partial sums of a few tokens x one 64-row
 // segment; second launch: one workgroup per token adds the segments in order,
 // adds the bias and selects.
-constexpr int kRouteBigTT = 4;      // tokens per thread of the first launch
+constexpr int kRouteBigGroup = 16;  // most tokens a first-launch workgroup takes
 constexpr int kRouteBigT = 32;      // calls with at least this many tokens take the two-launch path
 
 // How the 256 threads of a first-launch workgroup are used: `lanes` threads cover the expert
 // pairs (64, 128 or 256: a router of up to 128 experts needs one wave), and 256 / lanes token
-// subgroups of kRouteBigTT tokens sit side by side, so a small router does not leave three
-// waves of four idle.  More than 512 experts: a thread walks pairs tid, tid + 256, ...
+// subgroups sit side by side, so a small router does not leave three waves of four idle.  A
+// thread takes four tokens, or eight when all 256 threads are on expert pairs (a wide router:
+// fewer workgroups re-read its rows).  More than 512 experts: a thread walks pairs tid,
+// tid + 256, ...
 inline __host__ __device__ int route_big_lanes(int E)
 {
     const int pairs = (E + 1) >> 1;
     return pairs <= 64 ? 64 : (pairs <= 128 ? 128 : 256);
 }
-inline __host__ __device__ int route_big_group(int E) { return kRouteBigTT * (256 / route_big_lanes(E)); }
+inline __host__ __device__ int route_big_tokens(int E) { return route_big_lanes(E) == 256 ? 8 : 4; }
+inline __host__ __device__ int route_big_group(int E) { return route_big_tokens(E) * (256 / route_big_lanes(E)); }
 
-// partial sums of kRouteBigTT tokens x two neighbouring experts over one segment.
+// partial sums of TT tokens x two neighbouring experts over one segment.
 // EVEN: the expert count is even, so the pair is one aligned 4-byte load per row.
 // Eight rows of the router weight are loaded back to back (no branch in between:
 // the loads are what the loop waits for); the fma chains stay in row order.
-// xs: this thread's tokens, [row][kRouteBigTT] with row stride `xs_stride` floats.
-template <bool EVEN>
+// xs: this thread's tokens, [row][TT] with row stride `xs_stride` floats.
+template <bool EVEN, int TT>
 __device__ __forceinline__ void route_pair_segment(const RouteParams& p, const float* xs, int xs_stride, int e0,
-                                                   int h0, int hn, float (&part)[2][kRouteBigTT])
+                                                   int h0, int hn, float (&part)[2][TT])
 {
     const bool two = e0 + 1 < p.E;
     const _Float16* wcol = p.wr + (size_t)h0 * p.E + e0;
@@ -396,7 +399,7 @@ __device__ __forceinline__ void route_pair_segment(const RouteParams& p, const f
             // the sign of a zero partial sum never reaches a logit (0 + partial comes first)
             const float4_t* xrow = (const float4_t*)(xs + (size_t)(hb + i) * xs_stride);
 #pragma unroll
-            for (int q = 0; q < kRouteBigTT / 4; ++q) {
+            for (int q = 0; q < TT / 4; ++q) {
                 const float4_t xv = xrow[q];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -408,12 +411,12 @@ __device__ __forceinline__ void route_pair_segment(const RouteParams& p, const f
     }
 }
 
+template <int TT>
 __global__ __launch_bounds__(256) void moe_route_partial_kernel(RouteParams p)
 {
-    constexpr int kMaxGroup = kRouteBigTT * 4;
-    __shared__ __align__(16) float xs[kRouteSeg][kMaxGroup];        // [row][token]: one b128 read per 4 tokens
+    __shared__ __align__(16) float xs[kRouteSeg][kRouteBigGroup];   // [row][token]: one b128 read per 4 tokens
     const int lanes = route_big_lanes(p.E);
-    const int group = kRouteBigTT * (256 / lanes);                  // tokens of this workgroup
+    const int group = TT * (256 / lanes);                           // tokens of this workgroup
     const int seg = blockIdx.x, grp = blockIdx.y;
     const int t0 = grp * group;
     const int h0 = seg * kRouteSeg;
@@ -428,16 +431,16 @@ __global__ __launch_bounds__(256) void moe_route_partial_kernel(RouteParams p)
     __syncthreads();
     const bool even = (p.E & 1) == 0;
     const int sub = tid / lanes;                                    // token subgroup of this thread
-    const int ts = t0 + sub * kRouteBigTT;
+    const int ts = t0 + sub * TT;
     for (int e0 = 2 * (tid % lanes); e0 < p.E; e0 += 2 * lanes) {
-        float part[2][kRouteBigTT];
+        float part[2][TT];
 #pragma unroll
-        for (int tt = 0; tt < kRouteBigTT; ++tt) part[0][tt] = part[1][tt] = 0.0f;
-        if (even) route_pair_segment<true>(p, &xs[0][sub * kRouteBigTT], kMaxGroup, e0, h0, hn, part);
-        else route_pair_segment<false>(p, &xs[0][sub * kRouteBigTT], kMaxGroup, e0, h0, hn, part);
+        for (int tt = 0; tt < TT; ++tt) part[0][tt] = part[1][tt] = 0.0f;
+        if (even) route_pair_segment<true, TT>(p, &xs[0][sub * TT], kRouteBigGroup, e0, h0, hn, part);
+        else route_pair_segment<false, TT>(p, &xs[0][sub * TT], kRouteBigGroup, e0, h0, hn, part);
         const bool two = e0 + 1 < p.E;
 #pragma unroll
-        for (int tt = 0; tt < kRouteBigTT; ++tt) {
+        for (int tt = 0; tt < TT; ++tt) {
             if (ts + tt < p.T) {
                 float* dst = p.parts + ((size_t)(ts + tt) * p.nseg + seg) * p.E + e0;
                 dst[0] = part[0][tt];
@@ -798,7 +801,8 @@ std::string run_route(const void* x, const void* wr, const float* bias, int32_t*
     if (T >= kRouteBigT) {
         const int group = route_big_group(E);
         dim3 grid(p.nseg, (T + group - 1) / group);
-        hipLaunchKernelGGL(moe_route_partial_kernel, grid, dim3(256), 0, stream, p);
+        if (route_big_tokens(E) == 8) hipLaunchKernelGGL(moe_route_partial_kernel<8>, grid, dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL(moe_route_partial_kernel<4>, grid, dim3(256), 0, stream, p);
         hip_ok(hipGetLastError(), "moe_route_partial_kernel launch");
         hipLaunchKernelGGL(moe_route_finish_kernel, dim3(T), dim3(256), 0, stream, p);
         hip_ok(hipGetLastError(), "moe_route_finish_kernel launch");
