@@ -48,6 +48,14 @@ template <typename T>
 __device__ __forceinline__ global_ptr<T> as_global(T* p) { return (global_ptr<T>)p; }
 #endif
 
+// A workgroup that is about to tell another workgroup, through an agent-scope counter, that
+// its stores are there: every wave first waits until its own stores have completed.  The
+// workgroup-scope release fence does not do that (the waves of a workgroup share their
+// caches, so the compiler emits no wait on vector memory for it), and neither does a barrier.
+#ifndef BERTH_HOST_EMU
+__device__ __forceinline__ void wait_own_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+#endif
+
 __device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
 __device__ __forceinline__ uint32_t as_u32(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
 

@@ -234,6 +234,7 @@ __device__ __forceinline__ void gemm_tile_wide(const GemmParams& p, const int ti
             }
         }
         if (!finisher) {
+            wait_own_stores();
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
             __syncthreads();
             if (threadIdx.x == 0) __hip_atomic_fetch_add(written, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

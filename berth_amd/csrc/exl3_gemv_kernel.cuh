@@ -341,8 +341,8 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
         // The partial sums travel as agent-scope atomic stores and loads, which go
         // straight to the level of the memory hierarchy all compute dies share, so
         // no cache-wide write-back or invalidate is needed: it is enough that this
-        // workgroup's stores have completed (the workgroup-scope release waits for
-        // them) before the arrival counter is bumped.
+        // workgroup's stores have completed (every wave waits for its own) before the
+        // arrival counter is bumped.
         float* mine = p.partials + ((size_t)((size_t)unit * p.S + s) * MMAX) * 128;
         if (t < 128) {
 #pragma unroll
@@ -350,6 +350,7 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
                 if (MMAX == 1 || m < rows)
                     __hip_atomic_store(mine + m * 128 + t, z[m], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+        wait_own_stores();
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (t == 0) {

@@ -225,6 +225,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(RouteParams p)
                 __hip_atomic_store(p.parts + ((size_t)(t0 + tt) * p.nseg + seg) * p.E + e, part[tt],
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    wait_own_stores();
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     if (tid == 0) {
