@@ -25,8 +25,9 @@ TOKENS = [1, 1, 2, 3, 7, 8, 9, 16, 31, 32, 33, 64, 100, 130]
 
 
 def _cases():
-    """BERTH_SWEEP_REPEATS (default 1) passes over the token counts, each with fresh shapes."""
-    rng = np.random.default_rng(77031)
+    """BERTH_SWEEP_REPEATS (default 1) passes over the token counts, each with fresh shapes;
+    BERTH_SWEEP_SEED shifts the seed."""
+    rng = np.random.default_rng(77031 + int(os.environ.get("BERTH_SWEEP_SEED", "0")))
     out = []
     for T in TOKENS * int(os.environ.get("BERTH_SWEEP_REPEATS", "1")):
         H = 128 * int(rng.integers(1, 7))

@@ -17,8 +17,9 @@ ROWS = [1, 2, 7, 8, 9, 31, 32, 33, 64, 100, 127, 128, 129, 144, 145, 255, 256, 2
 
 
 def _cases():
-    """BERTH_SWEEP_REPEATS (default 2) passes over the row counts, each with fresh shapes."""
-    rng = np.random.default_rng(20251)
+    """BERTH_SWEEP_REPEATS (default 2) passes over the row counts, each with fresh shapes;
+    BERTH_SWEEP_SEED shifts the seed."""
+    rng = np.random.default_rng(20251 + int(os.environ.get("BERTH_SWEEP_SEED", "0")))
     out = []
     for i, m in enumerate(ROWS * int(os.environ.get("BERTH_SWEEP_REPEATS", "2"))):
         Kk = 128 * int(rng.integers(1, 13))
