@@ -134,6 +134,31 @@ def test_had_r_128_bit_exact(pre, fp32):
         assert np.array_equal(host_u16(d_o), want)
 
 
+@pytest.mark.parametrize("rows,cols", [(1, 128), (3, 256), (7, 640), (33, 1152), (700, 12032), (513, 17408)])
+def test_had_r_128_ragged_sizes_bit_exact(rows, cols):
+    """Block counts that are not multiples of the four blocks a wave takes, and tensors with
+    more blocks than one pass of the grid covers (the kernel strides over them); in place too."""
+    sc = synth.sign_scale(rows + cols, cols)
+    x16 = synth.activations(rows * 3 + cols, rows, cols)
+    d_sc = dev(sc.view(np.uint16))
+    for pre in (True, False):
+        d_x = dev(x16.view(np.uint16))
+        d_o = torch.zeros_like(d_x)
+        K.prefill_lin.had_r_128(d_x.data_ptr(), d_o.data_ptr(), d_sc.data_ptr(), pre, rows, cols, False)
+        torch.cuda.synchronize()
+        want = O.had_rows_f16(x16, sc, pre).view(np.uint16)
+        assert np.array_equal(host_u16(d_o).reshape(rows, cols), want)
+        K.prefill_lin.had_r_128(d_x.data_ptr(), d_x.data_ptr(), d_sc.data_ptr(), pre, rows, cols, False)   # in place
+        torch.cuda.synchronize()
+        assert np.array_equal(host_u16(d_x).reshape(rows, cols), want)
+    x32 = (x16.astype(np.float32) * 1.7).astype(np.float32)
+    d_x = torch.from_numpy(x32).to(DEV)
+    d_o = torch.zeros_like(d_x)
+    K.prefill_lin.had_r_128(d_x.data_ptr(), d_o.data_ptr(), d_sc.data_ptr(), False, rows, cols, True)
+    torch.cuda.synchronize()
+    assert np.array_equal(d_o.cpu().numpy().view(np.uint32), O.had_rows_f32(x32, sc, False).view(np.uint32))
+
+
 def test_silu_mul_reference_fixture_bit_exact(golden_dir):
     g = np.fromfile(os.path.join(golden_dir, "silu.gate.bin"), dtype=np.uint16)
     u = np.fromfile(os.path.join(golden_dir, "silu.up.bin"), dtype=np.uint16)
