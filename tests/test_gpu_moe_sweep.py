@@ -65,3 +65,43 @@ def test_moe_layer_ragged_configurations(T, H, E, k, I, bits, shared_I, skew):
     layer.forward(gpu, d_x, out2, T)
     torch.cuda.synchronize()
     assert np.array_equal(out2.cpu().numpy().view(np.uint32), out.cpu().numpy().view(np.uint32))
+
+
+def _route_cases():
+    rng = np.random.default_rng(8812 + int(os.environ.get("BERTH_SWEEP_SEED", "0")))
+    out = []
+    for T in [1, 1, 2, 5, 8, 9, 31, 32, 33, 70, 256, 300] * int(os.environ.get("BERTH_SWEEP_REPEATS", "1")):
+        E = int(rng.choice([int(rng.integers(1, 130)), int(rng.integers(130, 1025))]))
+        k = int(rng.integers(1, min(E, 32) + 1))
+        H = int(rng.choice([64 * int(rng.integers(1, 40)), int(rng.integers(1, 2500))]))
+        out.append((T, H, E, k, bool(rng.integers(0, 2)), bool(rng.integers(0, 2))))
+    return out
+
+
+@pytest.mark.parametrize("T,H,E,k,with_bias,renorm", _route_cases())
+def test_route_and_permute_ragged(T, H, E, k, with_bias, renorm):
+    """Router shapes from one expert to 1024, top-k up to 32, hidden sizes that are not
+    multiples of the 64-row segment: logits and top-k bit-exact; then the permutation of the
+    selection against the oracle's stable counting sort."""
+    from berth_amd import kernels as K
+    from tests.test_gpu_moe import _route
+    x = synth.activations(T + H + E, T, H)
+    wr = synth.router_weight(E + H, H, E)
+    bias = synth.zipf_bias(E + 1, E) if with_bias else None
+    idx, w, logits = _route(x, wr, k, bias=bias, renorm=renorm)
+    oi, ow, ol = O.moe_route(x, wr, k, bias=bias, renorm=renorm, want_logits=True)
+    assert np.array_equal(logits.view(np.uint32), ol.view(np.uint32))
+    assert np.array_equal(idx, oi)
+    assert np.allclose(w, ow, rtol=1e-5, atol=1e-7)
+    if T * k <= 65535:
+        d_idx = torch.from_numpy(idx).to(DEV)
+        off = torch.zeros(E + 1, dtype=torch.int32, device=DEV)
+        perm = torch.zeros(T * k, dtype=torch.int32, device=DEV)
+        inv = torch.zeros(T * k, dtype=torch.int32, device=DEV)
+        scratch = torch.zeros(K.moe.permute_scratch_bytes(T, k, E), dtype=torch.uint8, device=DEV)
+        K.moe.permute(d_idx.data_ptr(), off.data_ptr(), perm.data_ptr(), inv.data_ptr(), scratch.data_ptr(), T, k, E)
+        torch.cuda.synchronize()
+        ooff, operm = O.moe_permute(idx, E)
+        assert np.array_equal(off.cpu().numpy(), ooff)
+        assert np.array_equal(perm.cpu().numpy(), operm)
+        assert np.array_equal(inv.cpu().numpy()[operm], np.arange(T * k))
