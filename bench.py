@@ -139,9 +139,35 @@ def moe_bench(gpu, steps: int, warmup: int):
             layers[i % 2].forward(gpu, xs[i % 16], out, T)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
+        eager_us = dt / steps * 1e6
+        launch = "eager"
+        # the same 16 calls recorded once into a HIP graph and replayed (the library's launches
+        # keep no host state between calls, so a recorded layer replays bit for bit)
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream(device=gpu.device)
+        side.wait_stream(torch.cuda.current_stream(gpu.device))
+        with torch.cuda.stream(side):
+            for i in range(16):
+                layers[i % 2].forward(gpu, xs[i], out, T)
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(16):
+                    layers[i % 2].forward(gpu, xs[i], out, T)
+        torch.cuda.current_stream(gpu.device).wait_stream(side)
+        replays = max(2, steps // 16)
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(replays):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_us = (time.perf_counter() - t0) / (replays * 16) * 1e6
+        if graph_us < eager_us:
+            dt, launch = graph_us * 1e-6 * steps, "hip graph of 16 layers"
         nbytes = 2 * H * E + hit * expert_bytes + 2 * T * H + 4 * T * H
         res[f"T{T}"] = {"us_per_layer": round(dt / steps * 1e6, 2), "us_per_token": round(dt / steps / T * 1e6, 3),
-                        "experts_hit": round(hit, 1), "algorithmic_GBps": round(nbytes * steps / dt / 1e9, 1)}
+                        "experts_hit": round(hit, 1), "algorithmic_GBps": round(nbytes * steps / dt / 1e9, 1),
+                        "launch": launch, "eager_us_per_layer": round(eager_us, 2)}
     res["config"] = "hidden 2048, 128 experts, top-8, intermediate 768, 4 bpw, mul1"
     return res
 

@@ -74,7 +74,10 @@ def test_split_k_gemv_and_mlp_block_replay_bit_exact():
         torch.cuda.synchronize()
 
 
-def test_moe_one_token_layer_replays_bit_exact():
+@pytest.mark.parametrize("T", [1, 40])
+def test_moe_layer_replays_bit_exact(T):
+    """One token (route with the sort, two grouped launches) and forty tokens (two route
+    launches, permute, rotated rows, grouped MFMA launches, combine)."""
     gpu = Gpu(0)
     H, E, k, I, bits = 512, 16, 4, 256, 4
     experts = []
@@ -82,12 +85,12 @@ def test_moe_one_token_layer_replays_bit_exact():
         experts.append(tuple(Exl3Linear(gpu, f"e{e}.{n}", *synth.linear(5000 + 10 * e + 3 * j, *shape, bits))
                              for j, (n, shape) in enumerate((("gate", (H, I)), ("up", (H, I)), ("down", (I, H))))))
     layer = MoeLayer(gpu, synth.router_weight(51, H, E), experts, k)
-    xs = [gpu.upload(synth.activations(5200 + i, 1, H).view(np.uint16)) for i in range(3)]
+    xs = [gpu.upload(synth.activations(5200 + i, T, H).view(np.uint16)) for i in range(3)]
     x = torch.zeros_like(xs[0])
-    out = torch.zeros((1, H), dtype=torch.float32, device=gpu.device)
+    out = torch.zeros((T, H), dtype=torch.float32, device=gpu.device)
 
     def step():
-        layer.forward(gpu, x, out, 1)
+        layer.forward(gpu, x, out, T)
 
     want = []
     for xi in xs:
