@@ -110,3 +110,36 @@ def test_moe_layer_replays_bit_exact(T):
         x.copy_(xs[(rep + 1) % 3])
         step()                                              # eager call of the same layer in between
         torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("rows,Kk,N", [(24, 1024, 768), (200, 512, 8320), (300, 256, 16640)])
+def test_row_launches_replay_bit_exact(rows, Kk, N):
+    """The input rotation pre-pass and the MFMA kernels (32-row tiles with split-K, evenly dealt
+    128-row tiles, 256-row tiles): shared tiles are finished through self-resetting counters."""
+    from berth_amd.device import RowScratch
+    gpu = Gpu(0)
+    lin = Exl3Linear(gpu, "rows", *synth.linear(6100 + rows, Kk, N, 4))
+    scratch = RowScratch(gpu, rows, Kk, N)
+    xs = [gpu.upload(synth.activations(6200 + i, rows, Kk).view(np.uint16)) for i in range(2)]
+    x = torch.zeros_like(xs[0])
+    out = torch.zeros((rows, N), dtype=torch.float32, device=gpu.device)
+
+    def step():
+        lin.forward_rows(gpu, scratch, x, out, rows, OutDtype.F32)
+
+    want = []
+    for xi in xs:
+        x.copy_(xi)
+        step()
+        torch.cuda.synchronize()
+        want.append(out.cpu().numpy().copy())
+    graph = _capture(gpu, step)
+    for rep in range(6):
+        x.copy_(xs[rep % 2])
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy().view(np.uint32), want[rep % 2].view(np.uint32)), rep
+        x.copy_(xs[(rep + 1) % 2])
+        step()
+        torch.cuda.synchronize()
