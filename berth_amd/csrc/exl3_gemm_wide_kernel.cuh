@@ -14,10 +14,11 @@
 //   MFMA     wave w owns rows 128*(w/4) .. +127 and columns 64*(w%4) .. +63 of the tile:
 //            32 MFMAs per macro-step, A and B operands from LDS.
 //
-// A and B tiles are double-buffered; per macro-step one barrier.  Waves 0..3 run
-// "MFMA, then decode the next macro-step", waves 4..7 "decode, then MFMA", so the two
-// waves of a SIMD (w and w+4) face each other with different work.  Trellis and A
-// registers for macro-step s+2 are loaded while s+1 is being decoded.
+// A and B tiles are double-buffered; per macro-step one barrier.  Every wave decodes its
+// share of the next macro-step, then issues its MFMAs on the current one (running the two
+// waves of a SIMD in opposite order, so that one's decode faces the other's MFMAs, was
+// measured and is no faster: the two kinds of work do not overlap on a SIMD).  Trellis
+// registers run four macro-steps ahead of the decode, A registers two.
 //
 // Handoff between workgroups that share a tile and the epilogue are those of the
 // 128-row kernel (partial sums in register layout, summed in k order by the last
@@ -25,10 +26,6 @@
 #pragma once
 
 #include "exl3_gemm_kernel.cuh"
-
-#ifndef BERTH_WIDE_STAGGER
-#define BERTH_WIDE_STAGGER 0
-#endif
 
 namespace berth {
 
@@ -167,42 +164,18 @@ __device__ __forceinline__ void gemm_tile_wide(const GemmParams& p, const int ti
         __syncthreads();
         // sub-step u of a round works on macro-step s + u: MFMAs on buffer u % 2, and macro-step
         // s + u + 1 (ring slots (u + 1) % 4 and (u + 1) % 2) is decoded into the other buffer
-#ifdef BERTH_WIDE_TRACE
-        unsigned long long t_prev, t_sum[3] = {0, 0, 0};
-        asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t_prev) :: "memory");
-#define W_STAMP(i) do { unsigned long long t_; __builtin_amdgcn_sched_barrier(0); asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t_) :: "memory"); __builtin_amdgcn_sched_barrier(0); t_sum[(i)] += t_ - t_prev; t_prev = t_; } while (0)
-#else
-#define W_STAMP(i) do {} while (0)
-#endif
         for (int s = 0; s < nsteps; s += 4) {
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 if (s + u >= nsteps) break;                         // workgroup-uniform
                 const int buf = u & 1;
-                if (BERTH_WIDE_STAGGER && rh == 0) {
-                    mfma_step(buf);
-                    W_STAMP(0);
-                    decode_and_fill(buf ^ 1, tr_ring[(u + 1) & 3], a_ring[(u + 1) & 1]);
-                    issue_tr(s + u + 5, tr_ring[(u + 1) & 3]);
-                    issue_a(s + u + 3, a_ring[(u + 1) & 1]);
-                    W_STAMP(1);
-                } else {
-                    decode_and_fill(buf ^ 1, tr_ring[(u + 1) & 3], a_ring[(u + 1) & 1]);
-                    issue_tr(s + u + 5, tr_ring[(u + 1) & 3]);
-                    issue_a(s + u + 3, a_ring[(u + 1) & 1]);
-                    W_STAMP(1);
-                    mfma_step(buf);
-                    W_STAMP(0);
-                }
+                decode_and_fill(buf ^ 1, tr_ring[(u + 1) & 3], a_ring[(u + 1) & 1]);
+                issue_tr(s + u + 5, tr_ring[(u + 1) & 3]);
+                issue_a(s + u + 3, a_ring[(u + 1) & 1]);
+                mfma_step(buf);
                 __syncthreads();
-                W_STAMP(2);
             }
         }
-#ifdef BERTH_WIDE_TRACE
-        if ((blockIdx.x == 3 || blockIdx.x == 100) && cq == 0 && lane == 0)
-            printf("wg %d rh %d steps %d: mfma %lld  decode %lld  barrier %lld (cycles per macro-step)\n", (int)blockIdx.x, rh, nsteps,
-                   (long long)t_sum[0] / nsteps, (long long)t_sum[1] / nsteps, (long long)t_sum[2] / nsteps);
-#endif
     }
 
     // ---- handoff between the workgroups that share the tile (as in exl3_gemm_kernel.cuh)
