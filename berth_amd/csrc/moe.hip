@@ -83,18 +83,6 @@ __device__ __forceinline__ float wave_max(float v)
     v = fmaxf(v, lane_xor_swap16(v));
     return fmaxf(v, lane_xor_swap32(v));
 }
-__device__ __forceinline__ int wave_min(int v)
-{
-    auto x = [](int a) { return __builtin_bit_cast(float, a); };
-    auto y = [](float a) { return __builtin_bit_cast(int, a); };
-    v = min(v, y(lane_xor_dpp<1>(x(v))));
-    v = min(v, y(lane_xor_dpp<2>(x(v))));
-    v = min(v, y(lane_xor_dpp<4>(x(v))));
-    v = min(v, y(lane_xor_dpp<8>(x(v))));
-    v = min(v, y(lane_xor_swap16(x(v))));
-    return min(v, y(lane_xor_swap32(x(v))));
-}
-
 // PER: how many of the lane's registers can hold experts (ceil(E / 64) rounded up to 2, 8 or 16)
 template <int PER>
 __device__ __forceinline__ int route_topk_n(const float (&lg)[kRoutePer], int lane, const RouteParams& p, int t)
@@ -103,20 +91,24 @@ __device__ __forceinline__ int route_topk_n(const float (&lg)[kRoutePer], int la
     float sel_logit = 0.0f;         // lane j keeps the logit of slot j
     int sel_idx = 0;
     // One slot per round: the largest remaining logit of the wave (max butterflies), then the
-    // lowest expert index among the registers that hold it (min butterflies).  Two short
-    // reductions of one value each instead of one reduction of (value, index) pairs with a
-    // tie rule: the dependent instruction chain of a round is about a third as long.
+    // lowest expert index among the registers that hold it (ballots).  One short reduction of
+    // one value instead of a reduction of (value, index) pairs with a tie rule.
     for (int j = 0; j < p.k; ++j) {
         float lv = -INFINITY;
 #pragma unroll
         for (int i = 0; i < PER; ++i)
             if (lane + 64 * i < p.E && !((taken >> i) & 1u)) lv = fmaxf(lv, lg[i]);
         const float bv = wave_max(lv);
-        int ci = 0x7fffffff;
+        // the lowest expert index that holds it: register i of lane l is expert l + 64 i, so
+        // the first register with a holder wins and, inside it, the lowest lane (a ballot
+        // and a find-first-set on the scalar side instead of a second butterfly chain)
+        int bi = 0x7fffffff;
 #pragma unroll
-        for (int i = PER - 1; i >= 0; --i)
-            if (lane + 64 * i < p.E && !((taken >> i) & 1u) && lg[i] == bv) ci = lane + 64 * i;
-        const int bi = wave_min(ci);
+        for (int i = PER - 1; i >= 0; --i) {
+            const unsigned long long holders =
+                __builtin_amdgcn_ballot_w64(lane + 64 * i < p.E && !((taken >> i) & 1u) && lg[i] == bv);
+            if (holders) bi = 64 * i + __builtin_ctzll(holders);
+        }
         if ((bi & 63) == lane) taken |= 1u << (bi >> 6);
         if (lane == j) { sel_logit = bv; sel_idx = bi; }
     }
