@@ -430,6 +430,37 @@ def test_lm_head_shape_6bpw_slices_match_oracle():
         assert close(got[c0:c0 + 256], want.reshape(-1))[0] == 0, c0
 
 
+@pytest.mark.parametrize("name,kernel", [("gate_proj", "exl3_gemm_wide_kernel<4,2,256x256>"),
+                                         ("down_proj", "exl3_gemm_balanced_kernel<4,2,128x256>"),
+                                         ("q_proj", "exl3_gemm_balanced_kernel<4,2,128x256>"),
+                                         ("k_proj", "exl3_gemm_kernel<4,2,32x256>")])
+def test_prefill_27b_shapes_at_512_rows_slices_match_oracle(name, kernel):
+    """BASELINE configs[2] at full size (512 rows, 4 bpw, the 27B shapes): each of the four
+    launch forms the dispatcher picks there, with 256-column windows (first, an odd middle
+    one, last) of all 512 rows checked against the oracle on the matching trellis slice."""
+    Kk, N = synth.SHAPES_27B[name]
+    rows, bits = 512, 4
+    tr, suh, svh = synth.linear(880 + len(name), Kk, N, bits)
+    x = synth.activations(881, rows, Kk)
+    d = {k: dev(v.view(np.uint16)) for k, v in dict(tr=tr, suh=suh, svh=svh, x=x).items()}
+    c = torch.zeros((rows, N), dtype=torch.float16, device=DEV)
+    a_had = torch.zeros((rows, Kk), dtype=torch.float16, device=DEV)
+    w = torch.zeros(Kk * min(N, 32768), dtype=torch.float16, device=DEV)
+    K.prefill_lin.exl3_linear(d["x"].data_ptr(), d["tr"].data_ptr(), c.data_ptr(), d["suh"].data_ptr(),
+                              a_had.data_ptr(), d["svh"].data_ptr(), w.data_ptr(), rows, Kk, N, bits, Codebook.MUL1,
+                              OutDtype.F16)
+    torch.cuda.synchronize()
+    assert kernel in K.prefill_lin.last_launch(), K.prefill_lin.last_launch()
+    got = host_f16(c).reshape(rows, N)
+    mid = (N // 512) * 256 + 256 if N > 1024 else 256
+    for c0 in (0, mid, N - 256):
+        sub = np.ascontiguousarray(tr[:, c0 // 16:c0 // 16 + 16, :])
+        want, want_had = O.linear(x, sub, suh, svh[c0:c0 + 256], Kk, 256, bits, 2, out_fp32=False)
+        bad, worst = close(got[:, c0:c0 + 256], want)
+        assert bad == 0, (name, c0, bad, worst)
+    assert np.array_equal(host_u16(a_had).reshape(rows, Kk), want_had.view(np.uint16))
+
+
 # ---- multi-linear (exl3_mgemm)
 @pytest.mark.parametrize("rows,fp32", [(1, False), (1, True), (3, False)])
 def test_mgemm_sliced_qkv_bundle(rows, fp32):
