@@ -61,6 +61,30 @@ static int pick_split(const Workspace& ws, long units, int KB, int mmax)
     return (int)S;
 }
 
+// One-row launches whose whole k-blocks would leave each SIMD at most 1.5 waves (the
+// grouped launches of a single token's experts) walk half k-blocks instead: twice the
+// waves, each with half the decode.  Measured: the one-token MoE layer gains 1.8 us;
+// the attention projections of the dense set (1.9 and 2.5 waves per SIMD, split 10 -> 20)
+// lose 1.5 us each to the per-wave fixed work and the longer split-K reduction, so the
+// bound sits below them, and the split stays within one batch of the finisher's loads.
+static void pick_units(const Workspace& ws, GemvParams& p, long units, int mmax)
+{
+    static const int allow = [] {
+        const char* e = std::getenv("BERTH_GEMV_HALF_UNITS");
+        return e ? std::atoi(e) : 1;
+    }();
+    p.half_units = 0;
+    if (allow && mmax == 1 && units * p.KB <= (long)ws.cu_count * 6) {
+        const int S = pick_split(ws, units, 2 * p.KB, mmax);
+        if (S <= 16) {
+            p.half_units = 1;
+            p.S = S;
+            return;
+        }
+    }
+    p.S = pick_split(ws, units, p.KB, mmax);
+}
+
 std::string launch_gemv(const LinearArgs& a)
 {
     if (a.size_m < 1 || a.size_m > 8) throw std::runtime_error("exl3 gemv: rows must be in 1..=8");
@@ -85,13 +109,13 @@ std::string launch_gemv(const LinearArgs& a)
     p.KB = a.size_k / 128;
     p.out_fp32 = a.out_fp32;
     if (p.NB > kCounters) throw std::runtime_error("exl3 gemv: size_n exceeds the split-K counter table");
-    p.S = pick_split(ws, p.NB, p.KB, mmax);
+    pick_units(ws, p, p.NB, mmax);
     const int grid = p.NB * p.S;
     launch_bits(p, a.k_bits, a.codebook, mmax, dim3(grid), a.stream);
     hip_ok(hipGetLastError(), "exl3_gemv_kernel launch");
     return "exl3_gemv_kernel<" + std::to_string(a.k_bits) + "," + std::to_string(a.codebook) + "," +
            std::to_string(mmax) + (a.a_up ? ",silu" : "") + "> grid=" + std::to_string(grid) + " block=256 split_k=" +
-           std::to_string(p.S) + (a.out_fp32 ? " out=f32" : " out=f16");
+           std::to_string(p.S) + (p.half_units ? "/half" : "") + (a.out_fp32 ? " out=f32" : " out=f16");
 }
 
 std::string launch_gemv_pair(const PairArgs& a)
@@ -121,13 +145,13 @@ std::string launch_gemv_pair(const PairArgs& a)
     p.out_fp32 = 0;
     const long units = 2L * p.NB;
     if (units > kCounters) throw std::runtime_error("exl3 gemv: size_n exceeds the split-K counter table");
-    p.S = pick_split(ws, units, p.KB, mmax);
+    pick_units(ws, p, units, mmax);
     dim3 grid((unsigned)(p.NB * p.S), 2);
     launch_bits(p, a.k_bits, a.codebook, mmax, grid, a.stream);
     hip_ok(hipGetLastError(), "exl3_gemv_kernel pair launch");
     return "exl3_gemv_kernel<" + std::to_string(a.k_bits) + "," + std::to_string(a.codebook) + "," +
            std::to_string(mmax) + "> pair grid=" + std::to_string(grid.x) + "x2 block=256 split_k=" +
-           std::to_string(p.S) + " out=f16";
+           std::to_string(p.S) + (p.half_units ? "/half" : "") + " out=f16";
 }
 
 std::string launch_mgemm(const MgemmArgs& m)
@@ -160,13 +184,13 @@ std::string launch_mgemm(const MgemmArgs& m)
     p.out_fp32 = m.c_fp32;
     const long units = (long)m.bszm_out * p.NB;
     if (units > kCounters) throw std::runtime_error("exl3_mgemm: too many (slice, column block) units");
-    p.S = pick_split(ws, units, p.KB, mmax);
+    pick_units(ws, p, units, mmax);
     dim3 grid((unsigned)(m.bszm_out * p.NB * p.S));
     launch_bits(p, m.k_bits, m.codebook, mmax, grid, m.stream);
     hip_ok(hipGetLastError(), "exl3_gemv_kernel multi launch");
     return "exl3_gemv_kernel<" + std::to_string(m.k_bits) + "," + std::to_string(m.codebook) + "," +
            std::to_string(mmax) + "> " + (sliced ? "sliced" : "uniform") + " x" + std::to_string(m.bszm_out) +
-           " grid=" + std::to_string(grid.x) + " block=256 split_k=" + std::to_string(p.S) +
+           " grid=" + std::to_string(grid.x) + " block=256 split_k=" + std::to_string(p.S) + (p.half_units ? "/half" : "") +
            (m.c_fp32 ? " out=f32" : " out=f16");
 }
 
@@ -210,13 +234,13 @@ std::string launch_gemv_grouped(const GroupedArgs& g)
         p.comb_counters = ws.counters + units;
         p.comb_k = g.comb_k;
     }
-    p.S = pick_split(ws, units, p.KB, mmax);
+    pick_units(ws, p, units, mmax);
     dim3 grid((unsigned)(g.max_problems * p.NB * p.S), (unsigned)g.num_lins);
     launch_bits(p, g.k_bits, g.codebook, mmax, grid, g.stream);
     hip_ok(hipGetLastError(), "exl3_gemv_kernel grouped launch");
     return "exl3_gemv_kernel<" + std::to_string(g.k_bits) + "," + std::to_string(g.codebook) + "," +
            std::to_string(mmax) + "> grouped grid=" +
-           std::to_string(grid.x) + "x" + std::to_string(grid.y) + " split_k=" + std::to_string(p.S) +
+           std::to_string(grid.x) + "x" + std::to_string(grid.y) + " split_k=" + std::to_string(p.S) + (p.half_units ? "/half" : "") +
            (g.comb_out ? " +combine" : "");
 }
 

@@ -78,6 +78,7 @@ struct GemvParams {
     float* partials;            // [problem][lin][NB][S][MMAX][128]
     unsigned* counters;         // [problem][lin][NB]
     int K, N, NB, KB, S, out_fp32;
+    int half_units;             // 1: a unit of the K walk is half a k-block (one row only)
     // one-token expert combine folded into the down projection (grouped mode, one
     // row per problem, fp32 rows in c[0]): the last problem to finish a column
     // block writes comb_out[h] = fma chain over j of comb_w[j] * c[0][comb_inv[j]][h]
@@ -144,7 +145,13 @@ struct GemvWalk {
 // a_had store lives in its own instantiation, used by the column-block-0
 // workgroups): with a store or a branch in the body the compiler's wait counts
 // degrade to "wait for everything", which serialises the pipeline.
-template <int BITS, int CB, int MMAX, bool SILU, bool WRITE_HAD>
+//
+// TRS is the number of tile rows of a k-block one unit of the walk covers: 8 (a whole
+// k-block per unit) or 4 (half a k-block: both halves rotate the whole 128-element block
+// of the activation, each decodes only its 4 tile rows).  Half units double the number of
+// waves a narrow, shallow weight can spread over.  The walk's step is a multiple of 4, so
+// which half a wave owns never changes along its walk.
+template <int BITS, int CB, int MMAX, bool SILU, bool WRITE_HAD, int TRS>
 __device__ __forceinline__ void gemv_accumulate(const GemvWalk& w, const int (&src)[MMAX],
                                                 uint32_t (&xs)[MMAX][64], float (&acc)[MMAX][2])
 {
@@ -154,10 +161,13 @@ __device__ __forceinline__ void gemv_accumulate(const GemvWalk& w, const int (&s
 #pragma unroll
     for (int m = 0; m < MMAX; ++m) acc[m][0] = acc[m][1] = 0.0f;
 
-    uint32_t own[8][BITS];
+    constexpr int UPK = 8 / TRS;                        // units per k-block
+    uint32_t own[TRS][BITS];
     half2_t xr[MMAX], ur[MMAX], sc;
-    int kb = w.kb0;
-    if (kb >= w.KB) return;
+    int unit = w.kb0;                                   // w.kb0, w.step and w.KB count units
+    if (unit >= w.KB) return;
+    const int sub = unit % UPK;                         // constant along the walk
+    int kb = unit / UPK;
     {
         // same issue order as inside the loop (activation first, then the tile rows),
         // so that the wait counts the compiler derives at the loop head stay exact
@@ -169,17 +179,19 @@ __device__ __forceinline__ void gemv_accumulate(const GemvWalk& w, const int (&s
             if (SILU) ur[m] = ((global_ptr<const half2_t>)(w.a_up + (size_t)src[m] * w.K + kb * 128))[lane];
         }
         __builtin_amdgcn_sched_barrier(0);
-        const global_ptr<const uint32_t> base = w.tbase + (size_t)(kb * 8) * w.row_dw;
+        const global_ptr<const uint32_t> base = w.tbase + (size_t)(kb * 8 + sub * TRS) * w.row_dw;
 #pragma unroll
-        for (int tr = 0; tr < 8; ++tr) {
+        for (int tr = 0; tr < TRS; ++tr) {
             load_tile_dwords<BITS>(base + tr * w.row_dw + lane_dw, own[tr]);
             __builtin_amdgcn_sched_barrier(0);          // tile row 0 must be the oldest load in flight
         }
     }
 
-    for (; kb < w.KB; kb += w.step) {
-        const int nkb = kb + w.step;
-        const bool has_next = nkb < w.KB;
+    for (; unit < w.KB; unit += w.step) {
+        kb = unit / UPK;
+        const int nunit = unit + w.step;
+        const int nkb = nunit / UPK;
+        const bool has_next = nunit < w.KB;
         const int pkb = has_next ? nkb : kb;            // k-block whose activation is prefetched
         // rotate this k-block of the activation: Hh(x * suh), rounded to fp16
 #pragma unroll
@@ -197,7 +209,8 @@ __device__ __forceinline__ void gemv_accumulate(const GemvWalk& w, const int (&s
             r.x = (_Float16)(v0 * kRsqrt128);
             r.y = (_Float16)(v1 * kRsqrt128);
             xs[m][lane] = as_u32(r);
-            if (WRITE_HAD) ((global_ptr<half2_t>)(w.a_had + (size_t)m * w.K + kb * 128))[lane] = r;
+            if (WRITE_HAD && (UPK == 1 || sub == 0))
+                ((global_ptr<half2_t>)(w.a_had + (size_t)m * w.K + kb * 128))[lane] = r;
         }
         sc = w.suh[pkb * 64 + lane];
 #pragma unroll
@@ -214,10 +227,12 @@ __device__ __forceinline__ void gemv_accumulate(const GemvWalk& w, const int (&s
         // No branch inside the tile-row loop (the compiler would sink the decode below
         // it): a wave on its last k-block re-reads tile row 0 of its column block,
         // always the same cached KiB, and ignores the result.
-        const global_ptr<const uint32_t> nbase = w.tbase + (has_next ? (size_t)(nkb * 8) * w.row_dw : (size_t)0);
+        const global_ptr<const uint32_t> nbase =
+            w.tbase + (has_next ? (size_t)(nkb * 8 + sub * TRS) * w.row_dw : (size_t)0);
         const size_t nrow_dw = has_next ? w.row_dw : 0;
+        const uint32_t* xsub = &xs[0][sub * TRS * 8];
 #pragma unroll
-        for (int tr = 0; tr < 8; ++tr) {
+        for (int tr = 0; tr < TRS; ++tr) {
             uint32_t prev = fetch_prev(lane, own[tr][BITS - 1]);
             uint32_t w2[16];
             decode_lane<BITS, CB>(own[tr], prev, w2);
@@ -226,7 +241,7 @@ __device__ __forceinline__ void gemv_accumulate(const GemvWalk& w, const int (&s
 #pragma unroll
             for (int m = 0; m < MMAX; ++m) {
                 if (MMAX > 1 && m >= rows) break;       // wave-uniform
-                const uint4* xp = (const uint4*)&xs[m][tr * 8];
+                const uint4* xp = (const uint4*)(xsub + m * 64 + tr * 8);
                 uint4 xa = xp[0], xb = xp[1];
                 const uint32_t xk[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
 #pragma unroll
@@ -239,7 +254,7 @@ __device__ __forceinline__ void gemv_accumulate(const GemvWalk& w, const int (&s
     }
 }
 
-template <int BITS, int CB, int MMAX, bool SILU>
+template <int BITS, int CB, int MMAX, bool SILU, int TRS = 8>
 __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
 {
     __shared__ uint32_t xs[4][MMAX][64];    // wave-private: rotated k-block, one half2 per entry
@@ -311,12 +326,12 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
         w.a_had = as_global(p.a_had) + ((size_t)had_slab * rows + row0) * p.K;
         w.row_dw = row_dw;
         w.K = p.K;
-        w.KB = p.KB;
+        w.KB = p.KB * (8 / TRS);
         w.kb0 = s * 4 + wave;
         w.step = wc;
         w.rows = rows;
-        if (p.a_had && nb == 0 && which == 0) gemv_accumulate<BITS, CB, MMAX, SILU, true>(w, src, xs[wave], acc);
-        else gemv_accumulate<BITS, CB, MMAX, SILU, false>(w, src, xs[wave], acc);
+        if (p.a_had && nb == 0 && which == 0) gemv_accumulate<BITS, CB, MMAX, SILU, true, TRS>(w, src, xs[wave], acc);
+        else gemv_accumulate<BITS, CB, MMAX, SILU, false, TRS>(w, src, xs[wave], acc);
     }
 
     // ---- reduce the 4 waves (k split inside the workgroup), wave order

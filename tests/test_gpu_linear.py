@@ -223,6 +223,31 @@ def test_gemv_m1_shapes_split_k(Kk, N):
     assert bad == 0, (bad, worst, launch)
 
 
+@pytest.mark.parametrize("Kk,N,bits,half", [(2048, 768, 4, True), (768, 2048, 3, True), (128, 128, 5, True),
+                                             (384, 256, 2, True), (4096, 4096, 4, True), (5120, 8192, 4, False), (2048, 768, 4, None)])
+def test_gemv_m1_half_k_block_units(Kk, N, bits, half):
+    """One-row launches with few column blocks and k-blocks walk half k-blocks (two waves
+    share a k-block: both rotate it, each decodes 4 of its 8 tile rows, the first writes the
+    rotated activation); wide ones keep whole k-blocks.  half=None: the same shape with
+    half units switched off, in a fresh process (the switch is read once)."""
+    if half is None:
+        import subprocess, sys
+        code = ("import numpy as np\nfrom tests.test_gpu_linear import _run_linear\nfrom tests.gpu_util import close\n"
+                f"got, want, ah, want_ah, launch = _run_linear(1, {Kk}, {N}, {bits}, 2, True, 7)\n"
+                "assert '/half' not in launch, launch\nassert np.array_equal(ah, want_ah)\n"
+                "assert close(got, want)[0] == 0\nprint('ok')\n")
+        env = dict(os.environ, BERTH_GEMV_HALF_UNITS="0")
+        r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=240,
+                           cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+        assert r.returncode == 0 and "ok" in r.stdout, r.stdout + r.stderr
+        return
+    got, want, ah, want_ah, launch = _run_linear(1, Kk, N, bits, 2, True, 7)
+    assert ("/half" in launch) == half, launch
+    assert np.array_equal(ah, want_ah), launch
+    bad, worst = close(got, want)
+    assert bad == 0, (bad, worst, launch)
+
+
 def test_gemv_m1_is_deterministic_and_counters_reset():
     outs = []
     for _ in range(3):
