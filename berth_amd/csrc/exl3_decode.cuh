@@ -54,6 +54,31 @@ __device__ __forceinline__ global_ptr<T> as_global(T* p) { return (global_ptr<T>
 // caches, so the compiler emits no wait on vector memory for it), and neither does a barrier.
 #ifndef BERTH_HOST_EMU
 __device__ __forceinline__ void wait_own_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// Touches the first LINES 64-byte lines of the kernel-argument block with one scalar read
+// each, all in flight together, so that the argument fields the compiler reads one by one
+// further down (behind branches, each with a wait of its own) find their line in the scalar
+// cache instead of paying a miss per line in sequence.  The caller's argument block must
+// span LINES * 64 bytes (the hidden arguments that follow the explicit ones count).
+template <int LINES>
+__device__ __forceinline__ void touch_kernel_arguments()
+{
+    static_assert(LINES >= 1 && LINES <= 6, "one register per line");
+    const auto ka = __builtin_amdgcn_kernarg_segment_ptr();
+    int t0, t1, t2, t3, t4, t5;
+    if constexpr (LINES == 6)
+        asm volatile("s_load_dword %0, %6, 0x0\n\ts_load_dword %1, %6, 0x40\n\ts_load_dword %2, %6, 0x80\n\t"
+                     "s_load_dword %3, %6, 0xc0\n\ts_load_dword %4, %6, 0x100\n\ts_load_dword %5, %6, 0x140\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5) : "s"(ka));
+    else if constexpr (LINES >= 3)
+        asm volatile("s_load_dword %0, %3, 0x0\n\ts_load_dword %1, %3, 0x40\n\ts_load_dword %2, %3, 0x80\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&s"(t0), "=&s"(t1), "=&s"(t2) : "s"(ka));
+    else
+        asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %2, 0x40\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&s"(t0), "=&s"(t1) : "s"(ka));
+}
 #endif
 
 __device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }

@@ -261,6 +261,8 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
     __shared__ float red[4][MMAX][128];
     __shared__ unsigned s_last;
 
+    static_assert(sizeof(GemvParams) > 5 * 64, "the argument block spans six lines");
+    touch_kernel_arguments<6>();
     const int lane = threadIdx.x & 63;
     // wave-uniform on purpose: everything derived from it (k-block, addresses) stays in SGPRs
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
