@@ -277,6 +277,8 @@ constexpr int kRouteOneMaxE = 128;
 
 __global__ __launch_bounds__(1024) void moe_route_one_token_kernel(RouteParams p)
 {
+    static_assert(sizeof(RouteParams) > 2 * 64, "argument lines");
+    touch_kernel_arguments<3>();
     __shared__ float part_s[kRouteOneMaxSeg][kRouteOneMaxE];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
