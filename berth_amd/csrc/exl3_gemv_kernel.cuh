@@ -276,8 +276,14 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
     ExpertLin lin = p.pair ? p.shared[which] : p.lin;
     int row0 = 0, rows = p.rows;
     if (p.problems) {
-        if (prob >= *p.num_problems) return;
+        // the list holds an entry for every problem index of the grid: this one is read
+        // together with the count, not after it (one dependent read less ahead of the
+        // first weight load); the empty asm keeps the compiler from sinking the read
+        // below the branch again
         const GroupProblem gp = p.problems[prob];
+        const int count = *p.num_problems;
+        asm volatile("" ::"s"(gp.expert), "s"(count));
+        if (prob >= count) return;
         lin = gp.expert == p.shared_expert ? p.shared[p.lin_base + which]
                                            : p.experts[gp.expert * p.lins_per_expert + p.lin_base + which];
         row0 = gp.row0;
