@@ -9,7 +9,7 @@ random signs times lognormal(0,0.1).  One step = the seven linears of one layer 
 four launches: q/k/v as one sliced multi-linear (berth_ops_mgemm, as the
 reference bundles them), o_proj (berth_exl3_linear), gate+up as one multi-linear,
 down_proj.  Steps rotate
-over `--layers` distinct weight sets (default 8 = 1.36 GB) so that reads come
+over `--layers` distinct weight sets (default 10 = 1.7 GB) so that reads come
 from HBM, not from the 256 MB memory-side cache.  Inputs are resident in HBM
 before the timed region.
 
@@ -35,6 +35,9 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per GEMV launch of the default workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs scaled by a 1 GiB copy (profiles/exl3_gemv_4bpw_batch1_27b_linear_set.md)
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {4: int((42787 + 604) * 1024)}
+# vector instructions per weight of the GEMV launches of the default workload, from a rocprofv3
+# --pmc SQ_INSTS_VALU run of this file (same profile): wave instructions * 64 lanes / weights
+VALU_INSTR_PER_WEIGHT = 4.9
 ORDER = ["q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"]
 OUT_FP32 = {"q_proj": False, "k_proj": False, "v_proj": False, "o_proj": True,
             "gate_proj": False, "up_proj": False, "down_proj": True}
@@ -98,6 +101,59 @@ def cpu_baseline(bits: int, seconds: float):
         "sample": f"{n_gemv0} GEMVs and {n_deq} dequantisations of 4096x4096 at 4 bpw, {n_moe} one-token MoE layers "
                   f"(128 experts, top-8; 8 distinct synthetic experts repeated)"}
     return res
+
+
+def time_steps(gpu, step, steps: int, warmup: int, graph: bool = True):
+    """Time exactly `steps` calls of step(i), i = 0 .. steps-1, two ways: launched one by one
+    (eager), and recorded once into a HIP graph that holds all `steps` calls and is replayed
+    (the library's launches keep no host state between calls, so a recorded step replays bit
+    for bit).  Each way: (wall ms, device ms between two events on the launch stream).  The
+    graph pair is None when recording is switched off."""
+    import torch
+
+    def timed(run):
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        run()
+        e1.record()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3, e0.elapsed_time(e1)
+
+    for i in range(warmup):
+        step(i)
+    eager = timed(lambda: [step(i) for i in range(steps)])
+    if not graph:
+        return eager, None
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream(device=gpu.device)
+    side.wait_stream(torch.cuda.current_stream(gpu.device))
+    with torch.cuda.stream(side):
+        step(0)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(g, stream=side):
+            for i in range(steps):
+                step(i)
+    torch.cuda.current_stream(gpu.device).wait_stream(side)
+    g.replay()                                          # untimed: the first replay uploads the graph
+    runs = sorted((timed(g.replay) for _ in range(3)), key=lambda t: t[1])
+    return eager, runs[1]                               # the median of three replays
+
+
+def valu_ceiling(bits: int):
+    """The vector-ALU bound of the decode, measured live: lane-instructions per second of
+    the decode's instruction mix (libberth_probe.so) over the vector instructions the GEMV
+    kernel issues per weight (SQ_INSTS_VALU * 64 / weights of the layer set,
+    profiles/exl3_gemv_4bpw_batch1_27b_linear_set.md)."""
+    import ctypes
+    lib = ctypes.CDLL(os.path.join(ROOT, "berth_amd", "lib", "libberth_probe.so"))
+    lib.berth_probe_valu_lane_instr_per_s.restype = ctypes.c_double
+    rate = lib.berth_probe_valu_lane_instr_per_s()
+    ipw = VALU_INSTR_PER_WEIGHT
+    return {"lane_instr_per_s": round(rate / 1e12, 2), "unit": "T lane-instr/s", "instr_per_weight": ipw,
+            "weights_per_s": round(rate / ipw / 1e12, 2), "implied_GBps": round(rate / ipw * bits / 8 / 1e9, 1),
+            "implied_frac_of_hbm_peak": round(rate / ipw * bits / 8 / 1e9 / HBM_PEAK_GBS, 4)}
 
 
 def moe_bench(gpu, steps: int, warmup: int):
@@ -299,27 +355,18 @@ def bpw_sweep(gpu, rates, steps: int, nlayers: int = 8):
             lin["gate_up"].forward(gpu, xin[5120], [outs["gate_proj"], outs["up_proj"]], OutDtype.F16)
             lin["down_proj"].forward(gpu, xin[17408], outs["down_proj"], OutDtype.F32)
 
-        for i in range(10):
-            step(i)
-        torch.cuda.synchronize()
-        dt, wall = None, None
-        for _ in range(2):                                  # best of two passes
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            t0 = time.perf_counter()
-            e0.record()
-            for i in range(steps):
-                step(i)
-            e1.record()
-            torch.cuda.synchronize()
-            w = (time.perf_counter() - t0) / steps
-            d = e0.elapsed_time(e1) * 1e-3 / steps          # device time between the two events
-            if dt is None or d < dt:
-                dt, wall = d, w
+        (e_wall, e_dev), graphed = time_steps(gpu, step, steps, 10)
+        dt = e_dev * 1e-3 / steps
+        wall = e_wall * 1e-3 / steps
+        launch = "eager"
+        if graphed is not None and graphed[1] < e_dev:
+            dt, launch = graphed[1] * 1e-3 / steps, f"hip graph of {steps} steps"
         nbytes = sum(linear_bytes(*synth.SHAPES_27B[n], bits, 1, 4 if OUT_FP32[n] else 2) for n in ORDER)
         res[f"{bits}bpw"] = {"GBps": round(nbytes / dt / 1e9, 1), "us_per_step": round(dt * 1e6, 2),
                              "frac_of_hbm_peak": round(nbytes / dt / 1e9 / HBM_PEAK_GBS, 4),
-                             "Gweights_per_s": round(340787200 / dt / 1e9, 1),
-                             "host_us_per_step": round(wall * 1e6, 2)}
+                             "Gweights_per_s": round(340787200 / dt / 1e9, 1), "launch": launch,
+                             "eager_device_us_per_step": round(e_dev * 1e3 / steps, 2),
+                             "eager_host_us_per_step": round(wall * 1e6, 2)}
         del layers
         torch.cuda.empty_cache()
     return res
@@ -489,7 +536,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--layers", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=10)
     ap.add_argument("--bits", type=int, default=4)
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-cpu", action="store_true")
@@ -499,6 +546,7 @@ def main():
     ap.add_argument("--no-lm-head", action="store_true")
     ap.add_argument("--no-mlp", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only")
+    ap.add_argument("--no-valu", action="store_true", help="skip the vector-ALU rate probe")
     ap.add_argument("--moe-resident-layers", type=int, default=48)
     ap.add_argument("--unfused", action="store_true", help="seven separate launches instead of four")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -564,41 +612,10 @@ def main():
         lin["gate_up"].forward(gpu, xin[5120], [outs["gate_proj"], outs["up_proj"]], f16)
         lin["down_proj"].forward(gpu, xin[17408], outs["down_proj"], f32)
 
-    def timed(run_steps):
-        """(wall ms, device ms between two events on the launch stream) for args.steps steps."""
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        e0.record()
-        run_steps()
-        e1.record()
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3, e0.elapsed_time(e1)
-
-    for i in range(args.warmup):
-        step(i)
-    eager_wall_ms, eager_ev_ms = timed(lambda: [step(i) for i in range(args.steps)])
+    (eager_wall_ms, eager_ev_ms), graphed = time_steps(gpu, step, args.steps, args.warmup, graph=not args.no_graph)
     wall_ms, ev_ms, launch_mode = eager_wall_ms, eager_ev_ms, "eager"
-    if not args.no_graph and args.steps % len(layers) == 0:
-        # the same launches recorded once into a HIP graph (one pass over the rotated
-        # weight sets) and replayed: removes the per-launch host and dispatch cost
-        graph = torch.cuda.CUDAGraph()
-        side = torch.cuda.Stream(device=gpu.device)
-        side.wait_stream(torch.cuda.current_stream(gpu.device))
-        with torch.cuda.stream(side):
-            for i in range(len(layers)):
-                step(i)
-            torch.cuda.synchronize()
-            with torch.cuda.graph(graph, stream=side):
-                for i in range(len(layers)):
-                    step(i)
-        torch.cuda.current_stream(gpu.device).wait_stream(side)
-        replays = args.steps // len(layers)
-        for _ in range(2):
-            graph.replay()
-        g_wall_ms, g_ev_ms = timed(lambda: [graph.replay() for _ in range(replays)])
-        if g_ev_ms < ev_ms:
-            wall_ms, ev_ms, launch_mode = g_wall_ms, g_ev_ms, f"hip graph of {len(layers)} steps"
+    if graphed is not None and graphed[1] < ev_ms:
+        wall_ms, ev_ms, launch_mode = graphed[0], graphed[1], f"hip graph of {args.steps} steps"
     ms_per_step = wall_ms / args.steps
     value = step_bytes * args.steps / (wall_ms * 1e-3) / 1e9
 
@@ -621,14 +638,21 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"27B-shaped decode linear set (q,k,v,o,gate,up,down), batch 1, {bits} bpw, mul1",
                    "layers_rotated": len(layers), "bytes_per_step": step_bytes, "launch": launch_mode,
-                   "eager_GBps": round(step_bytes * args.steps / (eager_wall_ms * 1e-3) / 1e9, 1),
+                   "eager": {"GBps": round(step_bytes * args.steps / (eager_wall_ms * 1e-3) / 1e9, 1),
+                             "us_per_step": round(eager_wall_ms * 1e3 / args.steps, 2),
+                             "device_us_per_step": round(eager_ev_ms * 1e3 / args.steps, 2)},
+                   "graph": None if graphed is None else {
+                       "GBps": round(step_bytes * args.steps / (graphed[0] * 1e-3) / 1e9, 1),
+                       "us_per_step": round(graphed[0] * 1e3 / args.steps, 2),
+                       "device_us_per_step": round(graphed[1] * 1e3 / args.steps, 2)},
                    "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(bits) if len(layers) == 8 and not args.unfused else None,
+                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(bits) if not args.unfused else None,
                      "kernel": Kn.last_launch().split(" grid=")[0],
                      "avg_launch_us": round(avg_launch_us, 3),
-                     "bytes_per_launch": step_bytes // launches_per_step},
+                     "bytes_per_launch": step_bytes // launches_per_step,
+                     "valu_ceiling": None if args.no_valu else valu_ceiling(bits)},
     }
     if not args.no_sweep:
         line["bpw_sweep"] = bpw_sweep(gpu, [b for b in (2, 3, 4, 5) if b != bits], max(20, args.steps // 2))

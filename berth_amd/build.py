@@ -21,15 +21,18 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
 
 LIBRARIES = {
     "libberth_kernels_hip.so": ["api.hip", "exl3_gemv.hip", "exl3_gemv_cb0.hip", "exl3_gemv_cb1.hip",
-                                "exl3_gemv_cb2.hip", "exl3_gemm.hip", "exl3_gemm_cb0.hip", "exl3_gemm_cb1.hip",
+                                "exl3_gemv_cb2.hip", "exl3_gemv_stream_cb0.hip", "exl3_gemv_stream_cb1.hip",
+                                "exl3_gemv_stream_cb2.hip", "exl3_gemm.hip", "exl3_gemm_cb0.hip", "exl3_gemm_cb1.hip",
                                 "exl3_gemm_cb2.hip",
                                 "exl3_reconstruct.hip", "elementwise.hip", "moe.hip"],
     "libberth_hip.so": ["berth_hip.hip"],
+    # measurement probe used by bench.py only
+    "libberth_probe.so": ["probe/valu_rate.hip"],
 }
 
 
 def _compile(src: str) -> str:
-    obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+    obj = os.path.join(OBJ, os.path.splitext(src)[0].replace("/", "_") + ".o")
     cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:

@@ -31,6 +31,10 @@ Workspace& workspace_for_current_device()
         hip_ok(hipMalloc(&partials, kPartialBytes), "split-K workspace");
         hip_ok(hipMalloc(&counters, kCounters * sizeof(unsigned)), "split-K counters");
         hip_ok(hipMemset(counters, 0, kCounters * sizeof(unsigned)), "split-K counter memset");
+        void* tables = nullptr;
+        hip_ok(hipMalloc(&tables, 3 * 65536 * sizeof(uint16_t)), "state tables");
+        build_state_tables((uint16_t*)tables);
+        ws.state_tables = (uint16_t*)tables;
         int cus = 0;
         hip_ok(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device), "multiProcessorCount");
         ws.partials = (float*)partials;

@@ -16,9 +16,7 @@
 // k = 2q + 8h + {0,1} of column u + 8f.
 #pragma once
 
-#ifndef BERTH_HOST_EMU
 #include <hip/hip_runtime.h>
-#endif
 #include <stdint.h>
 
 namespace berth {
@@ -39,20 +37,17 @@ __host__ __device__ constexpr int pair_kk(int p) { return (p >> 2) + 4 * (p & 1)
 // Pointers that reach a kernel through memory (device tables of pointers) lose
 // their address space; these casts restore "global" so that loads and stores are
 // global_* instructions rather than flat_* ones.
-#ifndef BERTH_HOST_EMU
 template <typename T>
 using global_ptr = __attribute__((address_space(1))) T*;
 template <typename T>
 __device__ __forceinline__ global_ptr<const T> as_global(const T* p) { return (global_ptr<const T>)p; }
 template <typename T>
 __device__ __forceinline__ global_ptr<T> as_global(T* p) { return (global_ptr<T>)p; }
-#endif
 
 // A workgroup that is about to tell another workgroup, through an agent-scope counter, that
 // its stores are there: every wave first waits until its own stores have completed.  The
 // workgroup-scope release fence does not do that (the waves of a workgroup share their
 // caches, so the compiler emits no wait on vector memory for it), and neither does a barrier.
-#ifndef BERTH_HOST_EMU
 __device__ __forceinline__ void wait_own_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // Touches the first LINES 64-byte lines of the kernel-argument block with one scalar read
@@ -80,7 +75,6 @@ __device__ __forceinline__ void touch_kernel_arguments()
                      "s_waitcnt lgkmcnt(0)"
                      : "=&s"(t0), "=&s"(t1), "=&s"(t2) : "s"(ka));
 }
-#endif
 
 __device__ __forceinline__ half2_t as_half2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
 __device__ __forceinline__ uint32_t as_u32(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
@@ -174,7 +168,6 @@ __device__ __forceinline__ void decode_lane(const uint32_t (&own)[BITS], uint32_
 // The dword just before a lane's own dwords belongs to the previous lane of its
 // octet (octet-local rotate by one: lane u = 0 takes it from lane u = 7).  Two DPP
 // moves inside the 16-lane row and a select; no LDS traffic.
-#ifndef BERTH_HOST_EMU
 __device__ __forceinline__ uint32_t fetch_prev(int lane, uint32_t last_own)
 {
     const int v = (int)last_own;
@@ -182,6 +175,5 @@ __device__ __forceinline__ uint32_t fetch_prev(int lane, uint32_t last_own)
     const int from_above = __builtin_amdgcn_update_dpp(v, v, 0x107, 0xF, 0xF, false);   // row_shl:7, lane i <- i+7
     return (uint32_t)((lane & 7) ? from_below : from_above);
 }
-#endif
 
 }  // namespace berth

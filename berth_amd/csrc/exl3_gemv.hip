@@ -15,9 +15,11 @@
 //     workspace and the last workgroup to arrive adds them in split order,
 //     applies the output Hadamard and svh and stores c.  The arrival counter
 //     resets itself.  Summation order never depends on timing.
-#include "exl3_gemv_kernel.cuh"
+#include "exl3_gemv_stream_kernel.cuh"
 #include "launch.h"
 
+#include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 
@@ -35,6 +37,140 @@ static void launch_bits(const GemvParams& p, int bits, int cb, int mmax, dim3 gr
     case 1: launch_gemv_cb1(p, bits, mmax, grid, stream); break;
     default: launch_gemv_cb2(p, bits, mmax, grid, stream); break;
     }
+}
+
+void launch_gemv_stream_cb0(const StreamParams& p, int bits, int lutmask, dim3 grid, hipStream_t stream);
+void launch_gemv_stream_cb1(const StreamParams& p, int bits, int lutmask, dim3 grid, hipStream_t stream);
+void launch_gemv_stream_cb2(const StreamParams& p, int bits, int lutmask, dim3 grid, hipStream_t stream);
+
+// ---- state -> weight tables of the three codebooks (one launch each at workspace set-up)
+template <int CB>
+__global__ void state_table_kernel(uint16_t* table)
+{
+    const uint32_t s = blockIdx.x * blockDim.x + threadIdx.x;
+    if (s < 65536u) table[s] = (uint16_t)(decode_pair<CB>(s, s) & 0xffffu);
+}
+
+void build_state_tables(uint16_t* tables)
+{
+    hipLaunchKernelGGL(state_table_kernel<0>, dim3(256), dim3(256), 0, 0, tables);
+    hipLaunchKernelGGL(state_table_kernel<1>, dim3(256), dim3(256), 0, 0, tables + 65536);
+    hipLaunchKernelGGL(state_table_kernel<2>, dim3(256), dim3(256), 0, 0, tables + 2 * 65536);
+    hip_ok(hipGetLastError(), "state_table_kernel launch");
+    hip_ok(hipStreamSynchronize(0), "state tables");
+}
+
+// ---- the one-row streaming kernel: the static split and when it applies
+//
+// Of a problem's U = (N/128) * (K/16) units every wave of its Gp workgroups takes q (the
+// first `rem` waves q + 1).  The kernel applies when every wave gets at least
+// `stream_min_units` tile rows (below that the fixed cost of a sixteen-wave workgroup, its
+// table copy and its barriers, is not paid back), when the rotated activation of a
+// workgroup's units fits its LDS region and when the exact-division multipliers are exact
+// for the operands the kernel divides.
+struct StreamPlan {
+    bool ok = false;
+    int problems = 0, Gp = 0, maxc = 0;
+    unsigned q = 0, rem = 0, mq = 0, mq1 = 0, mtr = 0;
+};
+
+static int env_int(const char* name, int fallback)
+{
+    const char* e = std::getenv(name);
+    return e ? (int)std::strtol(e, nullptr, 0) : fallback;
+}
+
+// Knobs, read at every call (tests switch them inside one process):
+//   BERTH_GEMV_STREAM            0: never take the streaming kernel
+//   BERTH_GEMV_STREAM_MIN_UNITS  fewest tile rows per wave for which it is taken (default 4)
+//   BERTH_GEMV_STREAM_SHRINK     1: a smaller weight takes it with fewer workgroups instead of
+//                                falling back (default 0: the many-workgroup kernel is faster there)
+//   BERTH_GEMV_STREAM_WGS        cap on the workgroups per problem
+//   BERTH_GEMV_STREAM_LUT        table mask of the hybrid decode (bit pp: pair pp of every dword
+//                                comes from the table); 0: arithmetic only; unset: by size (below)
+// The 128 KiB table costs every workgroup a copy through its compute unit's load path (1.2 us
+// measured) and pays back about an eighth of the decode time at 4 bits per weight, where
+// the window halves feed the table addresses directly (335 MB weight: 103.6 -> 92.4 us); at
+// other bit rates the addresses cost a shift each and the gain was 1 % (27B lm_head, 6 bpw).
+// So: 4 bpw weights of at least 1 MiB per workgroup.
+static int stream_lut_mask(int bits, unsigned long long bytes_per_workgroup)
+{
+    const int forced = env_int("BERTH_GEMV_STREAM_LUT", -1);
+    if (forced >= 0) return forced;
+    return bits == 4 && bytes_per_workgroup >= (1ull << 20) ? 0xA : 0;
+}
+
+static unsigned magic(unsigned d) { return (unsigned)((1ull << 32) / d) + 1u; }
+
+static StreamPlan plan_stream(const Workspace& ws, int problems, int K, int N)
+{
+    StreamPlan pl;
+    if (!env_int("BERTH_GEMV_STREAM", 1) || problems < 1 || problems > ws.cu_count) return pl;
+    const unsigned TR = (unsigned)K / 16, NB = (unsigned)N / 128, KB = (unsigned)K / 128;
+    const unsigned long long U = (unsigned long long)NB * TR;
+    if (U >= (1ull << 31)) return pl;
+    const unsigned min_units = (unsigned)std::max(2, env_int("BERTH_GEMV_STREAM_MIN_UNITS", 4));
+    int Gp = ws.cu_count / problems;
+    const int cap = env_int("BERTH_GEMV_STREAM_WGS", 0);
+    if (cap > 0 && Gp > cap) Gp = cap;
+    if (U / ((unsigned)Gp * kStreamWaves) < min_units) {
+        if (!env_int("BERTH_GEMV_STREAM_SHRINK", 0)) return pl;
+        Gp = (int)(U / (min_units * kStreamWaves));
+        if (Gp < 1) return pl;
+    }
+    const unsigned waves = (unsigned)Gp * kStreamWaves;
+    const unsigned q = (unsigned)(U / waves), rem = (unsigned)(U % waves);
+    // exact division by multiply-high needs dividend * divisor < 2^32
+    if (U * (q + 2) >= (1ull << 32) || U * TR >= (1ull << 32)) return pl;
+    const unsigned L = kStreamWaves * (q + 1);                 // most units of one workgroup
+    if ((L + TR - 1) / TR + 1 > (unsigned)kStreamMaxCb) return pl;
+    if (KB > (unsigned)kStreamXsBlocks && (L + 16 >= TR || L / 8 + 2 > (unsigned)kStreamXsBlocks)) return pl;
+    const unsigned maxc = (TR + kStreamWaves * q - 1) / (kStreamWaves * q) + 1;   // workgroups that can share a column block
+    if ((unsigned long long)problems * NB > (unsigned long long)kCounters) return pl;
+    if ((unsigned long long)problems * NB * maxc * 128 * sizeof(float) > kPartialBytes) return pl;
+    pl.ok = true;
+    pl.problems = problems;
+    pl.Gp = Gp;
+    pl.maxc = (int)maxc;
+    pl.q = q;
+    pl.rem = rem;
+    pl.mq = magic(q);
+    pl.mq1 = magic(q + 1);
+    pl.mtr = magic(TR);
+    return pl;
+}
+
+static std::string run_stream(const Workspace& ws, const StreamPlan& pl, StreamParams& p, int bits, int cb,
+                              hipStream_t stream)
+{
+    int mask = ws.state_tables ? stream_lut_mask(bits, (unsigned long long)pl.q * kStreamWaves * 256 * bits) : 0;
+#ifndef BERTH_STREAM_EXTRA_MASKS
+    if (mask != 0) mask = 0xA;          // the one hybrid mask that is instantiated
+#endif
+    p.lut = ws.state_tables ? ws.state_tables + (size_t)cb * 65536 : nullptr;
+    p.partials = ws.partials;
+    p.counters = ws.counters;
+    p.TR = p.K / 16;
+    p.NB = p.N / 128;
+    p.Gp = pl.Gp;
+    p.q = pl.q;
+    p.rem = pl.rem;
+    p.mq = pl.mq;
+    p.mq1 = pl.mq1;
+    p.mtr = pl.mtr;
+    p.maxc = pl.maxc;
+    const dim3 grid((unsigned)(pl.problems * pl.Gp));
+    switch (cb) {
+    case 0: launch_gemv_stream_cb0(p, bits, mask, grid, stream); break;
+    case 1: launch_gemv_stream_cb1(p, bits, mask, grid, stream); break;
+    default: launch_gemv_stream_cb2(p, bits, mask, grid, stream); break;
+    }
+    hip_ok(hipGetLastError(), "exl3_gemv_stream_kernel launch");
+    char m[16];
+    std::snprintf(m, sizeof m, "0x%x", mask);
+    return "exl3_gemv_stream_kernel<" + std::to_string(bits) + "," + std::to_string(cb) + (p.a_up ? ",silu" : "") +
+           ",table=" + m + "> grid=" + std::to_string(grid.x) + " block=1024 units_per_wave=" + std::to_string(pl.q) +
+           (p.out_fp32 ? " out=f32" : " out=f16");
 }
 
 static int wg_per_cu()
@@ -91,6 +227,21 @@ std::string launch_gemv(const LinearArgs& a)
     if (a.size_k % 128 != 0) throw std::runtime_error("exl3 linear: size_k must be a multiple of 128");
     Workspace& ws = workspace_for_current_device();
     const int mmax = a.size_m == 1 ? 1 : 8;
+    if (a.size_m == 1) {
+        const StreamPlan pl = plan_stream(ws, 1, a.size_k, a.size_n);
+        if (pl.ok) {
+            StreamParams sp{};
+            sp.a = (const _Float16*)a.a;
+            sp.a_up = (const _Float16*)a.a_up;
+            sp.lin[0] = {(const uint32_t*)a.trellis, (const _Float16*)a.suh, (const _Float16*)a.svh};
+            sp.c[0] = a.c;
+            sp.a_had = (_Float16*)a.a_had;
+            sp.K = a.size_k;
+            sp.N = a.size_n;
+            sp.out_fp32 = a.out_fp32;
+            return run_stream(ws, pl, sp, a.k_bits, a.codebook, a.stream);
+        }
+    }
 
     GemvParams p{};
     p.a = (const _Float16*)a.a;
@@ -124,6 +275,22 @@ std::string launch_gemv_pair(const PairArgs& a)
     if (a.size_k % 128 != 0) throw std::runtime_error("exl3 linear: size_k must be a multiple of 128");
     Workspace& ws = workspace_for_current_device();
     const int mmax = a.size_m == 1 ? 1 : 8;
+    if (a.size_m == 1) {
+        const StreamPlan pl = plan_stream(ws, 2, a.size_k, a.size_n);
+        if (pl.ok) {
+            StreamParams sp{};
+            sp.a = (const _Float16*)a.a;
+            for (int i = 0; i < 2; ++i) {
+                sp.lin[i] = {(const uint32_t*)a.trellis[i], (const _Float16*)a.suh[i], (const _Float16*)a.svh[i]};
+                sp.c[i] = a.c[i];
+            }
+            sp.a_had = (_Float16*)a.a_had;
+            sp.K = a.size_k;
+            sp.N = a.size_n;
+            sp.out_fp32 = 0;
+            return "pair " + run_stream(ws, pl, sp, a.k_bits, a.codebook, a.stream);
+        }
+    }
     GemvParams p{};
     p.a = (const _Float16*)a.a;
     p.pair = 1;
@@ -161,6 +328,29 @@ std::string launch_mgemm(const MgemmArgs& m)
     Workspace& ws = workspace_for_current_device();
     const bool sliced = m.had_src_list != nullptr;
     const int mmax = m.size_m == 1 ? 1 : 8;
+    if (m.size_m == 1) {
+        const StreamPlan pl = plan_stream(ws, m.bszm_out, m.size_k, m.size_n);
+        if (pl.ok) {
+            StreamParams sp{};
+            sp.a = (const _Float16*)m.a;
+            sp.c[0] = m.c;
+            sp.a_had = (_Float16*)m.a_had;
+            sp.b_list = (const uint64_t*)m.b_list;
+            sp.suh_list = (const uint64_t*)m.suh_list;
+            sp.svh_list = (const uint64_t*)m.svh_list;
+            sp.c_ptrs = (const uint64_t*)m.c_ptrs;
+            sp.size_n_list = m.size_n_list;
+            sp.n_stride_list = m.n_stride_list;
+            sp.had_src_list = m.had_src_list;
+            sp.mode = sliced ? 2 : 1;
+            sp.in_stride = (!sliced && m.bszm_in > 1) ? m.size_k : 0;
+            sp.K = m.size_k;
+            sp.N = m.size_n;
+            sp.out_fp32 = m.c_fp32;
+            return std::string(sliced ? "sliced x" : "uniform x") + std::to_string(m.bszm_out) + " " +
+                   run_stream(ws, pl, sp, m.k_bits, m.codebook, m.stream);
+        }
+    }
     GemvParams p{};
     p.a = (const _Float16*)m.a;
     p.rows = m.size_m;

@@ -1,0 +1,67 @@
+// Per-codebook instantiations of the one-row streaming GEMV kernel (included by
+// exl3_gemv_stream_cb{0,1,2}.hip with BERTH_GEMV_CB defined): every bit rate, plain and
+// SiLU-gated input, all-arithmetic decode (table mask 0) and the hybrid decode masks.
+#include "exl3_gemv_stream_kernel.cuh"
+#include "launch.h"
+
+namespace berth {
+
+template <int BITS, int CB, bool SILU, int LUTMASK>
+static void launch_stream_one(const StreamParams& p, dim3 grid, hipStream_t stream)
+{
+    constexpr int lds_bytes = stream_lds_bytes(LUTMASK);
+    // the dynamic LDS limit is a per-device attribute of the function
+    static bool raised[64] = {};
+    int device = 0;
+    hip_ok(hipGetDevice(&device), "hipGetDevice");
+    if (device >= 0 && device < 64 && !raised[device]) {
+        hip_ok(hipFuncSetAttribute((const void*)exl3_gemv_stream_kernel<BITS, CB, SILU, LUTMASK>,
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes),
+               "exl3_gemv_stream_kernel: dynamic LDS limit");
+        raised[device] = true;
+    }
+    hipLaunchKernelGGL((exl3_gemv_stream_kernel<BITS, CB, SILU, LUTMASK>), grid, dim3(1024), lds_bytes, stream, p);
+}
+
+template <int BITS, int CB>
+static void launch_stream_bits(const StreamParams& p, int lutmask, dim3 grid, hipStream_t stream)
+{
+    const bool silu = p.a_up != nullptr;
+    switch (lutmask) {
+    case 0x0:
+        if (silu) launch_stream_one<BITS, CB, true, 0x0>(p, grid, stream);
+        else launch_stream_one<BITS, CB, false, 0x0>(p, grid, stream);
+        break;
+#ifdef BERTH_STREAM_EXTRA_MASKS
+    case 0x2: launch_stream_one<BITS, CB, false, 0x2>(p, grid, stream); break;
+    case 0x8: launch_stream_one<BITS, CB, false, 0x8>(p, grid, stream); break;
+    case 0xE: launch_stream_one<BITS, CB, false, 0xE>(p, grid, stream); break;
+    case 0xF: launch_stream_one<BITS, CB, false, 0xF>(p, grid, stream); break;
+#endif
+    default:
+        if (silu) launch_stream_one<BITS, CB, true, 0xA>(p, grid, stream);
+        else launch_stream_one<BITS, CB, false, 0xA>(p, grid, stream);
+        break;
+    }
+}
+
+#define BERTH_CAT2(a, b) a##b
+#define BERTH_CAT(a, b) BERTH_CAT2(a, b)
+
+void BERTH_CAT(launch_gemv_stream_cb, BERTH_GEMV_CB)(const StreamParams& p, int bits, int lutmask, dim3 grid,
+                                                    hipStream_t stream)
+{
+    constexpr int CB = BERTH_GEMV_CB;
+    switch (bits) {
+    case 1: launch_stream_bits<1, CB>(p, lutmask, grid, stream); break;
+    case 2: launch_stream_bits<2, CB>(p, lutmask, grid, stream); break;
+    case 3: launch_stream_bits<3, CB>(p, lutmask, grid, stream); break;
+    case 4: launch_stream_bits<4, CB>(p, lutmask, grid, stream); break;
+    case 5: launch_stream_bits<5, CB>(p, lutmask, grid, stream); break;
+    case 6: launch_stream_bits<6, CB>(p, lutmask, grid, stream); break;
+    case 7: launch_stream_bits<7, CB>(p, lutmask, grid, stream); break;
+    default: launch_stream_bits<8, CB>(p, lutmask, grid, stream); break;
+    }
+}
+
+}  // namespace berth

@@ -1,0 +1,544 @@
+// EXL3 linear for ONE row, as a single resident round of workgroups: one workgroup of
+// sixteen waves per compute unit, every wave a contiguous run of tile rows.
+//
+//   c = ( Hh(x * suh) @ W ) -> Hh(.) * svh          (Hh = 128-block Hadamard / sqrt(128))
+//
+// The operator of crates/berth-kernels/csrc/linear.cu:209-286 at m = 1 (and of the m = 1
+// bundles of crates/berth-kernels/csrc/ops/mgemm.cu:125-272), for weights large enough
+// that every wave gets several tile rows.
+//
+//   * Work of a problem (one linear, or one slice of a bundle) = its (column block, tile
+//     row) units, column block major: U = (N/128) * (K/16) units of `32*bits` bytes per
+//     lane-octet, 8 octets (128 columns) per wave.  The problem's waves split the units
+//     evenly: wave W takes q units, the first `rem` waves one more.  No second round, no
+//     tail of half-empty compute units: the grid is at most the number of compute units
+//     and every wave does the same amount of decode.
+//   * A wave keeps a ring of RING tile rows in registers; a tile row is reloaded with the
+//     tile row RING units ahead as soon as it has been decoded.  The walk crosses column
+//     block boundaries without draining the ring.
+//   * The workgroup rotates the activation of the k-blocks its units touch once, into
+//     LDS (every wave takes some k-blocks), and writes a_had for the k-blocks whose
+//     column-block-0 units it owns.
+//   * Decode is a hybrid: of the four weight pairs of a dword, those selected by LUTMASK
+//     come from a 128 KiB state -> fp16 table in LDS (copied from device memory with
+//     LDS-direct loads while the first tile rows are in flight), the others from the
+//     codebook arithmetic.  The table read costs address + read + pack (2.5 vector
+//     instructions per weight with the dot product) against 4.25 for the arithmetic;
+//     the LDS read rate bounds how many can go that way.
+//   * Partial sums: a wave writes one 128-column partial per column block it touched
+//     into LDS; a column block that lies entirely inside the workgroup's units is
+//     finished there; otherwise the workgroup's partial goes to the library workspace
+//     and the last workgroup to arrive adds the partials in workgroup order.  Every
+//     summation order is fixed by the static split.
+#pragma once
+
+#include "exl3_gemv_kernel.cuh"
+
+#include <utility>
+
+namespace berth {
+
+constexpr int kStreamWaves = 16;
+constexpr int kStreamXsBlocks = 64;        // k-blocks of rotated activation a workgroup can hold
+constexpr int kStreamMaxCb = 15;           // column blocks one workgroup's units can touch
+constexpr int kStreamPieces = kStreamWaves + kStreamMaxCb - 1;
+// dynamic LDS of a launch: [table 128 KiB, if any][rotated activation][partial pieces][piece bounds]
+__host__ __device__ constexpr int stream_lds_bytes(int lutmask)
+{
+    return (lutmask ? 131072 : 0) + kStreamXsBlocks * 256 + kStreamPieces * 512 + 128;
+}
+
+struct StreamParams {
+    const _Float16* a;          // input row(s): fp16 [K] (per problem when in_stride != 0)
+    const _Float16* a_up;       // optional: the input is silu(a) * a_up
+    ExpertLin lin[2];           // mode 0: the problems by value (one linear, or a pair)
+    void* c[2];                 // mode 0 outputs; modes 1, 2: c[0] is the uniform-mode output base
+    // modes 1 (uniform) and 2 (sliced): the device lists of crates/berth-kernels/src/ops.rs:264-293
+    const uint64_t* b_list;
+    const uint64_t* suh_list;
+    const uint64_t* svh_list;
+    const uint64_t* c_ptrs;
+    const int* size_n_list;
+    const int* n_stride_list;
+    const int* had_src_list;
+    _Float16* a_had;            // optional; slab per rotation source
+    const uint16_t* lut;        // [65536] fp16 bits of every state of this codebook (LUTMASK != 0)
+    float* partials;            // [problem][column block][contributor][128]
+    unsigned* counters;         // [problem][column block], zero between launches
+    int mode;                   // 0 by value, 1 uniform lists, 2 sliced lists
+    int in_stride;              // elements between the inputs of consecutive problems (0: shared)
+    int K, N, NB, TR;           // N: row stride of trellis and output in mode 0 / 1; TR = K / 16
+    int out_fp32;
+    int Gp;                     // workgroups per problem (gridDim.x = problems * Gp)
+    unsigned q, rem;            // units per wave; the first `rem` waves of a problem take q + 1
+    unsigned mq, mq1, mtr;      // floor(2^32 / d) + 1 for d = q, q + 1, TR (exact for the operands used)
+    int maxc;                   // contributor slots per column block in `partials`
+#ifdef BERTH_STREAM_TRACE
+    unsigned long long* trace;  // [wave][8] timestamps (instrumented builds only)
+#endif
+};
+
+__device__ __forceinline__ unsigned div_magic(unsigned n, unsigned m) { return __umulhi(n, m); }
+
+// phase timestamps of an instrumented build (a measurement aid; compiled out otherwise)
+#ifdef BERTH_STREAM_TRACE
+#define BERTH_STREAM_STAMP(i)                                                                      \
+    do {                                                                                           \
+        if (lane == 0)                                                                             \
+            p.trace[((size_t)blockIdx.x * kStreamWaves + wave) * 8 + (i)] = wall_clock64(); \
+    } while (0)
+#else
+#define BERTH_STREAM_STAMP(i) do { } while (0)
+#endif
+
+typedef __attribute__((address_space(3))) const uint16_t* lds_u16_ptr;
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+// LDS byte address 2 * s of the table entry of the 16-bit state in the low / high half of r
+__device__ __forceinline__ uint32_t lut_addr_lo(uint32_t r)
+{
+    uint32_t a;
+    asm("v_add_u32_sdwa %0, %1, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_0" : "=v"(a) : "v"(r));
+    return a;
+}
+__device__ __forceinline__ uint32_t lut_addr_hi(uint32_t r)
+{
+    uint32_t a;
+    asm("v_add_u32_sdwa %0, %1, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_1 src1_sel:WORD_1" : "=v"(a) : "v"(r));
+    return a;
+}
+__device__ __forceinline__ uint32_t lut_read(uint32_t addr) { return *(lds_u16_ptr)(uintptr_t)addr; }
+
+__host__ __device__ constexpr int popcount4(int m) { return (m & 1) + ((m >> 1) & 1) + ((m >> 2) & 1) + ((m >> 3) & 1); }
+
+// Decode of a lane's 32 weights of one tile row, some pairs through the table, in three
+// steps so that the table reads are in flight while the other pairs are computed:
+// addresses() fills the table addresses, the caller issues the reads, finish() decodes
+// the arithmetic pairs and packs the table values.
+//
+// 4 bits per weight: pair pp of dword j (w2[4j + pp]) holds the windows that end q bits
+// into the dword's big-endian chunk, pp 0: q = 4, 8; 1: q = 12, 16; 2: q = 20, 24; 3: q =
+// 28, 32.  A funnel shift of (previous chunk : chunk) by 16 - ph leaves the windows ending
+// at q = ph and q = 16 + ph in the two halves of one register, and q = 16 and 32 are the
+// halves of the dword as loaded; a half becomes a table address with one SDWA add.
+// Other bit rates: windows from the shared extraction, address = state << 1; pair p goes
+// through the table when bit (p & 3) of LUTMASK is set.
+template <int BITS, int CB, int LUTMASK>
+struct HybridDecode {
+    static constexpr int kTablePairs = 4 * popcount4(LUTMASK);
+    uint32_t X[BITS == 4 ? 5 : 1];
+    uint32_t m[BITS == 4 ? 4 : 1];
+
+    __device__ __forceinline__ void addresses(const uint32_t (&own)[BITS], uint32_t prev,
+                                              uint32_t (&addr)[kTablePairs ? 2 * kTablePairs : 1])
+    {
+        if constexpr (BITS == 4) {
+            X[0] = __builtin_amdgcn_alignbit(prev, prev, 16);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) X[j + 1] = __builtin_amdgcn_alignbit(own[j], own[j], 16);
+            int n = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t X0 = X[j], X1 = X[j + 1], raw = own[j], rawprev = j == 0 ? prev : own[j - 1];
+                uint32_t r4 = 0, r8 = 0, r12 = 0;
+                if constexpr ((LUTMASK & 1) || (LUTMASK & 4)) {
+                    r4 = __builtin_amdgcn_alignbit(X0, X1, 12);
+                    r8 = __builtin_amdgcn_alignbit(X0, X1, 8);
+                }
+                if constexpr ((LUTMASK & 2) || (LUTMASK & 8)) r12 = __builtin_amdgcn_alignbit(X0, X1, 4);
+                if constexpr (!(LUTMASK & 1) || !(LUTMASK & 2)) m[j] = (rawprev & 0xffff0000u) | (raw & 0x0000ffffu);
+                if constexpr (LUTMASK & 1) { addr[n++] = lut_addr_hi(r4); addr[n++] = lut_addr_hi(r8); }
+                if constexpr (LUTMASK & 2) { addr[n++] = lut_addr_hi(r12); addr[n++] = lut_addr_lo(raw); }
+                if constexpr (LUTMASK & 4) { addr[n++] = lut_addr_lo(r4); addr[n++] = lut_addr_lo(r8); }
+                if constexpr (LUTMASK & 8) { addr[n++] = lut_addr_lo(r12); addr[n++] = lut_addr_hi(raw); }
+            }
+        } else if constexpr (LUTMASK != 0) {
+            LaneWindows<BITS> win(own, prev);
+            int n = 0;
+#pragma unroll
+            for (int p = 0; p < 16; ++p)
+                if ((LUTMASK >> (p & 3)) & 1) {
+                    addr[n++] = win.state(2 * p) << 1;
+                    addr[n++] = win.state(2 * p + 1) << 1;
+                }
+        }
+    }
+
+    __device__ __forceinline__ void finish(const uint32_t (&own)[BITS], uint32_t prev,
+                                           const uint32_t (&t)[kTablePairs ? 2 * kTablePairs : 1], uint32_t (&w2)[16])
+    {
+        if constexpr (LUTMASK == 0) {
+            decode_lane<BITS, CB>(own, prev, w2);
+        } else if constexpr (BITS == 4) {
+            int n = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t X1 = X[j + 1];
+                if constexpr (LUTMASK & 1) { w2[4 * j] = t[n] | (t[n + 1] << 16); n += 2; }
+                else w2[4 * j] = decode_pair<CB>(__builtin_amdgcn_ubfe(m[j], 12, 16), __builtin_amdgcn_ubfe(m[j], 8, 16));
+                if constexpr (LUTMASK & 2) { w2[4 * j + 1] = t[n] | (t[n + 1] << 16); n += 2; }
+                else w2[4 * j + 1] = decode_pair<CB>(__builtin_amdgcn_ubfe(m[j], 4, 16), __builtin_amdgcn_ubfe(X1, 16, 16));
+                if constexpr (LUTMASK & 4) { w2[4 * j + 2] = t[n] | (t[n + 1] << 16); n += 2; }
+                else w2[4 * j + 2] = decode_pair<CB>(__builtin_amdgcn_ubfe(X1, 12, 16), __builtin_amdgcn_ubfe(X1, 8, 16));
+                if constexpr (LUTMASK & 8) { w2[4 * j + 3] = t[n] | (t[n + 1] << 16); n += 2; }
+                else w2[4 * j + 3] = decode_pair<CB>(__builtin_amdgcn_ubfe(X1, 4, 16), __builtin_amdgcn_ubfe(X1, 0, 16));
+            }
+        } else {
+            LaneWindows<BITS> win(own, prev);
+            int n = 0;
+#pragma unroll
+            for (int p = 0; p < 16; ++p) {
+                if ((LUTMASK >> (p & 3)) & 1) { w2[p] = t[n] | (t[n + 1] << 16); n += 2; }
+                else w2[p] = decode_pair<CB>(win.state(2 * p), win.state(2 * p + 1));
+            }
+        }
+    }
+};
+
+// f(0); if more: f(1); ... each call nested inside the previous one's branch
+template <int J, int N, class F>
+__device__ __forceinline__ void nested_tail(unsigned count, F&& f)
+{
+    if constexpr (J < N) {
+        if ((unsigned)J < count) {
+            f(std::integral_constant<int, J>{});
+            nested_tail<J + 1, N>(count, f);
+        }
+    }
+}
+
+#ifndef BERTH_STREAM_RING
+#define BERTH_STREAM_RING 4
+#endif
+template <int BITS> struct StreamRing {
+    static constexpr int depth = BITS <= 4 ? BERTH_STREAM_RING : (BITS <= 6 ? (BERTH_STREAM_RING * 3) / 4 : BERTH_STREAM_RING / 2);
+};
+
+template <int BITS, int CB, bool SILU, int LUTMASK>
+__global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    constexpr int kLutBytes = LUTMASK ? 131072 : 0;       // the table sits at LDS offset 0
+    constexpr int kXsOff = kLutBytes;
+    constexpr int kRedOff = kXsOff + kStreamXsBlocks * 256;
+    constexpr int kMetaOff = kRedOff + kStreamPieces * 512;
+    constexpr int RING = StreamRing<BITS>::depth;
+    constexpr int kRowLoads = BITS % 4 == 0 ? BITS / 4 : (BITS % 2 == 0 ? BITS / 2 : BITS);   // load instructions per tile row
+    uint32_t* const xs = (uint32_t*)(lds + kXsOff);
+    float* const red = (float*)(lds + kRedOff);
+    unsigned* const piece_first = (unsigned*)(lds + kMetaOff);
+    unsigned* const piece_last = piece_first + 16;
+
+    static_assert(sizeof(StreamParams) > 2 * 64 && sizeof(StreamParams) <= 6 * 64, "argument lines touched below");
+    touch_kernel_arguments<3>();
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int prob = blockIdx.x / p.Gp;
+    const int gl = blockIdx.x - prob * p.Gp;
+
+    // ---- this problem's tensors
+    ExpertLin lin = p.lin[p.mode == 0 ? prob : 0];
+    int n_stride = p.N, had_slab = 0, width = p.N;
+    void* cout = p.c[p.mode == 0 ? prob : 0];
+    if (p.mode) {
+        lin.trellis = (const uint32_t*)p.b_list[prob];
+        lin.svh = (const _Float16*)p.svh_list[prob];
+        if (p.mode == 2) {
+            width = p.size_n_list[prob];
+            n_stride = p.n_stride_list[prob];
+            had_slab = p.had_src_list[prob];
+            lin.suh = (const _Float16*)p.suh_list[had_slab];
+            cout = (void*)p.c_ptrs[prob];
+        } else {
+            lin.suh = (const _Float16*)p.suh_list[prob];
+            had_slab = prob;
+            cout = (char*)p.c[0] + (size_t)prob * p.N * (p.out_fp32 ? 4 : 2);
+        }
+    }
+    const bool write_had = p.a_had && (p.mode != 0 || prob == 0);
+
+    // ---- the static split: units of this workgroup and of this wave
+    // (a slice narrower than the bundle's width ends early: its units stop at its last column block)
+    const unsigned TR = (unsigned)p.TR;
+    const unsigned u_end = (unsigned)(width >> 7) * TR;
+    const unsigned W0 = (unsigned)gl * kStreamWaves;
+    const unsigned u0 = min(W0 * p.q + min(W0, p.rem), u_end);
+    const unsigned u1 = min((W0 + kStreamWaves) * p.q + min(W0 + kStreamWaves, p.rem), u_end);
+    if (u0 >= u1) return;
+    const unsigned Ww = W0 + (unsigned)wave;
+    const unsigned uw0 = min(Ww * p.q + min(Ww, p.rem), u_end);
+    const unsigned uw1 = min((Ww + 1) * p.q + min(Ww + 1, p.rem), u_end);
+    const unsigned cb_first = div_magic(u0, p.mtr);
+    const unsigned cb_last = div_magic(u1 - 1, p.mtr);
+    const unsigned ncb = cb_last - cb_first + 1;
+
+    BERTH_STREAM_STAMP(0);
+    if (threadIdx.x < 16) {
+        piece_first[threadIdx.x] = 0xffffffffu;
+        piece_last[threadIdx.x] = 0u;
+    }
+
+    // ---- rotate the k-blocks this workgroup's units touch.  Region A: the k-blocks of the
+    // first column block's units (or all of K); region B, behind it: those of the second
+    // column block's units, which start at k-block 0, when the two do not cover all of K.
+    const unsigned KB = TR >> 3;
+    unsigned a_lo, n_a, n_b;
+    {
+        const unsigned r_lo = u0 - cb_first * TR;
+        if (ncb == 1) {
+            a_lo = r_lo >> 3;
+            n_a = ((u1 - 1 - cb_first * TR) >> 3) - a_lo + 1;
+            n_b = 0;
+        } else {
+            a_lo = r_lo >> 3;
+            n_a = KB - a_lo;
+            n_b = ncb == 2 ? ((u1 - 1 - cb_last * TR) >> 3) + 1 : KB;
+            if (n_b >= a_lo) { a_lo = 0; n_a = KB; n_b = 0; }      // together they cover all of K
+        }
+    }
+    // the activation and scales of this wave's k-blocks (at most 64 / 16 = 4) are requested
+    // ahead of the ring; the rotation itself runs once they are there, with the ring in flight
+    constexpr int kRot = kStreamXsBlocks / kStreamWaves;
+    const global_ptr<const half2_t> xin = (global_ptr<const half2_t>)as_global(p.a + (size_t)prob * p.in_stride);
+    const global_ptr<const half2_t> uin = (global_ptr<const half2_t>)as_global(p.a_up + (size_t)prob * p.in_stride);
+    const global_ptr<const half2_t> sin = (global_ptr<const half2_t>)as_global(lin.suh);
+    half2_t rot_x[kRot], rot_s[kRot], rot_u[kRot];
+#pragma unroll
+    for (int t = 0; t < kRot; ++t) {
+        const unsigned i = (unsigned)wave + t * kStreamWaves;
+        const unsigned ic = i < n_a + n_b ? i : 0u;                     // past the end: any valid k-block, unused
+        const unsigned kb = ic < n_a ? a_lo + ic : ic - n_a;
+        rot_x[t] = xin[kb * 64 + lane];
+        rot_s[t] = sin[kb * 64 + lane];
+        if (SILU) rot_u[t] = uin[kb * 64 + lane];
+    }
+    // ---- the table: 128 KiB from device memory straight into LDS, 8 KiB per wave
+    if constexpr (LUTMASK != 0) {
+        const global_ptr<const unsigned char> src = (global_ptr<const unsigned char>)as_global((const unsigned char*)p.lut);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int off = (wave * 8 + i) * 1024;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + off + lane * 16),
+                                             (lds_void_ptr)(lds + off), 16, 0, 0);
+        }
+    }
+    // A compute unit serves its waves' vector memory requests in arrival order: the bulk loads
+    // of the ring must not get ahead of another wave's few loads above, on which the whole
+    // workgroup waits.  So every wave has issued those before any wave issues its ring.
+    __builtin_amdgcn_s_barrier();
+    BERTH_STREAM_STAMP(1);
+    // ---- ring prologue: the first RING tile rows of this wave
+    constexpr int tile_dw = 8 * BITS;
+    const long row_dw = (long)(n_stride >> 4) * tile_dw;
+    const long wrap_dw = (long)(8 * tile_dw) - (long)(TR - 1) * row_dw;
+    // (a wave without units, possible only behind the end of a narrow slice, reads the
+    // workgroup's first unit and never uses it)
+    const unsigned ufirst = uw0 < uw1 ? uw0 : u0;
+    unsigned cb = div_magic(ufirst, p.mtr);
+    unsigned r = ufirst - cb * TR;
+    const int lane_dw = lane * BITS;
+    global_ptr<const uint32_t> pbase = as_global(lin.trellis) + (long)cb * (8 * tile_dw) + (long)r * row_dw;
+    unsigned p_r = r;                                       // tile row of the unit pbase points at
+    unsigned p_left = uw0 < uw1 ? uw1 - uw0 - 1 : 0u;       // units after it that are still this wave's
+    uint32_t own[RING][BITS];
+#pragma unroll
+    for (int j = 0; j < RING; ++j) {
+        load_tile_dwords<BITS>(pbase + lane_dw, own[j]);
+        const long step = p_left == 0 ? 0 : (p_r == TR - 1 ? wrap_dw : row_dw);
+        pbase += step;
+        p_r = p_left == 0 ? p_r : (p_r == TR - 1 ? 0u : p_r + 1);
+        p_left = p_left == 0 ? 0u : p_left - 1;
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    BERTH_STREAM_STAMP(2);
+    half2_t rotated[kRot];
+#pragma unroll
+    for (int t = 0; t < kRot; ++t) {
+        const unsigned i = (unsigned)wave + t * kStreamWaves;
+        if (i >= n_a + n_b) break;
+        half2_t x = rot_x[t];
+        if (SILU) {
+            x.x = silu_mul_h(x.x, rot_u[t].x);
+            x.y = silu_mul_h(x.y, rot_u[t].y);
+        }
+        float v0 = (float)x.x * (float)rot_s[t].x;
+        float v1 = (float)x.y * (float)rot_s[t].y;
+        had128_wave(v0, v1, lane);
+        rotated[t].x = (_Float16)(v0 * kRsqrt128);
+        rotated[t].y = (_Float16)(v1 * kRsqrt128);
+        xs[i * 64 + lane] = as_u32(rotated[t]);
+    }
+    // The table has to be complete at the barrier; the ring stays in flight.  Vector memory
+    // operations complete in issue order, so "all but the ring's loads" covers the table copy.
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(RING * kRowLoads) : "memory");
+    if (write_had) {
+        // a_had: the workgroup that owns tile row 8 * kb of column block 0 writes k-block kb
+        const global_ptr<half2_t> hout = (global_ptr<half2_t>)as_global(p.a_had + (size_t)had_slab * p.K);
+#pragma unroll
+        for (int t = 0; t < kRot; ++t) {
+            const unsigned i = (unsigned)wave + t * kStreamWaves;
+            if (i >= n_a + n_b) break;
+            const unsigned kb = i < n_a ? a_lo + i : i - n_a;
+            if (u0 <= 8 * kb && 8 * kb < u1) hout[kb * 64 + lane] = rotated[t];
+        }
+    }
+    __syncthreads();
+    BERTH_STREAM_STAMP(3);
+
+    // ---- the walk
+    // LDS byte offset of the rotated activation of tile row r of the current column block
+    const unsigned xoff_wrap = kXsOff + (n_b ? n_a * 256u : 0u) - (n_b ? 0u : a_lo * 256u);   // tile row 0 of a later column block
+    unsigned xoff = kXsOff + (r << 5) - a_lo * 256u;
+    if (cb != cb_first) xoff = xoff_wrap + (r << 5);
+    unsigned piece = (unsigned)wave + (cb - cb_first);
+    unsigned left = uw0 < uw1 ? uw1 - uw0 : 0u;
+    float acc0 = 0.0f, acc1 = 0.0f;
+    const int col = (lane >> 3) * 16 + (lane & 7);
+
+    auto flush = [&](unsigned pc) {
+        red[pc * 128 + col] = acc0;
+        red[pc * 128 + col + 8] = acc1;
+        if (lane == 0) {
+            atomicMin(&piece_first[pc - (unsigned)wave], (unsigned)wave);
+            atomicMax(&piece_last[pc - (unsigned)wave], (unsigned)wave);
+        }
+    };
+
+    // One tile row: table addresses and reads first, the next tile row's load, the
+    // arithmetic pairs while the table reads are in flight, then the dot products.
+    auto stage = [&](uint32_t (&mine)[BITS], bool prefetch) {
+        using Dec = HybridDecode<BITS, CB, LUTMASK>;
+        constexpr int NT = Dec::kTablePairs ? 2 * Dec::kTablePairs : 1;
+        Dec dec;
+        const uint32_t prev = fetch_prev(lane, mine[BITS - 1]);
+        uint32_t addr[NT], t[NT], w2[16];
+        dec.addresses(mine, prev, addr);
+        const uint4* xp = (const uint4*)(lds + xoff);
+        const uint4 xa = xp[0], xb = xp[1];
+        if constexpr (Dec::kTablePairs != 0) {
+#pragma unroll
+            for (int i = 0; i < NT; ++i) t[i] = lut_read(addr[i]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        auto reload = [&]() {
+            if (prefetch) {
+                load_tile_dwords<BITS>(pbase + lane_dw, mine);
+                const long step = p_left == 0 ? 0 : (p_r == TR - 1 ? wrap_dw : row_dw);
+                pbase += step;
+                p_r = p_left == 0 ? p_r : (p_r == TR - 1 ? 0u : p_r + 1);
+                p_left = p_left == 0 ? 0u : p_left - 1;
+            }
+        };
+        // the 4-bit hybrid keeps what it still needs of the tile row in its own registers,
+        // so the reload can go out before the arithmetic pairs
+        if constexpr (BITS == 4 && LUTMASK != 0) {
+            reload();
+            dec.finish(mine, prev, t, w2);
+        } else {
+            dec.finish(mine, prev, t, w2);
+            reload();
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        const uint32_t xk[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+#pragma unroll
+        for (int qq = 0; qq < 16; ++qq) {
+            if (pair_col_half(qq)) acc1 = __builtin_amdgcn_fdot2(as_half2(w2[qq]), as_half2(xk[pair_kk(qq)]), acc1, false);
+            else acc0 = __builtin_amdgcn_fdot2(as_half2(w2[qq]), as_half2(xk[pair_kk(qq)]), acc0, false);
+        }
+        ++r;
+        xoff += 32;
+        if (r == TR) {
+            flush(piece);
+            acc0 = acc1 = 0.0f;
+            ++piece;
+            ++cb;
+            r = 0;
+            xoff = xoff_wrap;
+        }
+    };
+
+    // whole rings: straight-line, one exit, so that the wait before each tile row's use
+    // is exactly "all but the RING - 1 loads issued after it"
+    const unsigned groups = left / RING;
+    for (unsigned g = 0; g < groups; ++g) {
+#pragma unroll
+        for (int j = 0; j < RING; ++j) stage(own[j], true);
+    }
+    // the remaining tile rows (fewer than RING), nested so that each is reached one way only
+    const unsigned tail = left - groups * RING;
+    nested_tail<0, RING - 1>(tail, [&](auto J) { stage(own[decltype(J)::value], false); });
+    BERTH_STREAM_STAMP(4);
+    if (r != 0 && uw0 < uw1) flush(piece);
+    __syncthreads();
+    BERTH_STREAM_STAMP(5);
+
+    // ---- finish the column blocks: wave w takes column blocks cb_first + w, + 16, ...
+    const long pslot = (long)prob * p.NB;
+    for (unsigned cbi = (unsigned)wave; cbi < ncb; cbi += kStreamWaves) {
+        const unsigned cbx = cb_first + cbi;
+        if (cbx * 128u >= (unsigned)width) continue;             // a narrower slice of a bundle: nothing there
+        const unsigned wf = piece_first[cbi], wl = piece_last[cbi];
+        float z0 = 0.0f, z1 = 0.0f;
+        for (unsigned wv = wf; wv <= wl; ++wv) {
+            const float2_t part = *(const float2_t*)&red[(wv + cbi) * 128 + 2 * lane];
+            z0 += part.x;
+            z1 += part.y;
+        }
+        const bool whole = u0 <= cbx * TR && (cbx + 1) * TR <= u1;
+        if (!whole) {
+            // contributors: the workgroups from the owner of the column block's first unit
+            // to the owner of its last unit
+            const unsigned ua = cbx * TR, ub = (cbx + 1) * TR - 1;
+            const unsigned big = p.rem * (p.q + 1);
+            const unsigned wa = ua < big ? div_magic(ua, p.mq1) : p.rem + div_magic(ua - big, p.mq);
+            const unsigned wb = ub < big ? div_magic(ub, p.mq1) : p.rem + div_magic(ub - big, p.mq);
+            const unsigned gf = wa >> 4, count = (wb >> 4) - gf + 1;
+            float* slab = p.partials + ((pslot + cbx) * p.maxc) * 128;
+            union Pair { unsigned long long u; float f[2]; } mine;
+            mine.f[0] = z0;
+            mine.f[1] = z1;
+            __hip_atomic_store((unsigned long long*)(slab + ((unsigned)gl - gf) * 128 + 2 * lane), mine.u, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+            wait_own_stores();
+            unsigned old = 0;
+            if (lane == 0)
+                old = __hip_atomic_fetch_add(p.counters + pslot + cbx, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            old = (unsigned)__builtin_amdgcn_readfirstlane((int)old);
+            if (old != count - 1) continue;
+            if (lane == 0) __hip_atomic_store(p.counters + pslot + cbx, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            z0 = z1 = 0.0f;
+            for (unsigned j0 = 0; j0 < count; j0 += 8) {
+                Pair part[8];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const unsigned j = j0 + t < count ? j0 + t : count - 1;
+                    part[t].u = __hip_atomic_load((const unsigned long long*)(slab + j * 128 + 2 * lane), __ATOMIC_RELAXED,
+                                                  __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int t = 0; t < 8; ++t)
+                    if (j0 + t < count) {
+                        z0 += part[t].f[0];
+                        z1 += part[t].f[1];
+                    }
+            }
+        }
+        // output Hadamard, svh, store
+        const half2_t sv = ((global_ptr<const half2_t>)as_global(lin.svh + cbx * 128))[lane];
+        had128_wave(z0, z1, lane);
+        z0 = (z0 * kRsqrt128) * (float)sv.x;
+        z1 = (z1 * kRsqrt128) * (float)sv.y;
+        const size_t at = (size_t)cbx * 128 + 2 * lane;
+        if (p.out_fp32) {
+            float2_t o = {z0, z1};
+            *(float2_t*)((float*)cout + at) = o;
+        } else {
+            half2_t o = {(_Float16)z0, (_Float16)z1};
+            *(half2_t*)((_Float16*)cout + at) = o;
+        }
+    }
+    BERTH_STREAM_STAMP(6);
+}
+
+}  // namespace berth

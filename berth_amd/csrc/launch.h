@@ -22,12 +22,15 @@ inline void hip_ok(hipError_t e, const char* what)
 struct Workspace {
     float* partials = nullptr;      // kPartialBytes
     unsigned* counters = nullptr;   // kCounters entries, zero between launches
+    uint16_t* state_tables = nullptr;   // [3 codebooks][65536] fp16 bits of every trellis state, or null
     int device = -1;
     int cu_count = 0;
 };
 constexpr size_t kPartialBytes = (size_t)256 << 20;
 constexpr int kCounters = 65536;
 Workspace& workspace_for_current_device();
+// fills tables[cb][s] with the fp16 weight of state s for the three codebooks (synchronous)
+void build_state_tables(uint16_t* tables);
 
 struct LinearArgs {
     const void* a;

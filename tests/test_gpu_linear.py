@@ -447,7 +447,7 @@ def test_lm_head_shape_6bpw_slices_match_oracle():
     K.exl3_linear(d_x.data_ptr(), d_tr.data_ptr(), c.data_ptr(), d_suh.data_ptr(), a_had.data_ptr(),
                   d_svh.data_ptr(), 1, Kk, N, bits, Codebook.MUL1, OutDtype.F16)
     torch.cuda.synchronize()
-    assert "exl3_gemv_kernel<6,2,1>" in K.last_launch()
+    assert "exl3_gemv_stream_kernel<6,2" in K.last_launch()      # a weight this large takes the streaming kernel
     got = host_f16(c)
     for c0 in (0, 124160, N - 256):
         sub = np.ascontiguousarray(tr[:, c0 // 16:c0 // 16 + 16, :])

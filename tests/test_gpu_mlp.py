@@ -29,6 +29,15 @@ def _layer(gpu, H, I, bits, seed, rows):
 @pytest.mark.parametrize("rows,H,I,bits", [(1, 256, 384, 4), (3, 256, 384, 3), (8, 256, 384, 4), (1, 1024, 2816, 4),
                                            (2, 2048, 768, 2), (20, 256, 384, 4), (40, 512, 256, 5)])
 def test_fused_mlp_stage_by_stage(rows, H, I, bits):
+    launch = run_mlp_block(rows, H, I, bits)
+    if rows <= 8:
+        assert launch.count("exl3_gemv_kernel") == 2 and "pair" in launch and ",silu>" in launch
+    else:
+        assert launch.count("exl3_gemm_kernel") == 3 and "silu_mul" in launch
+
+
+def run_mlp_block(rows, H, I, bits):
+    """One berth_exl3_mlp call checked stage by stage against the oracle; returns the launch text."""
     gpu = Gpu(0)
     (gate, up, down), mlp = _layer(gpu, H, I, bits, 9000 + rows, rows)
     x = (synth.activations(9100 + rows, rows, H).astype(np.float32) / np.sqrt(H)).astype(np.float16)
@@ -36,10 +45,6 @@ def test_fused_mlp_stage_by_stage(rows, H, I, bits):
     mlp.forward(gpu, gpu.upload(x.view(np.uint16)), y, rows=rows)
     gpu.synchronize()
     launch = K.last_launch()
-    if rows <= 8:
-        assert launch.count("exl3_gemv_kernel") == 2 and "pair" in launch and ",silu>" in launch
-    else:
-        assert launch.count("exl3_gemm_kernel") == 3 and "silu_mul" in launch
 
     g_want, xh_want = O.linear(x, *gate, H, I, bits, 2)
     u_want, _ = O.linear(x, *up, H, I, bits, 2)
@@ -59,6 +64,7 @@ def test_fused_mlp_stage_by_stage(rows, H, I, bits):
         assert close(act, O.silu_mul(g_want, u_want).reshape(rows, I), rtol=4e-3, atol=2e-3)[0] == 0
     y_want, _ = O.linear(act, *down, I, H, bits, 2, out_fp32=True)
     assert close(y.cpu().numpy(), y_want.reshape(rows, H))[0] == 0
+    return launch
 
 
 def test_fused_mlp_equals_the_four_call_sequence_up_to_summation_order():
