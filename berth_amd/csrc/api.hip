@@ -40,6 +40,8 @@ Workspace& workspace_for_current_device()
         ws.partials = (float*)partials;
         ws.counters = (unsigned*)counters;
         ws.cu_count = cus;
+        ws.partial_bytes = kPartialBytes;
+        ws.counter_slots = kCounters;
         ws.device = device;
     }
     return ws;
@@ -106,6 +108,100 @@ extern "C" int berth_exl3_linear(const void* a, const void* trellis, void* c, co
             throw std::runtime_error("exl3 linear: sizes must be positive");
         check_shape("exl3 linear", args);
         g_exl3_launch = dispatch_linear(args);
+        return 0;
+    } catch (const std::exception& err) {
+        g_exl3_err = err.what();
+        g_exl3_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
+// ---- the entry point that allocates nothing -------------------------------------
+// Split-K scratch of berth_exl3_linear_noalloc: partial sums, then the arrival counters.
+// Every GPU the library runs on holds its own copy until the process ends.  In host code
+// the array's name is only a handle for hipGetSymbolAddress; the device address it
+// returns, kept per device, is what kernels and fills get.
+namespace {
+constexpr size_t kNoAllocPartialBytes = (size_t)8 << 20;
+constexpr int kNoAllocCounters = 65536;
+constexpr size_t kNoAllocBytes = kNoAllocPartialBytes + (size_t)kNoAllocCounters * sizeof(unsigned);
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kNoAllocBytes];
+
+namespace {
+struct NoAllocDevice {
+    unsigned char* ptr = nullptr;   // device address of this device's copy of `scratch`
+    int cu_count = 0;
+    bool cleared = false;           // the counters have been zeroed once on this device
+};
+std::mutex g_noalloc_mu;
+NoAllocDevice g_noalloc[kMaxDevices];
+
+__global__ void fill_zero_u32_kernel(unsigned* p, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+// the scratch of the current device as a Workspace; looks the address up on first use
+Workspace noalloc_scratch_for_current_device(hipStream_t stream)
+{
+    int device = 0;
+    hip_ok(hipGetDevice(&device), "hipGetDevice");
+    if (device < 0 || device >= kMaxDevices) throw std::runtime_error("device index out of range");
+    std::lock_guard<std::mutex> lock(g_noalloc_mu);
+    NoAllocDevice& d = g_noalloc[device];
+    if (!d.ptr) {
+        unsigned char* ptr = nullptr;
+        hip_ok(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+        if (!ptr) throw std::runtime_error("exl3 linear (no allocation): the scratch symbol has no device address");
+        int cus = 0;
+        hip_ok(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device), "multiProcessorCount");
+        d.ptr = ptr;
+        d.cu_count = cus;
+    }
+    unsigned* counters = (unsigned*)(d.ptr + kNoAllocPartialBytes);
+    if (!d.cleared) {
+        // Counters must start at zero; every launch leaves them at zero again (the last
+        // arrival resets its counter).  A fill kernel, not a memset: callers may be capturing.
+        hipLaunchKernelGGL(fill_zero_u32_kernel, dim3((kNoAllocCounters + 255) / 256), dim3(256), 0, stream, counters,
+                           kNoAllocCounters);
+        hip_ok(hipGetLastError(), "scratch counter fill");
+        d.cleared = true;
+    }
+    Workspace ws;
+    ws.partials = (float*)d.ptr;
+    ws.counters = counters;
+    ws.state_tables = nullptr;
+    ws.device = device;
+    ws.cu_count = d.cu_count;
+    ws.partial_bytes = kNoAllocPartialBytes;
+    ws.counter_slots = kNoAllocCounters;
+    ws.strict = true;
+    return ws;
+}
+}  // namespace
+
+extern "C" int berth_exl3_linear_noalloc(const void* a, const void* trellis, void* c, const void* suh,
+                                         void* a_had, const void* svh, int size_m, int size_k, int size_n,
+                                         int k_bits, int codebook, int out_fp32, void* stream)
+{
+    try {
+        g_exl3_err.clear();
+        g_exl3_launch.clear();
+        LinearArgs args{a, trellis, c, suh, a_had, svh, size_m, size_k, size_n,
+                        k_bits, codebook, out_fp32 ? 1 : 0, (hipStream_t)stream};
+        check_linear("exl3 linear (no allocation)", args);
+        if (size_m < 1 || size_k < 1 || size_n < 1)
+            throw std::runtime_error("exl3 linear (no allocation): sizes must be positive");
+        check_shape("exl3 linear (no allocation)", args);
+        if (size_m > 8)
+            throw std::runtime_error("exl3 linear (no allocation): at most 8 rows (more rows need the library's workspace)");
+        if (size_n / 128 > kNoAllocCounters)
+            throw std::runtime_error("exl3 linear (no allocation): size_n exceeds the scratch's counter table");
+        const Workspace ws = noalloc_scratch_for_current_device((hipStream_t)stream);
+        g_exl3_launch = launch_gemv(args, &ws);
         return 0;
     } catch (const std::exception& err) {
         g_exl3_err = err.what();

@@ -126,8 +126,8 @@ static StreamPlan plan_stream(const Workspace& ws, int problems, int K, int N)
     if ((L + TR - 1) / TR + 1 > (unsigned)kStreamMaxCb) return pl;
     if (KB > (unsigned)kStreamXsBlocks && (L + 16 >= TR || L / 8 + 2 > (unsigned)kStreamXsBlocks)) return pl;
     const unsigned maxc = (TR + kStreamWaves * q - 1) / (kStreamWaves * q) + 1;   // workgroups that can share a column block
-    if ((unsigned long long)problems * NB > (unsigned long long)kCounters) return pl;
-    if ((unsigned long long)problems * NB * maxc * 128 * sizeof(float) > kPartialBytes) return pl;
+    if ((unsigned long long)problems * NB > (unsigned long long)ws.counter_slots) return pl;
+    if ((unsigned long long)problems * NB * maxc * 128 * sizeof(float) > ws.partial_bytes) return pl;
     pl.ok = true;
     pl.problems = problems;
     pl.Gp = Gp;
@@ -175,25 +175,27 @@ static std::string run_stream(const Workspace& ws, const StreamPlan& pl, StreamP
 
 static int wg_per_cu()
 {
-    static const int v = [] {
-        const char* e = std::getenv("BERTH_GEMV_WG_PER_CU");
-        int x = e ? std::atoi(e) : 0;
-        return x > 0 ? x : 6;
-    }();
-    return v;
+    const int x = env_int("BERTH_GEMV_WG_PER_CU", 0);
+    return x > 0 ? x : 6;
 }
 
 // split-K factor: about wg_per_cu workgroups per compute unit (2-3 waves per SIMD
 // keep the vector ALU busy; each wave then walks several k-blocks with its loads
 // one k-block ahead), at most one k-block per wave, within the workspace
-static int pick_split(const Workspace& ws, long units, int KB, int mmax)
+static int pick_split(const Workspace& ws, long units, int KB, int mmax, bool trial = false)
 {
     const long target_wg = (long)ws.cu_count * wg_per_cu();
     long S = (target_wg + units / 2) / units;
     const int s_max = (KB + 3) / 4;
     if (S > s_max) S = s_max;
     if (S < 1) S = 1;
-    while (S > 1 && (size_t)units * S * mmax * 128 * sizeof(float) > kPartialBytes) --S;
+    const size_t need = (size_t)units * S * mmax * 128 * sizeof(float);
+    if (S > 1 && need > ws.partial_bytes && ws.strict) {
+        if (trial) return 1 << 30;      // the caller drops this choice
+        throw std::runtime_error("exl3 gemv: this launch needs " + std::to_string(need) +
+                                 " bytes of split-K scratch; the scratch given holds " + std::to_string(ws.partial_bytes));
+    }
+    while (S > 1 && (size_t)units * S * mmax * 128 * sizeof(float) > ws.partial_bytes) --S;
     return (int)S;
 }
 
@@ -211,7 +213,7 @@ static void pick_units(const Workspace& ws, GemvParams& p, long units, int mmax)
     }();
     p.half_units = 0;
     if (allow && mmax == 1 && units * p.KB <= (long)ws.cu_count * 6) {
-        const int S = pick_split(ws, units, 2 * p.KB, mmax);
+        const int S = pick_split(ws, units, 2 * p.KB, mmax, true);
         if (S <= 16) {
             p.half_units = 1;
             p.S = S;
@@ -221,11 +223,11 @@ static void pick_units(const Workspace& ws, GemvParams& p, long units, int mmax)
     p.S = pick_split(ws, units, p.KB, mmax);
 }
 
-std::string launch_gemv(const LinearArgs& a)
+std::string launch_gemv(const LinearArgs& a, const Workspace* scratch)
 {
     if (a.size_m < 1 || a.size_m > 8) throw std::runtime_error("exl3 gemv: rows must be in 1..=8");
     if (a.size_k % 128 != 0) throw std::runtime_error("exl3 linear: size_k must be a multiple of 128");
-    Workspace& ws = workspace_for_current_device();
+    const Workspace& ws = scratch ? *scratch : workspace_for_current_device();
     const int mmax = a.size_m == 1 ? 1 : 8;
     if (a.size_m == 1) {
         const StreamPlan pl = plan_stream(ws, 1, a.size_k, a.size_n);
@@ -259,7 +261,7 @@ std::string launch_gemv(const LinearArgs& a)
     p.NB = a.size_n / 128;
     p.KB = a.size_k / 128;
     p.out_fp32 = a.out_fp32;
-    if (p.NB > kCounters) throw std::runtime_error("exl3 gemv: size_n exceeds the split-K counter table");
+    if (p.NB > ws.counter_slots) throw std::runtime_error("exl3 gemv: size_n exceeds the split-K counter table");
     pick_units(ws, p, p.NB, mmax);
     const int grid = p.NB * p.S;
     launch_bits(p, a.k_bits, a.codebook, mmax, dim3(grid), a.stream);

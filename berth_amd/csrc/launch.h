@@ -25,6 +25,9 @@ struct Workspace {
     uint16_t* state_tables = nullptr;   // [3 codebooks][65536] fp16 bits of every trellis state, or null
     int device = -1;
     int cu_count = 0;
+    size_t partial_bytes = 0;       // capacity of `partials`
+    int counter_slots = 0;          // capacity of `counters`
+    bool strict = false;            // true: a launch that would not fit is refused instead of split less
 };
 constexpr size_t kPartialBytes = (size_t)256 << 20;
 constexpr int kCounters = 65536;
@@ -108,8 +111,9 @@ struct MgemmArgs {
 };
 std::string launch_mgemm(const MgemmArgs& args);
 
-// rows 1..8: VALU dot-product kernel.  Returns the launch description.
-std::string launch_gemv(const LinearArgs& args);
+// rows 1..8: VALU dot-product kernel.  Returns the launch description.  `scratch`: the
+// split-K scratch to use instead of the device's lazily allocated workspace.
+std::string launch_gemv(const LinearArgs& args, const Workspace* scratch = nullptr);
 // any row count: fp16 MFMA kernel (rows padded to 32 inside the kernel).
 std::string launch_gemm(const LinearArgs& args);
 // trellis -> fp16 [K][slice_n] (row stride slice_n), columns n_offset.. of a

@@ -45,6 +45,7 @@ def load() -> C.CDLL:
         L = C.CDLL(LIB_PATH)
         vp, ci = C.c_void_p, C.c_int
         L.berth_exl3_linear.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
+        L.berth_exl3_linear_noalloc.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
         L.berth_prefill_exl3_linear.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, vp]
         L.berth_prefill_hgemm.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, vp]
         L.berth_prefill_reconstruct.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, vp]
@@ -90,6 +91,16 @@ def exl3_linear(a, trellis, c, suh, a_had, svh, size_m, size_k, size_n, k_bits,
                              int(codebook), int(out), stream)
     if rc != 0:
         raise LaunchError(last_error() or f"exl3 linear launch failed ({rc})")
+
+
+def exl3_linear_noalloc(a, trellis, c, suh, a_had, svh, size_m, size_k, size_n, k_bits,
+                        codebook: Codebook, out: OutDtype, stream=None) -> None:
+    """The same operator for callers that cannot allocate device memory (HIP graph capture,
+    tight serving loops): up to 8 rows, split-K scratch in a fixed array inside the library."""
+    rc = load().berth_exl3_linear_noalloc(a, trellis, c, suh, a_had, svh, size_m, size_k, size_n, k_bits,
+                                          int(codebook), int(out), stream)
+    if rc != 0:
+        raise LaunchError(last_error() or f"exl3 linear (no allocation) launch failed ({rc})")
 
 
 class Exl3Lin(C.Structure):

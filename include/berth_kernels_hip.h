@@ -39,6 +39,19 @@ extern "C" {
 int berth_exl3_linear(const void* a, const void* trellis, void* c, const void* suh,
                       void* a_had, const void* svh, int size_m, int size_k, int size_n,
                       int k_bits, int codebook, int out_fp32, void* stream);
+/* The same operator for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
+ * reference (its shim allocates its workspace lazily, crates/berth-kernels/src/lib.rs:116-117).
+ * Allocates nothing: the split-K partial sums and arrival counters live in a fixed array
+ * inside the library (8 MiB + 256 KiB per GPU, held until the process ends).  Same arguments
+ * and conventions as berth_exl3_linear, with these limits: size_m <= 8; a launch whose
+ * split-K partial sums would not fit the 8 MiB is refused with an error (no weight of the
+ * shapes named in this header's tests comes near it at one row); size_n / 128 <= 65536.
+ * Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams)
+ * race, as overlapping calls of berth_exl3_linear do on the library's workspace. */
+int berth_exl3_linear_noalloc(const void* a, const void* trellis, void* c, const void* suh,
+                              void* a_had, const void* svh, int size_m, int size_k, int size_n,
+                              int k_bits, int codebook, int out_fp32, void* stream);
 const char* berth_exl3_last_error(void);   /* ffi.rs:23, linear.cu:396 */
 const char* berth_exl3_last_launch(void);  /* ffi.rs:24, linear.cu:401 */
 

@@ -155,3 +155,17 @@ def test_fused_mlp_validation():
     with pytest.raises(LaunchError, match="1..=8"):
         K.exl3_mlp(P, lins, P, P, P, P, P, 1, 256, 384, 9, Codebook.MUL1)
     assert K.last_launch() == ""
+
+
+def test_no_alloc_linear_validates_before_any_device_call():
+    """berth_exl3_linear_noalloc: the same checks as berth_exl3_linear plus its own limits,
+    all ahead of the first device call (dangling pointers, no GPU needed)."""
+    with pytest.raises(LaunchError, match="null"):
+        K.exl3_linear_noalloc(None, P, P, P, P, P, 1, 128, 256, 4, Codebook.MUL1, OutDtype.F16)
+    with pytest.raises(LaunchError, match="multiple of 128"):
+        K.exl3_linear_noalloc(P, P, P, P, P, P, 1, 128, 100, 4, Codebook.MUL1, OutDtype.F16)
+    with pytest.raises(LaunchError, match="at most 8 rows"):
+        K.exl3_linear_noalloc(P, P, P, P, P, P, 9, 128, 256, 4, Codebook.MUL1, OutDtype.F16)
+    with pytest.raises(LaunchError, match="counter table"):
+        K.exl3_linear_noalloc(P, P, P, P, P, P, 1, 128, 128 * 65537, 4, Codebook.MUL1, OutDtype.F16)
+    assert K.last_launch() == ""
