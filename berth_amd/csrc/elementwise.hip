@@ -202,6 +202,105 @@ std::string launch_rms_norm(const void* x, const void* weight, void* y, void* re
            ",float> block=256 grid=" + std::to_string(rows);
 }
 
+// RMS norm of fp16 rows to fp16 with a bf16 weight and no residual
+// (crates/berth-kernels/src/ops.rs:108-118,600-640, csrc/ops/norm.cu:80-112: the
+// normalisation ahead of the MTP input projection).  The fp16 input widens exactly to
+// fp32; from there the arithmetic is that of rms_norm_kernel.
+__global__ __launch_bounds__(256) void rms_norm_f16_kernel(const _Float16* __restrict__ x, const uint16_t* __restrict__ weight,
+                                                           _Float16* __restrict__ y, int dim, float epsilon,
+                                                           float constant_bias, float constant_scale)
+{
+    __shared__ double s_part[4];
+    __shared__ float s_rmf;
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const half4_t* xr = (const half4_t*)(x + (size_t)row * dim);
+    double ss = 0.0;
+    for (int i = tid; i < dim / 4; i += 256) {
+        const half4_t v = xr[i];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ss += (double)(float)v[j] * (double)(float)v[j];
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) ss += __shfl_xor(ss, d, 64);
+    if ((tid & 63) == 0) s_part[tid >> 6] = ss;
+    __syncthreads();
+    if (tid == 0) {
+        const double total = ((s_part[0] + s_part[1]) + s_part[2]) + s_part[3];
+        s_rmf = (float)(1.0 / sqrt(total / dim + (double)epsilon));
+    }
+    __syncthreads();
+    const float rmf = s_rmf;
+    for (int i = tid; i < dim / 4; i += 256) {
+        const half4_t v = xr[i];
+        half4_t o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float w = __builtin_bit_cast(float, (uint32_t)weight[4 * i + j] << 16);
+            float t = (float)v[j] * rmf;
+            t = t * (w + constant_bias);
+            t = t * constant_scale;
+            o[j] = (_Float16)t;
+        }
+        *(half4_t*)(y + (size_t)row * dim + 4 * i) = o;
+    }
+}
+
+std::string launch_rms_norm_f16(const void* x, const void* weight, void* y, int rows, int dim, float epsilon,
+                                float constant_bias, float constant_scale, hipStream_t stream)
+{
+    hipLaunchKernelGGL(rms_norm_f16_kernel, dim3((unsigned)rows), dim3(256), 0, stream, (const _Float16*)x,
+                       (const uint16_t*)weight, (_Float16*)y, dim, epsilon, constant_bias, constant_scale);
+    hip_ok(hipGetLastError(), "rms_norm_f16 launch");
+    return "rms_norm_kernel<0,half,half,bfloat16,half> block=256 grid=" + std::to_string(rows);
+}
+
+// Embedding rows (crates/berth-kernels/src/ops.rs:99-127, csrc/ops/embed.cu): out[t] =
+// weight[ids[t]], bf16 -> fp32 (an exact widen) or bf16 -> fp16 (the widen, then one
+// round-to-nearest-even).  ids are not range-checked, as in the reference.
+template <bool F16>
+__global__ __launch_bounds__(256) void embed_bf16_kernel(const uint16_t* __restrict__ weight, const int* __restrict__ ids,
+                                                         void* __restrict__ out, int hidden)
+{
+    const int token = blockIdx.x;
+    const uint16_t* row = weight + (size_t)ids[token] * hidden;
+    for (int i = threadIdx.x; i < hidden; i += 256) {
+        const float v = __builtin_bit_cast(float, (uint32_t)row[i] << 16);
+        if (F16) ((_Float16*)out)[(size_t)token * hidden + i] = (_Float16)v;
+        else ((float*)out)[(size_t)token * hidden + i] = v;
+    }
+}
+
+std::string launch_embed_tokens(const void* weight, const int* ids, void* out, int hidden, int n, int f16,
+                                hipStream_t stream)
+{
+    if (f16) hipLaunchKernelGGL(embed_bf16_kernel<true>, dim3((unsigned)n), dim3(256), 0, stream, (const uint16_t*)weight, ids, out, hidden);
+    else hipLaunchKernelGGL(embed_bf16_kernel<false>, dim3((unsigned)n), dim3(256), 0, stream, (const uint16_t*)weight, ids, out, hidden);
+    hip_ok(hipGetLastError(), f16 ? "embed_tokens_f16 launch" : "embed_tokens launch");
+    return std::string(f16 ? "embed_bf16_f16" : "embed_bf16_f32") + " block=256 grid=" + std::to_string(n);
+}
+
+// out[row] = embedding[row] followed by hidden[row], fp16 (crates/berth-kernels/src/ops.rs:136-143,
+// csrc/ops/copy.cu: the concatenation ahead of the MTP input projection)
+__global__ __launch_bounds__(256) void cat_f16_last_kernel(const uint16_t* __restrict__ embedding,
+                                                           const uint16_t* __restrict__ hidden,
+                                                           uint16_t* __restrict__ out, int width)
+{
+    const size_t row = blockIdx.x;
+    for (int i = threadIdx.x; i < width; i += 256) {
+        out[row * 2 * width + i] = embedding[row * width + i];
+        out[row * 2 * width + width + i] = hidden[row * width + i];
+    }
+}
+
+std::string launch_cat_f16_last(const void* embedding, const void* hidden, void* out, int rows, int width,
+                                hipStream_t stream)
+{
+    hipLaunchKernelGGL(cat_f16_last_kernel, dim3((unsigned)rows), dim3(256), 0, stream, (const uint16_t*)embedding,
+                       (const uint16_t*)hidden, (uint16_t*)out, width);
+    hip_ok(hipGetLastError(), "cat_f16_last launch");
+    return "cat_f16_last block=256 grid=" + std::to_string(rows);
+}
+
 // crates/berth-exl3/src/signs.rs:25-46: packed su / sv -> fp16 signs.  Little-endian
 // u16 words, bit i of a word is element i of its 16; a set bit is -1.0 (0xBC00),
 // a clear bit +1.0 (0x3C00).  One thread per output pair.

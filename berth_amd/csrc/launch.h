@@ -132,6 +132,12 @@ std::string launch_add_f32(const void* a, const void* b, void* c, int n, hipStre
 std::string launch_rms_norm(const void* x, const void* weight, void* y, void* residual, int rows, int dim,
                             float epsilon, float constant_bias, float constant_scale, int weight_bf16,
                             hipStream_t stream);
+std::string launch_rms_norm_f16(const void* x, const void* weight, void* y, int rows, int dim, float epsilon,
+                                float constant_bias, float constant_scale, hipStream_t stream);
+std::string launch_embed_tokens(const void* weight, const int* ids, void* out, int hidden, int n, int f16,
+                                hipStream_t stream);
+std::string launch_cat_f16_last(const void* embedding, const void* hidden, void* out, int rows, int width,
+                                hipStream_t stream);
 std::string launch_unpack_signs(const void* packed, void* out, int64_t words, hipStream_t stream);
 std::string launch_silu_mul(const void* gate, const void* up, void* out, int64_t numel,
                             float act_limit, hipStream_t stream);

@@ -55,6 +55,19 @@ def load() -> C.CDLL:
         L.berth_ops_rms_norm.argtypes = [vp, vp, vp, ci, ci, C.c_float, C.c_float, C.c_float, ci, vp]
         L.berth_ops_rms_norm_res_in.argtypes = [vp, vp, vp, vp, ci, ci, C.c_float, C.c_float, C.c_float, ci, vp]
         L.berth_ops_add_f32.argtypes = [vp, vp, vp, ci, vp]
+        L.berth_ops_rms_norm_f16.argtypes = [vp, vp, vp, ci, ci, C.c_float, C.c_float, C.c_float, vp]
+        L.berth_ops_embed_tokens.argtypes = [vp, vp, vp, ci, ci, vp]
+        L.berth_ops_embed_tokens_f16.argtypes = [vp, vp, vp, ci, ci, vp]
+        L.berth_ops_memcpy_d2d.argtypes = [vp, vp, C.c_uint64, vp]
+        L.berth_ops_cat_f16_last.argtypes = [vp, vp, vp, ci, ci, vp]
+        L.berth_exl3_gemm_tune_key.argtypes = [ci] * 9
+        L.berth_exl3_gemm_tune_key.restype = C.c_uint64
+        L.berth_exl3_salt_hash.argtypes = [C.c_uint64]
+        L.berth_exl3_salt_hash.restype = C.c_uint64
+        L.berth_ops_mgemm_tune_key.argtypes = [ci] * 12
+        L.berth_ops_mgemm_tune_key.restype = C.c_uint64
+        L.berth_exl3_gemv_cfg.argtypes = [ci] * 8
+        L.berth_exl3_smoke_int8.argtypes = [ci]
         L.berth_exl3_unpack_signs.argtypes = [vp, vp, C.c_int64, vp]
         L.berth_exl3_mlp.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         L.berth_exl3_unpack_signs.restype = C.c_int
@@ -226,6 +239,34 @@ class ops:
                                               constant_scale, int(weight_bf16), stream)
         if rc != 0:
             raise LaunchError(ops.last_error() or f"rms_norm_res_in launch failed ({rc})")
+
+    @staticmethod
+    def rms_norm_f16(x, weight, y, rows: int, dim: int, epsilon: float, constant_bias: float = 1.0,
+                     constant_scale: float = 1.0, stream=None) -> None:
+        """crates/berth-kernels/src/ops.rs:600-640."""
+        rc = load().berth_ops_rms_norm_f16(x, weight, y, rows, dim, epsilon, constant_bias, constant_scale, stream)
+        if rc != 0:
+            raise LaunchError(ops.last_error() or f"rms_norm_f16 launch failed ({rc})")
+
+    @staticmethod
+    def embed_tokens(weight, ids, out, hidden: int, n: int, f16: bool = False, stream=None) -> None:
+        """crates/berth-kernels/src/ops.rs:554-598 (bf16 rows to fp32, or to fp16)."""
+        fn = load().berth_ops_embed_tokens_f16 if f16 else load().berth_ops_embed_tokens
+        rc = fn(weight, ids, out, hidden, n, stream)
+        if rc != 0:
+            raise LaunchError(ops.last_error() or f"embed_tokens launch failed ({rc})")
+
+    @staticmethod
+    def memcpy_d2d(dst, src, nbytes: int, stream=None) -> None:
+        rc = load().berth_ops_memcpy_d2d(dst, src, nbytes, stream)
+        if rc != 0:
+            raise LaunchError(ops.last_error() or f"memcpy_d2d failed ({rc})")
+
+    @staticmethod
+    def cat_f16_last(embedding, hidden, out, rows: int, hidden_size: int, stream=None) -> None:
+        rc = load().berth_ops_cat_f16_last(embedding, hidden, out, rows, hidden_size, stream)
+        if rc != 0:
+            raise LaunchError(ops.last_error() or f"cat_f16_last launch failed ({rc})")
 
     @staticmethod
     def add_f32(a, b, c, n: int, stream=None) -> None:

@@ -55,6 +55,24 @@ int berth_exl3_linear_noalloc(const void* a, const void* trellis, void* c, const
 const char* berth_exl3_last_error(void);   /* ffi.rs:23, linear.cu:396 */
 const char* berth_exl3_last_launch(void);  /* ffi.rs:24, linear.cu:401 */
 
+/* Host-only symbols of the reference boundary, kept so that the unchanged crate links and
+ * its known-answer tests hold; nothing on this device consumes their results.
+ * tune keys (crates/berth-kernels/src/ffi.rs:33-46, src/ops.rs:40-53; csrc/linear.cu:347-360,
+ * csrc/ops/mgemm.cu:276-294, csrc/autotune.cu:61-66): the reference's shape-tuner cache keys.
+ * gemv_cfg (crates/berth-kernels/src/prefill_lin.rs:69-78, csrc/prefill_lin/gemv.cu:71-99):
+ * which QTIP GEMV configuration the reference's rows-2..8 route would take (0, 1, or -1).
+ * smoke (ffi.rs:29-30, csrc/linear.cu:404-465): one small one-row linear on buffers the
+ * function allocates and frees itself (4 bpw 128x256, and 6 bpw 128x512); 0 on success. */
+uint64_t berth_exl3_gemm_tune_key(int size_m, int size_k, int size_n, int k_bits, int out_fp32, int device,
+                                  int cc, int sms, int codebook);
+uint64_t berth_exl3_salt_hash(uint64_t hash);
+uint64_t berth_ops_mgemm_tune_key(int size_m, int size_k, int size_n, int k_bits, int c_fp32, int device, int cc,
+                                  int sms, int codebook, int bszm_in, int bszm_out, int sliced);
+int berth_exl3_gemv_cfg(int cc, int size_m, int size_k, int size_n, int k_bits, int codebook, int mode,
+                        int narrow_coresident);
+int berth_exl3_smoke_int8(int out_fp32);
+int berth_exl3_smoke_gemm(void);
+
 /* crates/berth-kernels/csrc/linear.cu:301-332.  cc is the gfx target number
  * (950 on MI355X); sms is the compute-unit count. */
 int berth_device_cc(int device);
@@ -121,6 +139,20 @@ int berth_ops_rms_norm_res_in(const void* x, const void* weight, void* y, void* 
 /* replaces crates/berth-kernels/src/ops.rs:91-97,522-552 / csrc/ops/add.cu: c = a + b, fp32,
  * n elements; c may alias a. */
 int berth_ops_add_f32(const void* a, const void* b, void* c, int n, void* stream);
+/* replaces crates/berth-kernels/src/ops.rs:108-118,600-640 / csrc/ops/norm.cu:80-112,163-190: the
+ * same norm for fp16 rows with a bf16 weight, fp16 out, no residual. */
+int berth_ops_rms_norm_f16(const void* x, const void* weight, void* y, int rows, int dim, float epsilon,
+                           float constant_bias, float constant_scale, void* stream);
+/* The remaining device entries of the reference's ops module, glue either side of the
+ * linear path, so that the unchanged Rust module links (crates/berth-kernels/src/ops.rs:99-143 /
+ * csrc/ops/embed.cu, csrc/ops/copy.cu): embedding rows bf16 [vocab][hidden] -> fp32 (exact
+ * widen) or fp16 (one rounding) for n token ids (not range-checked); device-to-device copy;
+ * out[row] = embedding[row] ++ hidden[row] in fp16. */
+int berth_ops_embed_tokens(const void* weight, const int* ids, void* out, int hidden, int n, void* stream);
+int berth_ops_embed_tokens_f16(const void* weight, const int* ids, void* out, int hidden, int n, void* stream);
+int berth_ops_memcpy_d2d(void* dst, const void* src, unsigned long long bytes, void* stream);
+int berth_ops_cat_f16_last(const void* embedding, const void* hidden, void* out, int rows, int hidden_size,
+                           void* stream);
 /* replaces crates/berth-kernels/src/ops.rs:17-38,247-367 / csrc/ops/mgemm.cu:296-340:
  * several EXL3 linears in one launch.  Every list is a DEVICE array.  Sliced
  * mode (all four slice lists given, bszm_in == 1): bszm_out slices sharing the

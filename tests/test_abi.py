@@ -169,3 +169,69 @@ def test_no_alloc_linear_validates_before_any_device_call():
     with pytest.raises(LaunchError, match="counter table"):
         K.exl3_linear_noalloc(P, P, P, P, P, P, 1, 128, 128 * 65537, 4, Codebook.MUL1, OutDtype.F16)
     assert K.last_launch() == ""
+
+
+def test_every_symbol_the_reference_crate_binds_for_the_path_is_exported():
+    """tests/golden/reference_extern_symbols.json lists what the reference's `extern "C"` blocks
+    declare (crates/berth-kernels/src/{ffi,prefill_lin,ops}.rs): with all of them exported the
+    unchanged Rust modules link against libberth_kernels_hip.so."""
+    import json
+    lib = K.load()
+    listed = json.load(open(os.path.join(ROOT, "tests", "golden", "reference_extern_symbols.json")))
+    declared = set(_declared("berth_kernels_hip.h"))
+    names = [n for entry in listed.values() for kind in ("always", "test_only") for n in entry[kind]]
+    assert len(names) == 25
+    for name in names:
+        assert hasattr(lib, name), name
+        assert name in declared, f"{name} is exported but not declared in include/berth_kernels_hip.h"
+
+
+def test_tune_keys_reproduce_the_reference_known_answers():
+    """crates/berth-kernels/src/lib.rs:223-233 (lm_head key and its salted form) and
+    src/ops.rs:738-770 (the two 27B bundle keys): pure host hashes, no device call."""
+    lib = K.load()
+    key = lib.berth_exl3_gemm_tune_key(1, 5120, 248320, 6, 0, 0, 2, 82, int(Codebook.MUL1))
+    assert key == 0x51F40C1BD7CAE3A7
+    assert lib.berth_exl3_salt_hash(key) == 0x0C94364FADC0CDF9
+    assert lib.berth_ops_mgemm_tune_key(1, 5120, 2048, 4, 1, 0, 2, 82, int(Codebook.MUL1), 1, 8, 1) == 0xD2297A8A33A33F5B
+    assert lib.berth_ops_mgemm_tune_key(1, 5120, 1024, 4, 0, 0, 2, 82, int(Codebook.MUL1), 1, 14, 1) == 0x9C25A0752178FB4A
+    # m = 1 shares the m = 2 entry of the single-linear key; the bundle key keeps m = 1 apart
+    assert lib.berth_exl3_gemm_tune_key(2, 5120, 248320, 6, 0, 0, 2, 82, 2) == key
+    assert lib.berth_ops_mgemm_tune_key(2, 5120, 2048, 4, 1, 0, 2, 82, 2, 1, 8, 1) != 0xD2297A8A33A33F5B
+
+
+def test_gemv_cfg_table_of_the_reference():
+    """The rows of crates/berth-kernels/src/prefill_lin.rs:385-442 (cc 2 = Ampere, 3 = Ada,
+    mode 1, 4 bpw, mul1, 164 co-resident narrow workgroups)."""
+    cfg = K.load().berth_exl3_gemv_cfg
+    AMPERE, ADA, MODE, BITS, CB, NARROW = 2, 3, 1, 4, 2, 164
+    for m in (3, 5, 8):
+        assert cfg(AMPERE, m, 5120, 17408, BITS, CB, MODE, NARROW) == -1      # gate / up
+        assert cfg(AMPERE, m, 17408, 5120, BITS, CB, MODE, NARROW) == 0       # down
+        assert cfg(AMPERE, m, 6144, 5120, BITS, CB, MODE, NARROW) == 0        # o_proj
+        assert cfg(AMPERE, m, 10240, 5120, BITS, CB, MODE, NARROW) == 0       # mtp.fc
+    assert cfg(AMPERE, 9, 17408, 5120, BITS, CB, MODE, NARROW) == -1
+    assert cfg(AMPERE, 2, 17408, 5120, BITS, CB, MODE, NARROW) == 0
+    assert cfg(AMPERE, 3, 17408, 5120, BITS, CB, 0, NARROW) == -1
+    assert cfg(AMPERE, 3, 5120, 8192, BITS, CB, MODE, NARROW) == 1
+    assert cfg(ADA, 3, 5120, 8192, BITS, CB, MODE, NARROW) == -1
+    # forced modes and the other bit rates
+    assert cfg(AMPERE, 3, 5120, 8192, BITS, CB, 2, NARROW) == 0 and cfg(AMPERE, 3, 5120, 8320, BITS, CB, 2, NARROW) == 1
+    assert cfg(AMPERE, 3, 5120, 17408, BITS, CB, 3, NARROW) == 0 and cfg(AMPERE, 3, 5120, 1024, BITS, CB, 4, NARROW) == 1
+    assert cfg(AMPERE, 3, 5120, 17408, 2, CB, MODE, NARROW) == 1 and cfg(AMPERE, 3, 5120, 17408, 5, CB, MODE, NARROW) == -1
+    assert cfg(AMPERE, 3, 5120, 17408, 3, 0, MODE, NARROW) == -1 and cfg(AMPERE, 3, 5100, 17408, BITS, CB, MODE, NARROW) == -1
+
+
+def test_glue_ops_validate_before_any_device_call():
+    """Messages of crates/berth-kernels/csrc/ops/{embed,copy,norm}.cu, with dangling pointers."""
+    with pytest.raises(LaunchError, match="embed_tokens: null device pointer"):
+        K.ops.embed_tokens(None, P, P, 16, 1)
+    with pytest.raises(LaunchError, match="embed_tokens_f16: hidden and n must be positive"):
+        K.ops.embed_tokens(P, P, P, 0, 1, f16=True)
+    with pytest.raises(LaunchError, match="memcpy_d2d: byte count is 0"):
+        K.ops.memcpy_d2d(P, P, 0)
+    with pytest.raises(LaunchError, match="cat_f16_last: rows and hidden must be positive"):
+        K.ops.cat_f16_last(P, P, P, 0, 8)
+    with pytest.raises(LaunchError, match="rms_norm: dim must be a multiple of 4"):
+        K.ops.rms_norm_f16(P, P, P, 1, 6, 1e-6)
+    assert K.ops.last_launch() == ""
