@@ -58,9 +58,22 @@ def build_all(jobs: int = 8, only: str | None = None) -> list[str]:
             raise RuntimeError(f"link failed for {name}:\n{r.stderr[-4000:]}")
         built.append(out)
     if only is None:
+        built.append(build_code_object())
         built.append(build_reader())
         built.append(build_host_check())
     return built
+
+
+def build_code_object() -> str:
+    """A stand-alone gfx950 code object (hipcc --genco) with the test kernels the runtime
+    library's module path is exercised with (tests/test_gpu_runtime.py)."""
+    out = os.path.join(LIB, "runtime_probe.hsaco")
+    cmd = [HIPCC, "--genco", "--offload-arch=gfx950", "-O3", "-ffp-contract=off",
+           os.path.join(CSRC, "probe", "runtime_probe.hip"), "-o", out]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"code object build failed:\n{r.stderr[-4000:]}")
+    return out
 
 
 def build_reader() -> str:
