@@ -8,6 +8,7 @@
 #include "../../include/berth_kernels_hip.h"
 
 #include <cstdlib>
+#include <cstring>
 #include <initializer_list>
 #include <mutex>
 
@@ -40,12 +41,39 @@ Workspace& workspace_for_current_device()
         hip_ok(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device), "multiProcessorCount");
         ws.partials = (float*)partials;
         ws.counters = (unsigned*)counters;
+        void* fault_host = nullptr;
+        void* fault_dev = nullptr;
+        hip_ok(hipHostMalloc(&fault_host, 64, hipHostMallocMapped), "fault word");
+        *(volatile unsigned*)fault_host = 0u;
+        hip_ok(hipHostGetDevicePointer(&fault_dev, fault_host, 0), "fault word device address");
+        ws.fault_host = (volatile unsigned*)fault_host;
+        ws.fault_dev = (unsigned*)fault_dev;
         ws.cu_count = cus;
         ws.partial_bytes = kPartialBytes;
         ws.counter_slots = kCounters;
         ws.device = device;
     }
     return ws;
+}
+
+void throw_pending_device_fault(const Workspace& ws)
+{
+    if (!ws.fault_host) return;
+    const unsigned code = *ws.fault_host;
+    if (code == 0u) return;
+    *ws.fault_host = 0u;
+    throw std::runtime_error(
+        "an earlier launch on this device gave up waiting for the split-K partial sums of tile " +
+        std::to_string(code - 1u) +
+        " and left it unwritten (the library's workspace serves one launch at a time per device: launches "
+        "that overlap on two streams mix their counters); this call launched nothing");
+}
+
+unsigned spin_limit()
+{
+    const char* e = std::getenv("BERTH_SPIN_LIMIT");
+    const long v = e ? std::strtol(e, nullptr, 0) : 0;
+    return v > 0 ? (unsigned)v : (1u << 20);
 }
 
 namespace {
@@ -214,6 +242,44 @@ extern "C" int berth_exl3_linear_noalloc(const void* a, const void* trellis, voi
 
 extern "C" const char* berth_exl3_last_error(void) { return g_exl3_err.c_str(); }
 extern "C" const char* berth_exl3_last_launch(void) { return g_exl3_launch.c_str(); }
+
+// Allocates the per-device internals of `device` now (workspace, counters, state tables,
+// fault word) instead of at the first launch: for callers whose first launch must not
+// allocate or synchronise (it would, for instance, fail inside a stream capture).
+extern "C" int berth_kernels_init(int device)
+{
+    try {
+        g_exl3_err.clear();
+        int before = 0;
+        hip_ok(hipGetDevice(&before), "hipGetDevice");
+        hip_ok(hipSetDevice(device), "hipSetDevice");
+        (void)workspace_for_current_device();
+        hip_ok(hipSetDevice(before), "hipSetDevice");
+        return 0;
+    } catch (const std::exception& err) {
+        g_exl3_err = err.what();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
+// Diagnostics: the per-device internals (allocated on first use), for tools that inspect or
+// reset the split-K state.
+extern "C" int berth_kernels_workspace(void** partials, size_t* partial_bytes, void** counters, int* counter_slots)
+{
+    try {
+        const Workspace& ws = workspace_for_current_device();
+        if (partials) *partials = ws.partials;
+        if (partial_bytes) *partial_bytes = ws.partial_bytes;
+        if (counters) *counters = ws.counters;
+        if (counter_slots) *counter_slots = ws.counter_slots;
+        return 0;
+    } catch (const std::exception& err) {
+        g_exl3_err = err.what();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
 
 extern "C" int berth_device_cc(int device)
 {

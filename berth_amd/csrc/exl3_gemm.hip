@@ -48,8 +48,11 @@ std::string launch_gemm(const LinearArgs& a)
 {
     if (a.size_k % 128 != 0) throw std::runtime_error("exl3 linear: size_k must be a multiple of 128");
     Workspace& ws = workspace_for_current_device();
+    throw_pending_device_fault(ws);
     std::string d0 = launch_had_r_128(a.a, a.a_had, a.suh, 1, a.size_m, a.size_k, 0, a.stream);
     GemmParams p{};
+    p.fault = ws.fault_dev;
+    p.spin_limit = spin_limit();
     p.a_had[0] = (const _Float16*)a.a_had;
     p.lin.trellis = (const uint32_t*)a.trellis;
     p.lin.svh = (const _Float16*)a.svh;
@@ -134,7 +137,10 @@ std::string launch_gemm_grouped(const GroupedArgs& g)
     if (g.size_k % 128 != 0 || g.size_n % 128 != 0)
         throw std::runtime_error("moe grouped linear: sizes must be multiples of 128");
     Workspace& ws = workspace_for_current_device();
+    throw_pending_device_fault(ws);
     GemmParams p{};
+    p.fault = ws.fault_dev;
+    p.spin_limit = spin_limit();
     p.a_had[0] = (const _Float16*)g.a_had;
     p.a_had[1] = (const _Float16*)g.a_had2;
     p.c[0] = g.c0;

@@ -15,16 +15,16 @@ static void gemm_launch_mb(const GemmParams& p, hipStream_t stream, std::string&
     const size_t smem_z = (size_t)32 * (256 + 4) * sizeof(float);
     const size_t smem = smem_a > smem_z ? smem_a : smem_z;
     if (smem > 64 * 1024) {
-        static const hipError_t attr = hipFuncSetAttribute((const void*)exl3_gemm_kernel<BITS, CB, MB>,
-                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        hip_ok(attr, "exl3_gemm_kernel shared-memory attribute");
+        static bool raised[64] = {};
+        raise_dynamic_lds_limit((const void*)exl3_gemm_kernel<BITS, CB, MB>, (int)smem, raised,
+                                "exl3_gemm_kernel shared-memory attribute");
     }
     if (p.units > 0) {
         // balanced dense launch (128-row tiles only): two workgroups per compute unit
         if constexpr (MB == 4) {
-            static const hipError_t attr2 = hipFuncSetAttribute((const void*)exl3_gemm_balanced_kernel<BITS, CB, MB>,
-                                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-            hip_ok(attr2, "exl3_gemm_balanced_kernel shared-memory attribute");
+            static bool raised2[64] = {};
+            raise_dynamic_lds_limit((const void*)exl3_gemm_balanced_kernel<BITS, CB, MB>, (int)smem, raised2,
+                                    "exl3_gemm_balanced_kernel shared-memory attribute");
             hipLaunchKernelGGL((exl3_gemm_balanced_kernel<BITS, CB, MB>), grid, dim3(256), smem, stream, p);
             desc = "exl3_gemm_balanced_kernel<" + std::to_string(BITS) + "," + std::to_string(CB) + "," +
                    std::to_string(BM) + "x256> grid=" + std::to_string(grid.x) + " units=" + std::to_string(p.units) +
@@ -44,9 +44,9 @@ template <int BITS, int CB>
 static void gemm_launch_wide(const GemmParams& p, hipStream_t stream, std::string& desc, dim3 grid)
 {
     if (p.units <= 0) throw std::runtime_error("exl3 gemm: 256-row tiles exist only as balanced launches");
-    static const hipError_t attr = hipFuncSetAttribute((const void*)exl3_gemm_wide_kernel<BITS, CB>,
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kWideSmem);
-    hip_ok(attr, "exl3_gemm_wide_kernel shared-memory attribute");
+    static bool raised[64] = {};
+    raise_dynamic_lds_limit((const void*)exl3_gemm_wide_kernel<BITS, CB>, kWideSmem, raised,
+                            "exl3_gemm_wide_kernel shared-memory attribute");
     hipLaunchKernelGGL((exl3_gemm_wide_kernel<BITS, CB>), grid, dim3(512), kWideSmem, stream, p);
     desc = "exl3_gemm_wide_kernel<" + std::to_string(BITS) + "," + std::to_string(CB) + ",256x256> grid=" +
            std::to_string(grid.x) + " units=" + std::to_string(p.units) + " max_parts=" + std::to_string(p.max_parts) +

@@ -54,7 +54,25 @@ struct GemmParams {
     int units;                  // tiles * K/128; 0: not a balanced launch
     int unit_q, unit_r;         // units = unit_q * gridDim.x + unit_r
     int max_parts;              // upper bound of workgroups that share one tile
+    // A tile's finisher waits for the other sharers' partial sums with a bound: after
+    // spin_limit polls it gives up, zeroes the tile's counters, stores 1 + the tile's counter
+    // index to *fault (host-visible memory; may be null) and leaves the tile unwritten.
+    unsigned* fault;
+    unsigned spin_limit;
 };
+
+// The finisher's wait for `counter` to reach `want`, bounded.  Called by one thread.  A
+// workgroup that has arrived is running and depends on nothing, so the counter gets there
+// within microseconds unless the counters were left inconsistent (two launches sharing the
+// workspace at once, a launch that was aborted); then this ends the wait instead of hanging.
+__device__ __forceinline__ bool wait_counter_bounded(unsigned* counter, unsigned want, unsigned limit)
+{
+    for (unsigned polls = 0; __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want; ++polls) {
+        if (polls >= limit) return false;
+        __builtin_amdgcn_s_sleep(2);
+    }
+    return true;
+}
 
 // the k-blocks of one tile that a workgroup accumulates, and its place among the
 // workgroups that share the tile
@@ -305,12 +323,15 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
             return;
         }
         if (threadIdx.x == 0) {
-            while (__hip_atomic_load(written, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != (unsigned)(kr.parts - 1))
-                __builtin_amdgcn_s_sleep(2);
+            const bool complete = wait_counter_bounded(written, (unsigned)(kr.parts - 1), p.spin_limit);
             __hip_atomic_store(written, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (!complete && p.fault)
+                __hip_atomic_store(p.fault, 1u + (unsigned)kr.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            s_last = complete ? 1u : 2u;
         }
         __syncthreads();
+        if (s_last == 2u) return;       // gave up: the tile stays unwritten, the host is told
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         if (active) {
             // part 0 first (from memory unless it is this workgroup's own), then parts 1, 2, ...

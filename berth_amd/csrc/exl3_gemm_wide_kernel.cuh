@@ -214,12 +214,15 @@ __device__ __forceinline__ void gemm_tile_wide(const GemmParams& p, const int ti
             return;
         }
         if (threadIdx.x == 0) {
-            while (__hip_atomic_load(written, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != (unsigned)(kr.parts - 1))
-                __builtin_amdgcn_s_sleep(2);
+            const bool complete = wait_counter_bounded(written, (unsigned)(kr.parts - 1), p.spin_limit);
             __hip_atomic_store(written, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (!complete && p.fault)
+                __hip_atomic_store(p.fault, 1u + (unsigned)kr.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            s_last = complete ? 1u : 2u;
         }
         __syncthreads();
+        if (s_last == 2u) return;       // gave up: the tile stays unwritten, the host is told
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         if (active) {
             constexpr int kGroup = 4;                           // (mb, f) register blocks per batch

@@ -10,16 +10,9 @@ template <int BITS, int CB, bool SILU, int LUTMASK>
 static void launch_stream_one(const StreamParams& p, dim3 grid, hipStream_t stream)
 {
     constexpr int lds_bytes = stream_lds_bytes(LUTMASK);
-    // the dynamic LDS limit is a per-device attribute of the function
     static bool raised[64] = {};
-    int device = 0;
-    hip_ok(hipGetDevice(&device), "hipGetDevice");
-    if (device >= 0 && device < 64 && !raised[device]) {
-        hip_ok(hipFuncSetAttribute((const void*)exl3_gemv_stream_kernel<BITS, CB, SILU, LUTMASK>,
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes),
-               "exl3_gemv_stream_kernel: dynamic LDS limit");
-        raised[device] = true;
-    }
+    raise_dynamic_lds_limit((const void*)exl3_gemv_stream_kernel<BITS, CB, SILU, LUTMASK>, lds_bytes, raised,
+                            "exl3_gemv_stream_kernel: dynamic LDS limit");
     hipLaunchKernelGGL((exl3_gemv_stream_kernel<BITS, CB, SILU, LUTMASK>), grid, dim3(1024), lds_bytes, stream, p);
 }
 

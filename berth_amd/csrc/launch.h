@@ -15,6 +15,17 @@ inline void hip_ok(hipError_t e, const char* what)
         throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
 }
 
+// Raises the dynamic-LDS limit of a kernel once per device (the attribute is kept per
+// device; a function-local static would set it on the first device only).
+inline void raise_dynamic_lds_limit(const void* kernel, int bytes, bool (&done)[64], const char* what)
+{
+    int device = 0;
+    hip_ok(hipGetDevice(&device), "hipGetDevice");
+    if (device < 0 || device >= 64 || done[device]) return;
+    hip_ok(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes), what);
+    done[device] = true;
+}
+
 // Per-device scratch owned by the library, allocated on first use and kept for
 // the life of the process: split-K partial sums and their arrival counters
 // (the role of the fixed workspace of
@@ -25,6 +36,11 @@ struct Workspace {
     uint16_t* state_tables = nullptr;   // [3 codebooks][65536] fp16 bits of every trellis state, or null
     int device = -1;
     int cu_count = 0;
+    // One word of host-pinned memory that kernels can write (device address fault_dev, host
+    // address fault_host): a split-K finisher that gives up its bounded wait stores a code
+    // there; the next launch of such a kernel on the device reports it and clears it.
+    unsigned* fault_dev = nullptr;
+    volatile unsigned* fault_host = nullptr;
     size_t partial_bytes = 0;       // capacity of `partials`
     int counter_slots = 0;          // capacity of `counters`
     bool strict = false;            // true: a launch that would not fit is refused instead of split less
@@ -32,6 +48,10 @@ struct Workspace {
 constexpr size_t kPartialBytes = (size_t)256 << 20;
 constexpr int kCounters = 65536;
 Workspace& workspace_for_current_device();
+// throws if a kernel of an earlier launch on this device reported a fault (and clears the report)
+void throw_pending_device_fault(const Workspace& ws);
+// polls a split-K finisher spends on its wait before it gives up (BERTH_SPIN_LIMIT, default 2^20)
+unsigned spin_limit();
 // fills tables[cb][s] with the fp16 weight of state s for the three codebooks (synchronous)
 void build_state_tables(uint16_t* tables);
 

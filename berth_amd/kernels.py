@@ -86,6 +86,7 @@ def load() -> C.CDLL:
         L.berth_moe_workspace_offsets.argtypes = [ci] * 6 + [C.POINTER(C.c_size_t)]
         L.berth_moe_last_error.restype = C.c_char_p
         L.berth_moe_last_launch.restype = C.c_char_p
+        L.berth_kernels_workspace.argtypes = [C.POINTER(vp), C.POINTER(C.c_size_t), C.POINTER(vp), C.POINTER(ci)]
         L.berth_device_cc.argtypes = [ci]
         L.berth_device_sms.argtypes = [ci]
         _lib = L

@@ -73,6 +73,21 @@ int berth_exl3_gemv_cfg(int cc, int size_m, int size_k, int size_n, int k_bits, 
 int berth_exl3_smoke_int8(int out_fp32);
 int berth_exl3_smoke_gemm(void);
 
+/* No counterpart in the reference (its shim allocates lazily, crates/berth-kernels/src/lib.rs:116-117):
+ * allocates the per-device internals of `device` now rather than inside the first launch,
+ * which would otherwise allocate and synchronise (and fail under stream capture). */
+int berth_kernels_init(int device);
+
+/* Diagnostics, no counterpart in the reference: the per-device internals of the current
+ * device (allocated by this call if no launch has done so yet): the split-K partial-sum
+ * workspace and the arrival-counter table (zero between launches).  Any out pointer may be
+ * NULL.  The internals serve one launch at a time per device: launches that overlap on two
+ * streams mix their partial sums and counters.  A tile finisher of the MFMA kernels that
+ * finds its counters inconsistent gives up after a bounded wait (BERTH_SPIN_LIMIT polls,
+ * default 2^20), leaves its tile unwritten and the next call that would launch an MFMA
+ * kernel on the device returns -1 with that report instead of launching. */
+int berth_kernels_workspace(void** partials, size_t* partial_bytes, void** counters, int* counter_slots);
+
 /* crates/berth-kernels/csrc/linear.cu:301-332.  cc is the gfx target number
  * (950 on MI355X); sms is the compute-unit count. */
 int berth_device_cc(int device);

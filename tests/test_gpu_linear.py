@@ -573,3 +573,40 @@ def test_linear_from_packed_signs():
     torch.cuda.synchronize()
     want, _ = O.linear(x, tr, suh, svh, Kk, N, bits, 2, out_fp32=True)
     assert close(c.cpu().numpy(), want.ravel())[0] == 0
+
+
+def _window_check(name, Kk, N, bits, out_fp32, seed):
+    """One row through berth_exl3_linear at a 27B shape; three 256-column windows (first,
+    middle, last) against the oracle on the matching trellis slices, a_had bit-exact."""
+    tr, suh, svh = synth.linear(seed, Kk, N, bits)
+    x = synth.activations(seed + 1, 1, Kk)
+    d_tr, d_suh, d_svh, d_x = dev(tr), dev(suh.view(np.uint16)), dev(svh.view(np.uint16)), dev(x.view(np.uint16))
+    a_had = torch.zeros(Kk, dtype=torch.float16, device=DEV)
+    c = torch.zeros(N, dtype=torch.float32 if out_fp32 else torch.float16, device=DEV)
+    K.exl3_linear(d_x.data_ptr(), d_tr.data_ptr(), c.data_ptr(), d_suh.data_ptr(), a_had.data_ptr(),
+                  d_svh.data_ptr(), 1, Kk, N, bits, Codebook.MUL1, OutDtype.F32 if out_fp32 else OutDtype.F16)
+    launch = K.last_launch()
+    torch.cuda.synchronize()
+    got = c.cpu().numpy() if out_fp32 else host_f16(c)
+    want_had = None
+    for c0 in (0, (N // 512) * 256, N - 256):
+        sub = np.ascontiguousarray(tr[:, c0 // 16:c0 // 16 + 16, :])
+        want, want_had = O.linear(x, sub, suh, svh[c0:c0 + 256], Kk, 256, bits, 2, out_fp32=out_fp32)
+        bad, worst = close(got[c0:c0 + 256], want.reshape(-1))
+        assert bad == 0, (name, bits, c0, bad, worst, launch)
+    assert np.array_equal(host_u16(a_had), want_had.view(np.uint16).reshape(-1)), (name, launch)
+
+
+@pytest.mark.parametrize("name", ["q_proj", "o_proj", "down_proj"])
+def test_27b_shapes_batch1_4bpw_windows_match_oracle(name):
+    """BASELINE configs[1] at 4 bpw, the shapes the other full-size tests leave out."""
+    Kk, N = synth.SHAPES_27B[name]
+    _window_check(name, Kk, N, 4, name != "q_proj", 7100 + Kk % 97)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 5])
+@pytest.mark.parametrize("name", ["gate_proj", "down_proj"])
+def test_27b_shapes_batch1_other_rates_windows_match_oracle(name, bits):
+    """BASELINE configs[1] at 2, 3 and 5 bpw on the two large shapes."""
+    Kk, N = synth.SHAPES_27B[name]
+    _window_check(name, Kk, N, bits, name == "down_proj", 7200 + 10 * bits + Kk % 97)

@@ -202,6 +202,29 @@ def test_moe_config3_shape_decode_token():
     assert np.abs(out.cpu().numpy() - want).max() <= 2e-3 * np.abs(want).max()
 
 
+def test_moe_config3_shape_batch64():
+    """BASELINE configs[3] at 64 tokens (hidden 2048, 128 experts, top-8, intermediate 768,
+    4 bpw) at full size: the whole layer against the oracle, stage by stage and end to end."""
+    gpu = Gpu(0)
+    T, H, E, k, I, bits = 64, 2048, 128, 8, 768, 4
+    wr, experts_np, experts, _, _ = _make_layer(gpu, 61, H, E, I, bits)
+    layer = MoeLayer(gpu, wr, experts, k)
+    x = (synth.activations(62, T, H).astype(np.float32) / np.sqrt(H)).astype(np.float16)
+    out = torch.zeros((T, H), dtype=torch.float32, device=DEV)
+    idx = torch.zeros((T, k), dtype=torch.int32, device=DEV)
+    w = torch.zeros((T, k), dtype=torch.float32, device=DEV)
+    layer.forward(gpu, dev(x.view(np.uint16)), out, T, idx, w)
+    torch.cuda.synchronize()
+    launch = K.moe.last_launch()
+    want, oi, ow = O.moe_layer(x, wr, experts_np, k, I, bits, 2)
+    assert np.array_equal(idx.cpu().numpy(), oi), launch
+    assert len(np.unique(oi)) > 100                          # nearly every expert is hit
+    assert np.allclose(w.cpu().numpy(), ow, rtol=1e-5, atol=1e-7)
+    _check_stages(layer, x, experts_np, None, oi, w.cpu().numpy(), out.cpu().numpy(), T, H, E, k, I, bits, 0)
+    assert np.abs(out.cpu().numpy() - want).max() <= 2e-3 * np.abs(want).max(), launch
+    assert "exl3_gemm_kernel" in launch
+
+
 def test_moe_config4_shape_zipf_shared():
     """hidden 2048, 512 experts top-10 plus an always-on shared expert, intermediate
     512, 3 bpw, 256 tokens, Zipf(1.1)-biased router: skewed problem list (hot
