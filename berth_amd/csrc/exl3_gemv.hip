@@ -415,6 +415,11 @@ std::string launch_gemv_grouped(const GroupedArgs& g)
     const long units = (long)g.max_problems * g.num_lins * p.NB;
     if (units > kCounters) throw std::runtime_error("moe grouped linear: too many (problem, column block) units");
     const int mmax = g.single_row ? 1 : 8;
+    if (g.route_params) {
+        if (!g.single_row || g.a_up || g.gather_div < 1)
+            throw std::runtime_error("moe grouped linear: the inline routing serves the one-token gate / up launch");
+        p.route = *(const RouteParams*)g.route_params;
+    }
     if (g.comb_out) {
         if (!g.single_row || g.num_lins != 1 || !g.out_fp32 || !g.a_up || !g.comb_w || !g.comb_inv || g.comb_k < 1)
             throw std::runtime_error("moe grouped linear: the folded combine needs one-row problems of a silu-input fp32 linear");
@@ -433,7 +438,7 @@ std::string launch_gemv_grouped(const GroupedArgs& g)
     return "exl3_gemv_kernel<" + std::to_string(g.k_bits) + "," + std::to_string(g.codebook) + "," +
            std::to_string(mmax) + "> grouped grid=" +
            std::to_string(grid.x) + "x" + std::to_string(grid.y) + " split_k=" + std::to_string(p.S) + (p.half_units ? "/half" : "") +
-           (g.comb_out ? " +combine" : "");
+           (g.comb_out ? " +combine" : "") + (g.route_params ? " +route" : "");
 }
 
 }  // namespace berth

@@ -10,7 +10,11 @@ namespace berth {
 template <int BITS, int CB>
 static void launch_rows(const GemvParams& p, int mmax, dim3 grid, hipStream_t stream)
 {
-    if (p.half_units && mmax == 1) {
+    if (p.route.parts) {
+        // one-token gate / up launch of an MoE layer with the routing's last part inline
+        if (p.half_units) hipLaunchKernelGGL((exl3_gemv_kernel<BITS, CB, 1, false, 4, true>), grid, dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((exl3_gemv_kernel<BITS, CB, 1, false, 8, true>), grid, dim3(256), 0, stream, p);
+    } else if (p.half_units && mmax == 1) {
         if (p.a_up) hipLaunchKernelGGL((exl3_gemv_kernel<BITS, CB, 1, true, 4>), grid, dim3(256), 0, stream, p);
         else hipLaunchKernelGGL((exl3_gemv_kernel<BITS, CB, 1, false, 4>), grid, dim3(256), 0, stream, p);
     } else if (p.a_up && mmax == 1) hipLaunchKernelGGL((exl3_gemv_kernel<BITS, CB, 1, true>), grid, dim3(256), 0, stream, p);

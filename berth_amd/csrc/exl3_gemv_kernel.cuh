@@ -22,6 +22,7 @@
 
 #include "exl3_decode.cuh"
 #include "hadamard.cuh"
+#include "moe_route.cuh"
 
 namespace berth {
 
@@ -30,14 +31,6 @@ struct ExpertLin {
     const uint32_t* trellis;
     const _Float16* suh;
     const _Float16* svh;
-};
-
-// one unit of grouped work: rows [row0, row0 + nrows) of the expert-sorted order
-struct GroupProblem {
-    int expert;
-    int row0;
-    int nrows;
-    int pad;
 };
 
 struct GemvParams {
@@ -90,6 +83,11 @@ struct GemvParams {
     float* comb_out;
     unsigned* comb_counters;    // [NB], zero between launches
     int comb_k;
+    // grouped mode, one token, ROUTE instantiation: there is no problem list yet; problem i is
+    // the selected expert with sorted position i, which every wave works out itself from the
+    // router's segment sums (route.parts); the first workgroup's first wave stores the routing
+    // results for the launches that follow.  route.k (+ 1 with an always-on expert) problems.
+    RouteParams route;
 };
 
 // silu(g) * u with every step rounded to fp16: e = exp(-g); s = 1 + e; r = 1 / s;
@@ -254,14 +252,14 @@ __device__ __forceinline__ void gemv_accumulate(const GemvWalk& w, const int (&s
     }
 }
 
-template <int BITS, int CB, int MMAX, bool SILU, int TRS = 8>
+template <int BITS, int CB, int MMAX, bool SILU, int TRS = 8, bool ROUTE = false>
 __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
 {
     __shared__ uint32_t xs[4][MMAX][64];    // wave-private: rotated k-block, one half2 per entry
     __shared__ float red[4][MMAX][128];
     __shared__ unsigned s_last;
 
-    static_assert(sizeof(GemvParams) > 5 * 64, "the argument block spans six lines");
+    static_assert(sizeof(GemvParams) > 5 * 64, "the argument block spans at least six lines");
     touch_kernel_arguments<6>();
     const int lane = threadIdx.x & 63;
     // wave-uniform on purpose: everything derived from it (k-block, addresses) stays in SGPRs
@@ -275,7 +273,18 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
 
     ExpertLin lin = p.pair ? p.shared[which] : p.lin;
     int row0 = 0, rows = p.rows;
-    if (p.problems) {
+    auto expert_lin = [&](int expert) -> ExpertLin {
+        return expert == p.shared_expert ? p.shared[p.lin_base + which]
+                                         : p.experts[expert * p.lins_per_expert + p.lin_base + which];
+    };
+    if constexpr (ROUTE) {
+        static_assert(MMAX == 1 && !SILU, "the inline routing serves the one-token gate / up launch");
+        const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && wave == 0;
+        const int expert = route_finish_one_token(p.route, lane, prob, writer);
+        lin = expert_lin(expert);
+        row0 = prob;
+        rows = 1;
+    } else if (p.problems) {
         // the list holds an entry for every problem index of the grid: this one is read
         // together with the count, not after it (one dependent read less ahead of the
         // first weight load); the empty asm keeps the compiler from sinking the read
@@ -284,8 +293,7 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
         const int count = *p.num_problems;
         asm volatile("" ::"s"(gp.expert), "s"(count));
         if (prob >= count) return;
-        lin = gp.expert == p.shared_expert ? p.shared[p.lin_base + which]
-                                           : p.experts[gp.expert * p.lins_per_expert + p.lin_base + which];
+        lin = expert_lin(gp.expert);
         row0 = gp.row0;
         rows = gp.nrows;
     }
@@ -321,7 +329,7 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
 #pragma unroll
     for (int m = 0; m < MMAX; ++m) {
         int r = row0 + in_row0 + (m < rows ? m : 0);
-        src[m] = p.gather ? p.gather[r] / p.gather_div : r;
+        src[m] = ROUTE ? 0 : (p.gather ? p.gather[r] / p.gather_div : r);
     }
 
     float acc[MMAX][2];

@@ -104,6 +104,9 @@ struct GroupedArgs {
     // VALU path, single_row, one linear, fp32 out, silu input: also combine the
     // problems' rows into comb_out[size_n] (weights comb_w[comb_k], rows
     // comb_inv[comb_k] of c0, start value comb_shared[size_n] or zero)
+    // VALU path, single_row, first launch of a one-token layer: RouteParams of the routing whose
+    // last part every workgroup redoes for itself (the problem list does not exist yet)
+    const void* route_params = nullptr;
     const float* comb_w = nullptr;
     const int32_t* comb_inv = nullptr;
     const float* comb_shared = nullptr;

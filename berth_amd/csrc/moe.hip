@@ -21,163 +21,11 @@
 
 namespace berth {
 
-constexpr int kRouteSeg = 64;       // rows of the router weight per partial sum
-constexpr int kRouteTT = 4;         // tokens per route workgroup
-constexpr int kMaxExperts = 1024;
-constexpr int kMaxTopK = 32;
 constexpr int kValuPairs = 8;       // calls with one token or at most this many rows use the VALU kernel only
 constexpr int kGemmRows = 32;       // rows per small MFMA problem
 constexpr int kGemmBigRows = 128;   // rows per big MFMA problem
 
 // ------------------------------------------------------------------ route
-
-struct PermuteParams {
-    const int32_t* idx;     // [P] expert of each (token, slot) pair, P = T * k; distinct within a token
-    int32_t* offsets;       // [E + 1]
-    int32_t* perm;          // [R] sorted position -> pair (pair / k = token)
-    int32_t* inv;           // [P] pair -> sorted position
-    int32_t* row_expert;    // [R] sorted position -> expert
-    int32_t* counts;        // [3] number of VALU problems, small MFMA problems, big MFMA problems
-    GroupProblem* vprob;
-    GroupProblem* mprob;    // <= 32 rows each
-    GroupProblem* bprob;    // <= 128 rows each
-    int T, k, E;
-    int use_valu;           // 1: every expert is one VALU problem (<= 8 rows each); 0: MFMA problems: an
-                            // expert's rows go to big problems of 128 and the rest to small ones of <= 32
-    int shared_rows;        // 1: rows P .. P + T - 1 belong to an always-on expert with index E (token order)
-    int big_min;            // a remainder of at least this many rows becomes a (partial) big problem
-};
-
-struct RouteParams {
-    const _Float16* x;      // [T][H]
-    const _Float16* wr;     // [H][E]
-    const float* bias;      // [E] or null
-    float* parts;           // [T][nseg][E]
-    unsigned* counters;     // [ceil(T / kRouteTT)]
-    int32_t* idx;           // [T][k]
-    float* w;               // [T][k]
-    float* logits;          // [T][E] or null
-    int T, H, E, k, nseg, renorm;
-    // one token only: the wave that selected the experts also sorts them and writes
-    // what the permute kernel would (sort.perm != nullptr), saving its launch
-    PermuteParams sort;
-};
-
-// Top-k of one token by one wave: lane holds the logits of experts lane + 64 i.
-// Largest first, ties to the lowest expert index; weights exp(l - max) normalised
-// over the selected k (renorm) or over all experts.
-constexpr int kRoutePer = kMaxExperts / 64;
-
-__device__ __forceinline__ float lane_value(float v, int lane_index)
-{
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane_index));
-}
-
-// the same value in every lane: butterflies over lane distances 1 .. 32
-__device__ __forceinline__ float wave_max(float v)
-{
-    v = fmaxf(v, lane_xor_dpp<1>(v));
-    v = fmaxf(v, lane_xor_dpp<2>(v));
-    v = fmaxf(v, lane_xor_dpp<4>(v));
-    v = fmaxf(v, lane_xor_dpp<8>(v));
-    v = fmaxf(v, lane_xor_swap16(v));
-    return fmaxf(v, lane_xor_swap32(v));
-}
-// PER: how many of the lane's registers can hold experts (ceil(E / 64) rounded up to 2, 8 or 16)
-template <int PER>
-__device__ __forceinline__ int route_topk_n(const float (&lg)[kRoutePer], int lane, const RouteParams& p, int t)
-{
-    unsigned taken = 0;
-    float sel_logit = 0.0f;         // lane j keeps the logit of slot j
-    int sel_idx = 0;
-    // One slot per round: the largest remaining logit of the wave (max butterflies), then the
-    // lowest expert index among the registers that hold it (ballots).  One short reduction of
-    // one value instead of a reduction of (value, index) pairs with a tie rule.
-    for (int j = 0; j < p.k; ++j) {
-        float lv = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < PER; ++i)
-            if (lane + 64 * i < p.E && !((taken >> i) & 1u)) lv = fmaxf(lv, lg[i]);
-        const float bv = wave_max(lv);
-        // the lowest expert index that holds it: register i of lane l is expert l + 64 i, so
-        // the first register with a holder wins and, inside it, the lowest lane (a ballot
-        // and a find-first-set on the scalar side instead of a second butterfly chain)
-        int bi = 0x7fffffff;
-#pragma unroll
-        for (int i = PER - 1; i >= 0; --i) {
-            const unsigned long long holders =
-                __builtin_amdgcn_ballot_w64(lane + 64 * i < p.E && !((taken >> i) & 1u) && lg[i] == bv);
-            if (holders) bi = 64 * i + __builtin_ctzll(holders);
-        }
-        if ((bi & 63) == lane) taken |= 1u << (bi >> 6);
-        if (lane == j) { sel_logit = bv; sel_idx = bi; }
-    }
-    // lane j is wave-uniform here: v_readlane instead of a round trip through the LDS crossbar
-    const float mx = lane_value(sel_logit, 0);
-    float ev = (lane < p.k) ? expf(sel_logit - mx) : 0.0f;
-    float denom = 0.0f;
-    if (p.renorm) {
-        for (int j = 0; j < p.k; ++j) denom += lane_value(ev, j);       // slot order
-    } else {
-        float loc = 0.0f;
-#pragma unroll
-        for (int i = 0; i < PER; ++i)
-            if (lane + 64 * i < p.E) loc += expf(lg[i] - mx);
-#pragma unroll
-        for (int d = 32; d >= 1; d >>= 1) loc += __shfl_xor(loc, d, 64);
-        denom = loc;
-    }
-    if (lane < p.k) {
-        p.idx[(size_t)t * p.k + lane] = sel_idx;
-        p.w[(size_t)t * p.k + lane] = ev / denom;
-    }
-    return sel_idx;     // lane j < k: expert of slot j
-}
-
-__device__ __forceinline__ int route_topk(const float (&lg)[kRoutePer], int lane, const RouteParams& p, int t)
-{
-    if (p.E <= 128) return route_topk_n<2>(lg, lane, p, t);         // workgroup-uniform
-    if (p.E <= 512) return route_topk_n<8>(lg, lane, p, t);
-    return route_topk_n<kRoutePer>(lg, lane, p, t);
-}
-
-// One token: what moe_permute_kernel writes, by the wave that holds the selection
-// (lane j < k has the expert of slot j; the k experts are distinct).  Sorted position
-// of slot j = number of selected experts with a smaller index; every expert is one
-// single-row VALU problem; an always-on expert (shared_rows) takes row k.
-__device__ __forceinline__ void route_sort_one_token(const PermuteParams& q, int lane, int sel_idx)
-{
-    const int k = q.k;
-    int rank = 0;
-    for (int j = 0; j < k; ++j) {
-        const int other = __builtin_amdgcn_readlane(sel_idx, j);
-        rank += (lane < k && other < sel_idx) ? 1 : 0;
-    }
-    if (lane < k) {
-        q.perm[rank] = lane;
-        q.inv[lane] = rank;
-        q.row_expert[rank] = sel_idx;
-        q.vprob[rank] = GroupProblem{sel_idx, rank, 1, 0};
-    }
-    // offsets[e] = number of selected experts below e
-    for (int e0 = 0; e0 <= q.E; e0 += 64) {         // wave-uniform loop: every lane takes part in the exchanges
-        const int e = e0 + lane;
-        int below = 0;
-        for (int j = 0; j < k; ++j) below += (__builtin_amdgcn_readlane(sel_idx, j) < e) ? 1 : 0;
-        if (e <= q.E) q.offsets[e] = below;
-    }
-    if (lane == 0) {
-        if (q.shared_rows) {
-            q.perm[k] = 0;
-            q.row_expert[k] = q.E;
-            q.vprob[k] = GroupProblem{q.E, k, 1, 0};
-        }
-        q.counts[0] = k + (q.shared_rows ? 1 : 0);
-        q.counts[1] = 0;
-        q.counts[2] = 0;
-    }
-}
-
 
 __global__ __launch_bounds__(256) void moe_route_kernel(RouteParams p)
 {
@@ -327,6 +175,38 @@ __global__ __launch_bounds__(1024) void moe_route_one_token_kernel(RouteParams p
     }
     const int sel = route_topk(lg, lane, p, 0);
     if (p.sort.perm) route_sort_one_token(p.sort, lane, sel);
+}
+
+// One token and a small router, first part only: workgroup `seg` (one wave) leaves the sums
+// of its 64 rows in parts[seg][e].  The routing's last part (ordered sum of the segments,
+// top-k, sort) is then redone by every workgroup of the gate / up launch for itself
+// (route_finish_one_token), which costs less than one workgroup doing it once and all the
+// others waiting for its launch to end.  Same fma chains as moe_route_one_token_kernel.
+__global__ __launch_bounds__(64) void moe_route_segments_kernel(RouteParams p)
+{
+    const int lane = threadIdx.x;
+    const int seg = blockIdx.x;
+    const int pairs = p.E >> 1;
+    const int col = min(lane, pairs - 1);
+    const global_ptr<const uint32_t> wr = (global_ptr<const uint32_t>)as_global((const uint32_t*)p.wr);
+    const int h0 = seg * kRouteSeg;
+    const int hn = min(kRouteSeg, p.H - h0);
+    const float xv = lane < hn ? (float)p.x[h0 + lane] : 0.0f;
+    uint32_t wv[kRouteSeg];
+#pragma unroll
+    for (int i = 0; i < kRouteSeg; ++i) wv[i] = wr[(size_t)(h0 + min(i, hn - 1)) * pairs + col];
+    float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kRouteSeg; ++i) {
+        const float xi = lane_value(xv, i);
+        const half2_t w2 = as_half2(wv[i]);
+        a0 = __builtin_fmaf(xi, (float)w2.x, a0);
+        a1 = __builtin_fmaf(xi, (float)w2.y, a1);
+    }
+    if (lane < pairs) {
+        float2_t o = {a0, a1};
+        *(float2_t*)(p.parts + (size_t)seg * p.E + 2 * lane) = o;
+    }
 }
 
 // Many tokens: the same arithmetic in two launches, so that the segment sums of a
@@ -714,6 +594,14 @@ bool fold_combine_enabled()
     return v;
 }
 
+// One token with a small router: the routing's last part runs inside the gate / up launch
+// (BERTH_MOE_INLINE_ROUTE=0 keeps the single-workgroup routing kernel).
+bool inline_route_enabled()
+{
+    const char* e = std::getenv("BERTH_MOE_INLINE_ROUTE");
+    return !e || std::atoi(e) != 0;
+}
+
 // The always-on expert runs as one more expert of the grouped launches (rows P ..
 // P + T - 1, token order) when it has the routed experts' intermediate size.
 bool shared_is_folded(int I, int shared_I) { return shared_I > 0 && shared_I == I; }
@@ -965,8 +853,27 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
                 throw std::runtime_error("moe layer: null shared-expert pointer");
 
     const PermuteParams pp = permute_params(idx, wsb, L, T, k, E, fold);
-    desc += run_route(x, wr, bias, idx, w, nullptr, (float*)(wsb + L.parts), T, H, E, k, renorm, stream, &pp);
-    if (T > 1) desc += " + " + run_permute(pp, stream);
+    RouteParams inline_route{};
+    const bool route_inline = T == 1 && E % 2 == 0 && E <= kRouteOneMaxE && L.nseg <= kRouteOneMaxSeg && L.max_v > 0 &&
+                              inline_route_enabled();
+    if (route_inline) {
+        RouteParams& r = inline_route;
+        r.x = (const _Float16*)x;
+        r.wr = (const _Float16*)wr;
+        r.bias = bias;
+        r.parts = (float*)(wsb + L.parts);
+        r.idx = idx;
+        r.w = w;
+        r.T = 1; r.H = H; r.E = E; r.k = k; r.renorm = renorm;
+        r.nseg = L.nseg;
+        r.sort = pp;
+        hipLaunchKernelGGL(moe_route_segments_kernel, dim3(L.nseg), dim3(64), 0, stream, r);
+        hip_ok(hipGetLastError(), "moe_route_segments_kernel launch");
+        desc += "moe_route_segments_kernel grid=" + std::to_string(L.nseg) + " (top-k and sort inside the next launch)";
+    } else {
+        desc += run_route(x, wr, bias, idx, w, nullptr, (float*)(wsb + L.parts), T, H, E, k, renorm, stream, &pp);
+        if (T > 1) desc += " + " + run_permute(pp, stream);
+    }
 
     GroupedArgs g{};
     g.experts = experts;
@@ -994,7 +901,9 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
         g.problems = wsb + L.vprob;
         g.num_problems = (const int*)(wsb + L.counts);
         g.max_problems = L.max_v;
+        g.route_params = route_inline ? &inline_route : nullptr;
         desc += " + " + launch_gemv_grouped(g);
+        g.route_params = nullptr;
     }
     if (L.max_m > 0) {
         HadRowsParams h{};

@@ -319,3 +319,34 @@ def test_moe_validation_errors():
         K.moe.layer(None, None, None, None, None, None, None, None, None, 0, 1, 128, 8, 2, 128, 0, 4, K.Codebook.MUL1)
     with pytest.raises(K.LaunchError, match="top-k"):
         K.moe.route(1, 1, None, 1, 1, None, 1, 1, 128, 4, 5)
+
+
+def test_moe_one_token_inline_routing_equals_the_routing_kernel():
+    """One token, at most 128 experts: by default only the router's 64-row segment sums come
+    from a launch of their own and every workgroup of the gate / up launch redoes the ordered
+    sum, the top-k and the sort for itself; BERTH_MOE_INLINE_ROUTE=0 keeps the routing kernel.
+    Same arithmetic in the same order: the same experts, weights and output bits."""
+    import os
+    gpu = Gpu(0)
+    for H, E, k, I, bits, shared_I in ((2048, 128, 8, 768, 4, 0), (512, 16, 4, 256, 3, 256), (1024, 64, 6, 384, 4, 512)):
+        wr, _, experts, _, shared = _make_layer(gpu, 8800 + H + E, H, E, I, bits, shared_I)
+        layer = MoeLayer(gpu, wr, experts, k, shared=shared, bias=synth.zipf_bias(3, E))
+        x = (synth.activations(8801 + H, 1, H).astype(np.float32) / np.sqrt(H)).astype(np.float16)
+        d_x = dev(x.view(np.uint16))
+        res = {}
+        for mode in ("1", "0"):
+            os.environ["BERTH_MOE_INLINE_ROUTE"] = mode
+            try:
+                out = torch.zeros((1, H), dtype=torch.float32, device=DEV)
+                idx = torch.full((1, k), -1, dtype=torch.int32, device=DEV)
+                w = torch.zeros((1, k), dtype=torch.float32, device=DEV)
+                layer.forward(gpu, d_x, out, 1, idx, w)
+                torch.cuda.synchronize()
+                res[mode] = (out.cpu().numpy().view(np.uint32), idx.cpu().numpy(), w.cpu().numpy().view(np.uint32),
+                             K.moe.last_launch())
+            finally:
+                del os.environ["BERTH_MOE_INLINE_ROUTE"]
+        assert "moe_route_segments_kernel" in res["1"][3] and "+route" in res["1"][3], res["1"][3]
+        assert "moe_route_one_token_kernel" in res["0"][3] and "+route" not in res["0"][3], res["0"][3]
+        for a, b in zip(res["1"][:3], res["0"][:3]):
+            assert np.array_equal(a, b), (H, E, res["1"][3])
