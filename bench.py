@@ -156,6 +156,35 @@ def valu_ceiling(bits: int):
             "implied_frac_of_hbm_peak": round(rate / ipw * bits / 8 / 1e9 / HBM_PEAK_GBS, 4)}
 
 
+def moe_plan_bytes(H: int, E: int, k: int, I: int, bits: int, shared_I: int = 0):
+    """Bytes of one MoE layer by the reference's placement model (crates/berth-plan/src/place.rs:345-376),
+    through the planner this build ships: the layer's tensors are listed under the names a checkpoint
+    gives them, `is_routed_expert` splits them into backbone (router, shared expert) and expert pool, and
+    `bytes_moved` = backbone + pool * k / E is what one decoded token reads.  Returns (backbone, pool,
+    bytes_moved).  A configuration without a shared expert lists none of its tensors; the plan record
+    still needs a non-zero width for it."""
+    from berth_amd import plan as P
+
+    def linear_bytes(kk, nn):                      # trellis + fp16 suh + svh
+        return kk * nn * bits // 8 + 2 * (kk + nn)
+
+    mlp = "model.language_model.layers.0.mlp"
+    tensors = [(f"{mlp}.gate.weight", 2 * H * E)]
+    for e in range(E):
+        tensors += [(f"{mlp}.experts.{e}.gate_proj", linear_bytes(H, I)), (f"{mlp}.experts.{e}.up_proj", linear_bytes(H, I)),
+                    (f"{mlp}.experts.{e}.down_proj", linear_bytes(I, H))]
+    if shared_I:
+        tensors += [(f"{mlp}.shared_expert.gate_proj", linear_bytes(H, shared_I)),
+                    (f"{mlp}.shared_expert.up_proj", linear_bytes(H, shared_I)),
+                    (f"{mlp}.shared_expert.down_proj", linear_bytes(shared_I, H))]
+    shape = P.ModelShape(P.ARCH_QWEN3_5_MOE, 1, [P.LayerKind.FULL_ATTENTION], H, 256, 16, 2, P.GdnDims(16, 32, 128, 128, 4),
+                         P.MoeDims(E, k, I, shared_I or I), 248_320)
+    listed = P.TensorBytes(tensors)
+    placed = P.place(P.build_plan(shape), listed)
+    pool = sum(b for n, b in listed.tensors if P.is_routed_expert(n))
+    return listed.total() - pool, pool, placed.bytes_moved.vram
+
+
 def moe_bench(gpu, steps: int, warmup: int):
     """BASELINE.json configs[3]: hidden 2048, 128 experts, top-8 softmax routing,
     expert intermediate 768, 4 bpw, router fp16 N(0, 0.02); batch 1 and 64.  One
@@ -176,7 +205,7 @@ def moe_bench(gpu, steps: int, warmup: int):
                                  for j, (n, shape) in enumerate((("gate_proj", (H, I)), ("up_proj", (H, I)),
                                                                  ("down_proj", (I, H))))))
         layers.append(MoeLayer(gpu, synth.router_weight(77 + li, H, E), experts, k))
-    expert_bytes = 3 * H * I * bits // 8 + 2 * (2 * (H + I) + (I + H))
+    backbone, pool, moved = moe_plan_bytes(H, E, k, I, bits)
     res = {}
     for T in (1, 64):
         xs = [gpu.upload(synth.activations(300 + i, T, H).view(np.uint16)) for i in range(16)]
@@ -220,11 +249,15 @@ def moe_bench(gpu, steps: int, warmup: int):
         graph_us = (time.perf_counter() - t0) / (replays * 16) * 1e6
         if graph_us < eager_us:
             dt, launch = graph_us * 1e-6 * steps, "hip graph of 16 layers"
-        nbytes = 2 * H * E + hit * expert_bytes + 2 * T * H + 4 * T * H
+        # one token: the placement model's bytes_moved; a batch reads each expert it hits once
+        weights = moved if T == 1 else backbone + pool * hit / E
+        nbytes = weights + 2 * T * H + 4 * T * H
         res[f"T{T}"] = {"us_per_layer": round(dt / steps * 1e6, 2), "us_per_token": round(dt / steps / T * 1e6, 3),
                         "experts_hit": round(hit, 1), "algorithmic_GBps": round(nbytes * steps / dt / 1e9, 1),
                         "launch": launch, "eager_us_per_layer": round(eager_us, 2)}
     res["config"] = "hidden 2048, 128 experts, top-8, intermediate 768, 4 bpw, mul1"
+    res["bytes_model"] = {"backbone": backbone, "expert_pool": pool, "bytes_moved_per_token": moved,
+                          "source": "berth_amd.plan.place (place.rs:345-376)"}
     return res
 
 
@@ -306,8 +339,8 @@ def moe_large_bench(gpu, steps: int, resident_layers: int = 48):
     graph_dt = (time.perf_counter() - t0) / (replays * n)
     if graph_dt < dt:
         dt, launch = graph_dt, f"hip graph of {n} layers"
-    expert_bytes = 3 * H * I * bits // 8 + 2 * (2 * (H + I) + (I + H))
-    nbytes = 2 * H * E + (hit + 1) * expert_bytes + 2 * T * H + 4 * T * H
+    backbone, pool, moved = moe_plan_bytes(H, E, k, I, bits, shared_I=I)
+    nbytes = backbone + pool * hit / E + 2 * T * H + 4 * T * H
     flops = 2.0 * (T * k + T) * 3 * H * I
     return {"config": "hidden 2048, 512 experts top-10 + shared expert, intermediate 512, 3 bpw, 256 tokens, "
                       "Zipf(1.1) router bias, mul1",
@@ -315,6 +348,8 @@ def moe_large_bench(gpu, steps: int, resident_layers: int = 48):
             "us_per_layer": round(dt * 1e6, 1), "us_per_token": round(dt / T * 1e6, 3),
             "launch": launch, "eager_us_per_layer": round(eager_us, 1),
             "experts_hit": round(hit, 1), "hottest_expert_rows": hottest,
+            "bytes_model": {"backbone": backbone, "expert_pool": pool, "bytes_moved_per_token": moved,
+                            "source": "berth_amd.plan.place (place.rs:345-376)"},
             "algorithmic_GBps": round(nbytes / dt / 1e9, 1), "tflops": round(flops / dt / 1e12, 2)}
 
 

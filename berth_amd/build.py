@@ -77,10 +77,11 @@ def build_code_object() -> str:
 
 
 def build_reader() -> str:
-    """The EXL3 checkpoint reader (csrc/host/exl3_reader_capi.cpp): host-only C++."""
+    """The EXL3 checkpoint reader and the model planner (csrc/host/exl3_reader_capi.cpp,
+    plan_capi.cpp): host-only C++ in one library."""
     out = os.path.join(LIB, "libberth_exl3_reader.so")
     cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-shared", "-fPIC", "-Wall",
-           os.path.join(CSRC, "host", "exl3_reader_capi.cpp"), "-o", out]
+           os.path.join(CSRC, "host", "exl3_reader_capi.cpp"), os.path.join(CSRC, "host", "plan_capi.cpp"), "-o", out]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"checkpoint reader build failed:\n{r.stderr[-4000:]}")

@@ -731,6 +731,24 @@ static int smoke_linear(int k, int n, int bits, int out_fp32)
 extern "C" int berth_exl3_smoke_int8(int out_fp32) { return smoke_linear(128, 256, 4, out_fp32 ? 1 : 0); }
 extern "C" int berth_exl3_smoke_gemm(void) { return smoke_linear(128, 512, 6, 0); }
 
+extern "C" int berth_ops_add_bias(void* c, const float* bias, int rows, int n, int c_fp32, void* stream)
+{
+    try {
+        g_ops_err.clear();
+        g_ops_launch.clear();
+        if (!c || !bias) throw std::runtime_error("add_bias: null device pointer");
+        if (rows < 1 || n < 1) throw std::runtime_error("add_bias: rows and n must be positive");
+        if (c_fp32 != 0 && c_fp32 != 1) throw std::runtime_error("add_bias: c_fp32 must be 0 or 1");
+        g_ops_launch = launch_add_bias(c, bias, rows, n, c_fp32, (hipStream_t)stream);
+        return 0;
+    } catch (const std::exception& err) {
+        g_ops_err = err.what();
+        g_ops_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
 extern "C" int berth_ops_add_f32(const void* a, const void* b, void* c, int n, void* stream)
 {
     try {

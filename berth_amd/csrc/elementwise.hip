@@ -128,6 +128,35 @@ std::string launch_add_f32(const void* a, const void* b, void* c, int n, hipStre
     return "add_f32 block=256 grid=" + std::to_string(blocks);
 }
 
+// c[r][j] += bias[j] for a linear that carries a bias (crates/berth-exl3/src/linear.rs:131-133; the
+// reference's engine refuses such a linear, crates/berth-engine/src/mlp.rs:67-75).  c is the linear's
+// output as written, fp16 or fp32; the sum is formed in fp32 and rounded once to c's type.
+template <bool F32>
+__global__ __launch_bounds__(256) void add_bias_kernel(void* c, const float* __restrict__ bias, int n, long long total)
+{
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const float b = bias[(int)(i % n)];
+    if (F32) {
+        ((float*)c)[i] += b;
+    } else {
+        _Float16* h = (_Float16*)c;
+        h[i] = (_Float16)((float)h[i] + b);
+    }
+}
+
+std::string launch_add_bias(void* c, const void* bias, int rows, int n, int c_fp32, hipStream_t stream)
+{
+    const long long total = (long long)rows * n;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    if (c_fp32)
+        hipLaunchKernelGGL(add_bias_kernel<true>, dim3(blocks), dim3(256), 0, stream, c, (const float*)bias, n, total);
+    else
+        hipLaunchKernelGGL(add_bias_kernel<false>, dim3(blocks), dim3(256), 0, stream, c, (const float*)bias, n, total);
+    hip_ok(hipGetLastError(), "add_bias launch");
+    return std::string("add_bias ") + (c_fp32 ? "f32" : "f16") + " block=256 grid=" + std::to_string(blocks);
+}
+
 // RMS norm of fp32 rows to fp16, optionally with the fused residual
 // (crates/berth-kernels/src/ops.rs:398-500, csrc/ops/norm.cu): residual += x in
 // place (fp32), then y = fp16((v * rmf) * (w + constant_bias) * constant_scale),

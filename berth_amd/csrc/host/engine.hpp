@@ -6,16 +6,19 @@
 // (device.rs:176-212), MlpLayer (crates/berth-engine/src/mlp.rs:25-334), and a
 // MoeLayer for the Ffn::Moe{router, shared, experts} of
 // crates/berth-plan/src/plan.rs:24-59 with every tensor resident in HBM.
-// Exl3Linear::load, MlpLayer::load and upload_tensor read an EXL3 checkpoint
-// directory through exl3_checkpoint.hpp (device.rs:49-125, mlp.rs:52-112).
+// Exl3Linear::load, MlpLayer::load, MoeLayer::load and upload_tensor read an EXL3
+// checkpoint directory through exl3_checkpoint.hpp (device.rs:49-125, mlp.rs:52-112);
+// MoeLayer::load is sized by the plan's Ffn::Moe record (plan.hpp).
 // Header-only; no torch, no HIP headers: everything goes through the C ABIs.
 #pragma once
 
 #include "../../../include/berth_hip.h"
 #include "../../../include/berth_kernels_hip.h"
 #include "exl3_checkpoint.hpp"
+#include "plan.hpp"
 
 #include <cstdint>
+#include <cstring>
 #include <stdexcept>
 #include <string>
 #include <utility>
@@ -142,6 +145,72 @@ private:
 
 using Half = uint16_t;      // fp16 bit patterns on the host
 
+// fp32 -> fp16 bits, round to nearest even, overflow to infinity, NaN kept quiet
+inline Half f32_to_f16_bits(float f)
+{
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    x &= 0x7FFFFFFFu;
+    if (x >= 0x7F800000u) return (Half)(sign | 0x7C00u | (x > 0x7F800000u ? 0x200u : 0));
+    if (x >= 0x477FF000u) return (Half)(sign | 0x7C00u);                 // rounds to 65520 or above
+    if (x < 0x33000001u) return (Half)sign;                              // at most half of the smallest subnormal
+    if (x < 0x38800000u) {                                               // subnormal result
+        const int shift = 126 - (int)(x >> 23);                          // 14..24
+        const uint32_t man = (x & 0x7FFFFFu) | 0x800000u;
+        const uint32_t q = man >> shift, rem = man & ((1u << shift) - 1), half = 1u << (shift - 1);
+        return (Half)(sign | (q + (rem > half || (rem == half && (q & 1)))));
+    }
+    const uint32_t q = ((x - 0x38000000u) >> 13), rem = x & 0x1FFFu;
+    return (Half)(sign | (q + (rem > 0x1000u || (rem == 0x1000u && (q & 1)))));
+}
+inline float f16_bits_to_f32(Half h)
+{
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, exp = (h >> 10) & 0x1F, man = h & 0x3FFu;
+    uint32_t x;
+    if (exp == 0x1F) {
+        x = sign | 0x7F800000u | (man << 13);
+    } else if (exp) {
+        x = sign | ((exp + 112) << 23) | (man << 13);
+    } else if (man) {
+        int e = 113;
+        uint32_t m = man;
+        while (!(m & 0x400u)) { m <<= 1; --e; }
+        x = sign | ((uint32_t)e << 23) | ((m & 0x3FFu) << 13);
+    } else {
+        x = sign;
+    }
+    float f;
+    std::memcpy(&f, &x, 4);
+    return f;
+}
+
+// an F16 / BF16 / F32 checkpoint tensor as fp32 values (the dtypes a bias may have: linear.rs:219-231)
+inline std::vector<float> read_float_tensor(const exl3::TensorInfo& info)
+{
+    const std::vector<uint8_t> body = exl3::read_tensor(info);
+    std::vector<float> out;
+    if (info.dtype == exl3::DType::F32) {
+        out.resize(body.size() / 4);
+        std::memcpy(out.data(), body.data(), out.size() * 4);
+    } else if (info.dtype == exl3::DType::F16 || info.dtype == exl3::DType::Bf16) {
+        out.resize(body.size() / 2);
+        for (size_t i = 0; i < out.size(); ++i) {
+            uint16_t v;
+            std::memcpy(&v, body.data() + 2 * i, 2);
+            if (info.dtype == exl3::DType::F16) {
+                out[i] = f16_bits_to_f32(v);
+            } else {
+                const uint32_t x = (uint32_t)v << 16;
+                std::memcpy(&out[i], &x, 4);
+            }
+        }
+    } else {
+        throw WeightsError(info.name + ": expected a float tensor, got " + exl3::dtype_name(info.dtype));
+    }
+    return out;
+}
+
 // the checkpoint's EXL3 linear with this prefix (device.rs:167-173)
 inline const exl3::LinearExl3& find_linear(const exl3::Checkpoint& ckpt, const std::string& prefix)
 {
@@ -189,9 +258,11 @@ public:
         a_had_ = DeviceBuffer<Half>::zeroed(gpu, (size_t)size_k);
     }
 
-    // <prefix>.trellis, .suh / .svh (or packed .su / .sv, expanded on the device) from a
-    // checkpoint (device.rs:92-125).  Half-integer rates are refused as in the reference;
-    // packed signs, which the reference refuses at this point, are accepted.
+    // <prefix>.trellis, .suh / .svh (or packed .su / .sv, expanded on the device) and an
+    // optional .bias from a checkpoint (device.rs:92-125).  Half-integer rates are refused as
+    // in the reference; packed signs, which the reference refuses at this point, are accepted;
+    // a bias, which the reference's engine refuses (mlp.rs:67-75), is kept in fp32 and added
+    // to every output row after the linear (y = W x + b).
     static Exl3Linear load(const Gpu& gpu, const exl3::Checkpoint& ckpt, const std::string& prefix)
     {
         const exl3::LinearExl3& linear = find_linear(ckpt, prefix);
@@ -213,8 +284,19 @@ public:
         const std::vector<uint8_t> body = exl3::read_tensor(linear.trellis);
         out.trellis_ = DeviceBuffer<uint16_t>::from_host(gpu, (const uint16_t*)body.data(), body.size() / 2);
         out.a_had_ = DeviceBuffer<Half>::zeroed(gpu, (size_t)out.size_k_);
+        if (linear.bias) out.set_bias(gpu, read_float_tensor(*linear.bias));
         return out;
     }
+
+    // fp32 bias of size_n values, added to every output row after the linear
+    void set_bias(const Gpu& gpu, const std::vector<float>& bias)
+    {
+        if ((int)bias.size() != size_n_)
+            throw WeightsError(prefix_ + ": bias has " + std::to_string(bias.size()) + " values for " +
+                               std::to_string(size_n_) + " outputs");
+        bias_ = DeviceBuffer<float>::from_host(gpu, bias);
+    }
+    bool has_bias() const { return bias_.len() != 0; }
 
     const std::string& prefix() const { return prefix_; }
     int size_k() const { return size_k_; }
@@ -232,6 +314,7 @@ public:
         if (berth_exl3_linear(a.raw(), trellis_.raw(), (void*)(uintptr_t)c, suh_.raw(), a_had_.raw(), svh_.raw(), 1,
                               size_k_, size_n_, k_bits_, (int)codebook_, (int)out, gpu.raw_stream()) != 0)
             throw KernelError(berth_exl3_last_error());
+        add_bias(gpu, c, 1, out);
     }
 
     // rows > 1 with the chunk's scratch (device.rs:210-272)
@@ -249,6 +332,7 @@ public:
                                       svh_.raw(), weight, rows, size_k_, size_n_, k_bits_, (int)codebook_, (int)out,
                                       gpu.raw_stream()) != 0)
             throw KernelError(berth_prefill_last_error());
+        add_bias(gpu, c, rows, out);
     }
 
     // 1..144 rows with a caller-owned rotated-input buffer (device.rs:288-366)
@@ -265,10 +349,18 @@ public:
                                       nullptr, rows, size_k_, size_n_, k_bits_, (int)codebook_, (int)out,
                                       gpu.raw_stream()) != 0)
             throw KernelError(berth_prefill_last_error());
+        add_bias(gpu, c, rows, out);
     }
 
 private:
     Exl3Linear() = default;
+    void add_bias(const Gpu& gpu, uint64_t c, int rows, OutDtype out) const
+    {
+        if (!has_bias()) return;
+        if (berth_ops_add_bias((void*)(uintptr_t)c, (const float*)bias_.raw(), rows, size_n_, out == OutDtype::F32 ? 1 : 0,
+                               gpu.raw_stream()) != 0)
+            throw KernelError(berth_ops_last_error());
+    }
     // fp16 vector as stored, or packed sign words expanded to fp16 +-1 on the device
     static DeviceBuffer<Half> load_scale(const Gpu& gpu, const exl3::HadamardScale& scale, int* channels)
     {
@@ -290,6 +382,7 @@ private:
     Codebook codebook_ = Codebook::Mul1;
     DeviceBuffer<uint16_t> trellis_;
     DeviceBuffer<Half> suh_, svh_, a_had_;
+    DeviceBuffer<float> bias_;
 };
 
 // gate -> up -> silu_mul -> down (mlp.rs:118-150 decode, :219-303 prefill)
@@ -310,20 +403,20 @@ public:
         // the one-call path takes one bit rate and codebook for the three linears
         uniform_ = gate_.k_bits() == up_.k_bits() && gate_.k_bits() == down_.k_bits() &&
                    gate_.codebook() == up_.codebook() && gate_.codebook() == down_.codebook();
+        has_bias_ = gate_.has_bias() || up_.has_bias() || down_.has_bias();
     }
     // layer `layer`'s MLP weights (mlp.rs:52-56)
     static MlpLayer load(const Gpu& gpu, const exl3::Checkpoint& ckpt, uint32_t layer, int max_rows = 1)
     {
         return load_prefixed(gpu, ckpt, "model.language_model.layers." + std::to_string(layer) + ".mlp", max_rows);
     }
-    // {prefix}.gate_proj, .up_proj and .down_proj (mlp.rs:58-112); a bias is refused because
-    // it would not be applied
+    // {prefix}.gate_proj, .up_proj and .down_proj (mlp.rs:58-112).  The reference refuses a bias
+    // here (mlp.rs:67-75); this loader keeps it, forward / prefill add it after each linear, and
+    // forward_fused, which has no place for it, refuses the layer.
     static MlpLayer load_prefixed(const Gpu& gpu, const exl3::Checkpoint& ckpt, const std::string& prefix,
                                   int max_rows = 1)
     {
         const std::string parts[3] = {prefix + ".gate_proj", prefix + ".up_proj", prefix + ".down_proj"};
-        for (const std::string& part : parts)
-            if (find_linear(ckpt, part).bias) throw WeightsError(part + ": bias is present and is not applied");
         Exl3Linear gate = Exl3Linear::load(gpu, ckpt, parts[0]);
         Exl3Linear up = Exl3Linear::load(gpu, ckpt, parts[1]);
         Exl3Linear down = Exl3Linear::load(gpu, ckpt, parts[2]);
@@ -339,12 +432,14 @@ public:
 
     int hidden() const { return hidden_; }
     int intermediate() const { return intermediate_; }
+    bool has_bias() const { return has_bias_; }
 
     // x fp16 [rows][hidden] -> y fp32 [rows][hidden] through berth_exl3_mlp: gate and up in one
     // launch, silu(g) * u evaluated inside the down projection (two launches up to 8 rows)
     void forward_fused(const Gpu& gpu, const DeviceBuffer<Half>& x, DeviceBuffer<float>& y, int rows = 1) const
     {
         if (!uniform_) throw InputError("mlp: the one-call path needs one bit rate and codebook");
+        if (has_bias_) throw InputError("mlp: the one-call path does not add a bias");
         if (rows < 1 || rows > max_rows_) throw InputError("mlp: rows exceed the layer scratch");
         if (x.len() < (size_t)rows * hidden_ || y.len() < (size_t)rows * hidden_)
             throw InputError(gate_.prefix() + ": buffer too small");
@@ -382,8 +477,68 @@ private:
     }
     Exl3Linear gate_, up_, down_;
     int hidden_ = 0, intermediate_ = 0, max_rows_;
-    bool uniform_ = false;
+    bool uniform_ = false, has_bias_ = false;
     DeviceBuffer<Half> g_, u_, x_had_, act_had_;
+};
+
+// An EXL3 linear that stacks `blocks` equal linears along K: tile rows [b * K/16, (b+1) * K/16)
+// and input scales [b * K, (b+1) * K) belong to block b; the output scale either spans the
+// columns once or once per block.  window() copies one block's rows, restricted to a column
+// range, into an ordinary linear.  This is how a checkpoint's `experts.gate_up_proj` /
+// `experts.down_proj` pair (crates/berth-plan/tests/plan.rs:111-118) is read here; the reference
+// names those tensors but never opens one, so the stacking order is this loader's assumption.
+class StackedLinear {
+public:
+    StackedLinear(const exl3::Checkpoint& ckpt, const std::string& prefix, int blocks) : prefix_(prefix), blocks_(blocks)
+    {
+        const exl3::LinearExl3& linear = find_linear(ckpt, prefix);
+        if (linear.k.is_half()) throw WeightsError(prefix + ": half-integer rate");
+        if (linear.input_scale.packed || linear.output_scale.packed)
+            throw WeightsError(prefix + ": packed signs in a stacked expert tensor");
+        if (linear.bias) throw WeightsError(prefix + ": bias is present and is not applied");
+        bits_ = linear.k.whole();
+        tiles_k_all_ = linear.trellis.shape[0];
+        tiles_n_ = linear.trellis.shape[1];
+        codebook_ = linear.codebook == exl3::Codebook::Mul1  ? Codebook::Mul1
+                    : linear.codebook == exl3::Codebook::Mcg ? Codebook::Mcg
+                                                             : Codebook::Default;
+        if (blocks < 1 || tiles_k_all_ % (uint64_t)blocks)
+            throw WeightsError(prefix + ": " + std::to_string(tiles_k_all_) + " tile rows do not split into " +
+                               std::to_string(blocks) + " experts");
+        trellis_ = exl3::read_tensor(linear.trellis);
+        suh_ = exl3::read_tensor(linear.input_scale.tensor);
+        svh_ = exl3::read_tensor(linear.output_scale.tensor);
+        const uint64_t n = tiles_n_ * 16;
+        if (suh_.size() / 2 != tiles_k_all_ * 16 || (svh_.size() / 2 != n && svh_.size() / 2 != n * (uint64_t)blocks))
+            throw WeightsError(prefix + ": scales do not match the stacked tensor");
+        svh_per_block_ = blocks > 1 && svh_.size() / 2 == n * (uint64_t)blocks;
+    }
+    int size_k() const { return (int)(tiles_k_all_ / (uint64_t)blocks_ * 16); }
+    int size_n() const { return (int)(tiles_n_ * 16); }
+
+    Exl3Linear window(const Gpu& gpu, const std::string& name, int block, int n0, int n) const
+    {
+        const uint64_t tiles_k = tiles_k_all_ / (uint64_t)blocks_, words = 16ull * bits_;
+        if (block < 0 || block >= blocks_ || n0 < 0 || n < 16 || n0 % 16 || n % 16 || (uint64_t)(n0 + n) > tiles_n_ * 16)
+            throw WeightsError(prefix_ + ": window " + name + " lies outside the stacked tensor");
+        std::vector<uint16_t> tr((size_t)(tiles_k * (n / 16) * words));
+        const uint16_t* src = (const uint16_t*)trellis_.data();
+        for (uint64_t r = 0; r < tiles_k; ++r)
+            std::memcpy(tr.data() + r * (n / 16) * words,
+                        src + (((uint64_t)block * tiles_k + r) * tiles_n_ + (uint64_t)n0 / 16) * words,
+                        (size_t)(n / 16) * words * 2);
+        const Half* su = (const Half*)suh_.data() + (size_t)block * tiles_k * 16;
+        const Half* sv = (const Half*)svh_.data() + (svh_per_block_ ? (size_t)block * tiles_n_ * 16 : 0) + n0;
+        return Exl3Linear(gpu, name, tr.data(), tr.size(), su, (int)(tiles_k * 16), sv, n, codebook_);
+    }
+
+private:
+    std::string prefix_;
+    int blocks_, bits_ = 0;
+    uint64_t tiles_k_all_ = 0, tiles_n_ = 0;
+    bool svh_per_block_ = false;
+    Codebook codebook_ = Codebook::Mul1;
+    std::vector<uint8_t> trellis_, suh_, svh_;
 };
 
 // router + E routed experts of three linears + optional always-on shared expert
@@ -413,8 +568,88 @@ public:
         router_ = DeviceBuffer<Half>::from_host(gpu, router, (size_t)hidden * num_experts);
         if (bias) bias_ = DeviceBuffer<float>::from_host(gpu, bias, (size_t)num_experts);
     }
+    // Layer `layer`'s MoE block from a checkpoint, sized by the plan's Ffn::Moe record
+    // (crates/berth-plan/src/plan.rs:45-57; tensor names as in crates/berth-plan/tests/plan.rs:96-120
+    // and tests/from_exl3_bytes.rs):
+    //   {mlp}.gate.weight                      router, [experts][hidden] in F16 / BF16 / F32 as a linear
+    //                                          layer stores it; transposed here to [hidden][experts] fp16
+    //   {mlp}.experts.<e>.{gate,up,down}_proj  one EXL3 linear per routed expert and projection, or
+    //   {mlp}.experts.{gate_up,down}_proj      the stacked pair (StackedLinear; gate columns, then up)
+    //   {mlp}.shared_expert.{gate,up,down}_proj the always-on expert
+    // with {mlp} = model.language_model.layers.<layer>.mlp.  Refused: a plan layer that is not MoE,
+    // sizes that differ from the plan's, a quantized router, a bias on an expert linear (the grouped
+    // launches have no place for it) and {mlp}.shared_expert_gate.weight (a per-token scale of the
+    // shared expert that no launch here applies).
+    static MoeLayer load(const Gpu& gpu, const exl3::Checkpoint& ckpt, uint32_t layer, const plan::Ffn& ffn,
+                         bool renorm = true)
+    {
+        if (!ffn.is_moe) throw InputError("moe: layer " + std::to_string(layer) + " is planned with a dense MLP");
+        const std::string mlp = "model.language_model.layers." + std::to_string(layer) + ".mlp";
+        const int E = (int)ffn.router.num_experts, I = (int)ffn.experts.intermediate_size;
+
+        if (ckpt.find_linear(mlp + ".gate")) throw WeightsError(mlp + ".gate: a quantized router is not handled");
+        const exl3::TensorInfo* gate = ckpt.tensors.get(mlp + ".gate.weight");
+        if (!gate) throw WeightsError("tensor " + mlp + ".gate.weight is missing");
+        if (gate->shape.size() != 2 || gate->shape[0] != (uint64_t)E)
+            throw WeightsError(gate->name + ": expected [" + std::to_string(E) + "][hidden]");
+        const int H = (int)gate->shape[1];
+        const std::vector<float> w = read_float_tensor(*gate);
+        std::vector<Half> router((size_t)H * E);
+        for (int e = 0; e < E; ++e)
+            for (int h = 0; h < H; ++h) router[(size_t)h * E + e] = f32_to_f16_bits(w[(size_t)e * H + h]);
+        if (ckpt.tensors.get(mlp + ".shared_expert_gate.weight"))
+            throw WeightsError(mlp + ".shared_expert_gate.weight is present and is not applied");
+
+        auto checked = [&](Exl3Linear lin, int k, int n) {
+            if (lin.size_k() != k || lin.size_n() != n)
+                throw WeightsError(lin.prefix() + ": " + std::to_string(lin.size_k()) + "x" + std::to_string(lin.size_n()) +
+                                   " where the plan has " + std::to_string(k) + "x" + std::to_string(n));
+            if (lin.has_bias()) throw WeightsError(lin.prefix() + ": bias is present and is not applied");
+            return lin;
+        };
+        std::vector<Expert> experts;
+        experts.reserve((size_t)E);
+        const std::string pool = mlp + ".experts";
+        if (ckpt.find_linear(pool + ".gate_up_proj")) {
+            const StackedLinear gate_up(ckpt, pool + ".gate_up_proj", E), down(ckpt, pool + ".down_proj", E);
+            if (gate_up.size_k() != H || gate_up.size_n() != 2 * I || down.size_k() != I || down.size_n() != H)
+                throw WeightsError(pool + ": stacked tensors are " + std::to_string(gate_up.size_k()) + "x" +
+                                   std::to_string(gate_up.size_n()) + " and " + std::to_string(down.size_k()) + "x" +
+                                   std::to_string(down.size_n()) + " per expert where the plan has " + std::to_string(H) +
+                                   "x" + std::to_string(2 * I) + " and " + std::to_string(I) + "x" + std::to_string(H));
+            for (int e = 0; e < E; ++e) {
+                const std::string p = pool + "." + std::to_string(e);
+                experts.push_back(Expert{gate_up.window(gpu, p + ".gate_proj", e, 0, I),
+                                         gate_up.window(gpu, p + ".up_proj", e, I, I),
+                                         down.window(gpu, p + ".down_proj", e, 0, H)});
+            }
+        } else {
+            for (int e = 0; e < E; ++e) {
+                const std::string p = pool + "." + std::to_string(e);
+                experts.push_back(Expert{checked(Exl3Linear::load(gpu, ckpt, p + ".gate_proj"), H, I),
+                                         checked(Exl3Linear::load(gpu, ckpt, p + ".up_proj"), H, I),
+                                         checked(Exl3Linear::load(gpu, ckpt, p + ".down_proj"), I, H)});
+            }
+        }
+        MoeLayer out(gpu, router.data(), H, E, std::move(experts), (int)ffn.router.experts_per_tok, nullptr, renorm);
+        const int SI = (int)ffn.shared.intermediate_size;
+        const std::string sh = mlp + ".shared_expert";
+        out.set_shared(Expert{checked(Exl3Linear::load(gpu, ckpt, sh + ".gate_proj"), H, SI),
+                              checked(Exl3Linear::load(gpu, ckpt, sh + ".up_proj"), H, SI),
+                              checked(Exl3Linear::load(gpu, ckpt, sh + ".down_proj"), SI, H)});
+        return out;
+    }
+    int hidden() const { return hidden_; }
+    int num_experts() const { return num_experts_; }
+    int top_k() const { return top_k_; }
+    int intermediate() const { return intermediate_; }
+    int shared_intermediate() const { return shared_.empty() ? 0 : shared_[0].gate.size_n(); }
+
     void set_shared(Expert shared)
     {
+        if (shared.gate.k_bits() != k_bits_ || shared.up.k_bits() != k_bits_ || shared.down.k_bits() != k_bits_ ||
+            shared.gate.codebook() != codebook_)
+            throw InputError("moe: the shared expert must use the routed experts' bit rate and codebook");
         shared_.clear();
         shared_.push_back(std::move(shared));
     }

@@ -3,32 +3,12 @@
 // status and leaves the message in a thread-local string.
 #include "../../../include/berth_exl3_reader.h"
 #include "exl3_checkpoint.hpp"
+#include "reader_handles.hpp"
 
 #include <algorithm>
 #include <new>
 
 using namespace berth::exl3;
-
-struct berth_ckpt_config {
-    ModelConfig cfg;
-    std::vector<int> kinds;
-    std::vector<const char*> names;
-    void index()
-    {
-        kinds.clear();
-        names.clear();
-        for (const LayerType& t : cfg.layer_types) {
-            kinds.push_back((int)t.kind);
-            names.push_back(t.name.c_str());
-        }
-    }
-};
-
-struct berth_ckpt {
-    Checkpoint ckpt;
-    berth_ckpt_config config;
-    std::vector<const TensorInfo*> tensors;   // name order
-};
 
 namespace {
 

@@ -6,6 +6,10 @@
 //   host_check ckpt-info <checkpoint dir>                    (no device) lists the linears the reader found
 //   host_check ckpt-linear <checkpoint dir> <prefix> <dir>   Exl3Linear::load, one row of <dir>/x.bin, fp32 out
 //   host_check ckpt-mlp <checkpoint dir> <layer> <dir>       MlpLayer::load, one row of <dir>/x.bin
+//   host_check ckpt-plan <checkpoint dir>                    (no device) config -> shape -> plan -> placement
+//   host_check f16 <dir>                                     (no device) x.f32 -> fp16 bits y.u16 and back y.f32
+//   host_check ckpt-moe <checkpoint dir> <layer> <dir>       MoeLayer::load from the plan's Ffn::Moe record,
+//                                                            meta.txt: tokens; x.bin [tokens][hidden]
 // Tensors are raw little-endian files in <dir>; outputs go to <dir>/y.bin (+ idx.bin).
 #include "engine.hpp"
 
@@ -188,19 +192,77 @@ static int run_ckpt_mlp(const Gpu& gpu, const std::string& ckpt_dir, uint32_t la
     return 0;
 }
 
+static int run_ckpt_plan(const std::string& ckpt_dir)
+{
+    namespace plan = berth::plan;
+    const berth::exl3::Checkpoint ckpt = berth::exl3::Checkpoint::open(ckpt_dir);
+    const plan::ModelPlan model = plan::build_plan(plan::model_shape(ckpt.config));
+    const plan::TensorBytes bytes = plan::tensor_bytes(ckpt);
+    const plan::Placement placed = plan::place(model, bytes, plan::MachineBudget::mi355x());
+    size_t moe_layers = 0, expert_tensors = 0;
+    for (const plan::LayerPlan& l : model.layers) moe_layers += l.ffn.is_moe ? 1 : 0;
+    for (const plan::PlacedTensor& t : placed.tensors) expert_tensors += plan::is_routed_expert(t.name) ? 1 : 0;
+    std::printf("plan arch=%s layers=%zu moe_layers=%zu tensors=%zu expert_tensors=%zu resident_vram=%llu "
+                "bytes_moved_vram=%llu\n",
+                model.arch_string.c_str(), model.layers.size(), moe_layers, placed.tensors.size(), expert_tensors,
+                (unsigned long long)placed.resident.vram, (unsigned long long)placed.bytes_moved.vram);
+    if (moe_layers) {
+        const plan::Ffn& f = model.layers[0].ffn;
+        std::printf("ffn router=%u/%u shared=%u experts=%u/%u/%u\n", f.router.num_experts, f.router.experts_per_tok,
+                    f.shared.intermediate_size, f.experts.num_experts, f.experts.experts_per_tok,
+                    f.experts.intermediate_size);
+    }
+    return 0;
+}
+
+static int run_ckpt_moe(const Gpu& gpu, const std::string& ckpt_dir, uint32_t layer, const std::string& dir)
+{
+    namespace plan = berth::plan;
+    const berth::exl3::Checkpoint ckpt = berth::exl3::Checkpoint::open(ckpt_dir);
+    const plan::ModelPlan model = plan::build_plan(plan::model_shape(ckpt.config));
+    if (layer >= model.layers.size()) throw InputError("layer " + std::to_string(layer) + " is not in the plan");
+    MoeLayer moe = MoeLayer::load(gpu, ckpt, layer, model.layers[layer].ffn);
+    const int T = (int)read_meta(dir).at(0);
+    const auto x = DeviceBuffer<Half>::from_host(gpu, read_file<Half>(dir + "/x.bin"));
+    auto y = DeviceBuffer<float>::zeroed(gpu, (size_t)T * moe.hidden());
+    auto idx = DeviceBuffer<int32_t>::zeroed(gpu, (size_t)T * moe.top_k());
+    moe.forward(gpu, x, y, T, &idx);
+    gpu.synchronize();
+    write_file(dir + "/y.bin", y.copy_to_host());
+    write_file(dir + "/idx.bin", idx.copy_to_host());
+    std::printf("ckpt-moe ok layer=%u tokens=%d hidden=%d experts=%d top_k=%d intermediate=%d shared=%d launch=%s\n", layer, T,
+                moe.hidden(), moe.num_experts(), moe.top_k(), moe.intermediate(), moe.shared_intermediate(),
+                berth_moe_last_launch());
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
     if (argc < 3) {
-        std::fprintf(stderr, "usage: host_check linear|mlp|moe <dir> | ckpt-info <ckpt> | ckpt-linear <ckpt> <prefix> <dir> "
-                             "| ckpt-mlp <ckpt> <layer> <dir>\n");
+        std::fprintf(stderr, "usage: host_check linear|mlp|moe <dir> | ckpt-info <ckpt> | ckpt-plan <ckpt> | ckpt-linear <ckpt> "
+                             "<prefix> <dir> | ckpt-mlp <ckpt> <layer> <dir> | ckpt-moe <ckpt> <layer> <dir>\n");
         return 2;
     }
     try {
         const std::string what = argv[1], dir = argv[2];
         if (what == "ckpt-info") return run_ckpt_info(dir);
+        if (what == "ckpt-plan") return run_ckpt_plan(dir);
+        if (what == "f16") {
+            const auto x = read_file<float>(dir + "/x.f32");
+            std::vector<Half> h(x.size());
+            std::vector<float> back(x.size());
+            for (size_t i = 0; i < x.size(); ++i) {
+                h[i] = f32_to_f16_bits(x[i]);
+                back[i] = f16_bits_to_f32(h[i]);
+            }
+            write_file(dir + "/y.u16", h);
+            write_file(dir + "/y.f32", back);
+            return 0;
+        }
         Gpu gpu(0);
         if (what == "ckpt-linear" && argc >= 5) return run_ckpt_linear(gpu, dir, argv[3], argv[4]);
         if (what == "ckpt-mlp" && argc >= 5) return run_ckpt_mlp(gpu, dir, (uint32_t)std::stoul(argv[3]), argv[4]);
+        if (what == "ckpt-moe" && argc >= 5) return run_ckpt_moe(gpu, dir, (uint32_t)std::stoul(argv[3]), argv[4]);
         if (what == "linear") return run_linear(gpu, dir);
         if (what == "mlp") return run_mlp(gpu, dir);
         if (what == "moe") return run_moe(gpu, dir);

@@ -152,6 +152,7 @@ std::string launch_reconstruct_had(void* unpacked, const void* packed, const voi
 std::string launch_had_r_128(const void* in, void* out, const void* scale, int pre_scale,
                              int rows, int cols, int fp32, hipStream_t stream);
 std::string launch_add_f32(const void* a, const void* b, void* c, int n, hipStream_t stream);
+std::string launch_add_bias(void* c, const void* bias, int rows, int n, int c_fp32, hipStream_t stream);
 std::string launch_rms_norm(const void* x, const void* weight, void* y, void* residual, int rows, int dim,
                             float epsilon, float constant_bias, float constant_scale, int weight_bf16,
                             hipStream_t stream);

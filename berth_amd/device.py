@@ -31,6 +31,19 @@ def find_linear(ckpt, prefix: str):
     raise WeightsError(f"{prefix} is not an EXL3 linear")
 
 
+def read_float_tensor(info) -> np.ndarray:
+    """An F16 / BF16 / F32 checkpoint tensor as fp32 values (the dtypes a bias may have:
+    crates/berth-exl3/src/linear.rs:219-231)."""
+    name = info.dtype.as_str()
+    if name == "F32":
+        return info.read_array(np.float32).ravel().copy()
+    if name == "F16":
+        return info.read_array(np.float16).ravel().astype(np.float32)
+    if name == "BF16":
+        return (info.read_array(np.uint16).ravel().astype(np.uint32) << 16).view(np.float32)
+    raise WeightsError(f"{info.name}: expected a float tensor, got {name}")
+
+
 class Gpu:
     """Device 0 and the stream every launch goes on (device.rs:14-43)."""
 
@@ -97,6 +110,7 @@ class Exl3Linear:
         self.suh = gpu.upload(suh.view(np.uint16))
         self.svh = gpu.upload(svh.view(np.uint16))
         self.a_had = torch.zeros(self.size_k, dtype=torch.float16, device=gpu.device)
+        self.bias = None
 
     @classmethod
     def from_device(cls, prefix: str, trellis: torch.Tensor, suh: torch.Tensor, svh: torch.Tensor, k_bits: int,
@@ -113,7 +127,20 @@ class Exl3Linear:
             raise InputError(f"{prefix}: trellis shape does not match suh / svh")
         self.trellis, self.suh, self.svh = trellis, suh, svh
         self.a_had = a_had if a_had is not None else torch.zeros(self.size_k, dtype=torch.float16, device=trellis.device)
+        self.bias = None
         return self
+
+    def set_bias(self, gpu: Gpu, bias: np.ndarray) -> None:
+        """A bias of `size_n` values, kept in fp32 and added to every output row after the
+        linear.  The reference classifies the tensor (crates/berth-exl3/src/linear.rs:131-133)
+        and its engine refuses it (mlp.rs:67-75): what is added here follows y = W x + b."""
+        if bias.size != self.size_n:
+            raise WeightsError(f"{self.prefix}: bias has {bias.size} values for {self.size_n} outputs")
+        self.bias = gpu.upload(np.ascontiguousarray(bias, dtype=np.float32).ravel())
+
+    def _add_bias(self, gpu: Gpu, c: torch.Tensor, rows: int, out: OutDtype) -> None:
+        if self.bias is not None:
+            K.ops.add_bias(ptr(c), ptr(self.bias), rows, self.size_n, out == OutDtype.F32, gpu.raw_stream())
 
     @classmethod
     def from_packed_signs(cls, gpu: Gpu, prefix: str, trellis: np.ndarray, su: np.ndarray, sv: np.ndarray,
@@ -135,9 +162,9 @@ class Exl3Linear:
     @classmethod
     def load(cls, gpu: Gpu, ckpt, prefix: str) -> "Exl3Linear":
         """`<prefix>.trellis`, `.suh` / `.svh` (or packed `.su` / `.sv`, expanded on the
-        device) from a `berth_amd.exl3.Checkpoint` (device.rs:92-125).  Half-integer
-        rates are refused as in the reference; packed signs, which the reference
-        refuses at this point, are accepted."""
+        device) and an optional `.bias` from a `berth_amd.exl3.Checkpoint`
+        (device.rs:92-125).  Half-integer rates are refused as in the reference; packed
+        signs, which the reference refuses at this point, are accepted."""
         linear = find_linear(ckpt, prefix)
         if linear.k.is_half():
             raise WeightsError(f"{prefix}: half-integer rate")
@@ -157,8 +184,11 @@ class Exl3Linear:
             raise WeightsError(f"{prefix}: trellis {tiles_k}x{tiles_n} tiles do not match "
                                f"{halves[0].numel()} x {halves[1].numel()} scales")
         trellis = gpu.upload(linear.trellis.read_array(np.uint16).ravel())
-        return cls.from_device(prefix, trellis, halves[0], halves[1], linear.k.twice // 2,
+        self = cls.from_device(prefix, trellis, halves[0], halves[1], linear.k.twice // 2,
                                Codebook(linear.kernel_codebook))
+        if linear.bias is not None:
+            self.set_bias(gpu, read_float_tensor(linear.bias))
+        return self
 
     def trellis_bytes(self) -> int:
         return self.trellis.numel() * 2
@@ -170,6 +200,7 @@ class Exl3Linear:
             raise InputError(f"{self.prefix}: buffer too small")
         K.exl3_linear(ptr(a), ptr(self.trellis), ptr(c), ptr(self.suh), ptr(self.a_had), ptr(self.svh),
                       1, self.size_k, self.size_n, self.k_bits, self.codebook, out, gpu.raw_stream())
+        self._add_bias(gpu, c, 1, out)
 
     # device.rs:210-272
     def forward_rows(self, gpu: Gpu, scratch: RowScratch, a: torch.Tensor, c: torch.Tensor, rows: int,
@@ -185,6 +216,7 @@ class Exl3Linear:
         K.prefill_lin.exl3_linear(ptr(a), ptr(self.trellis), ptr(c), ptr(self.suh), ptr(scratch.a_had),
                                   ptr(self.svh), weight, rows, self.size_k, self.size_n, self.k_bits,
                                   self.codebook, out, gpu.raw_stream())
+        self._add_bias(gpu, c, rows, out)
 
     # device.rs:288-366
     def forward_n(self, gpu: Gpu, a_had: torch.Tensor, a: torch.Tensor, c: torch.Tensor, rows: int,
@@ -204,6 +236,7 @@ class Exl3Linear:
             K.prefill_lin.exl3_linear(ptr(a), ptr(self.trellis), ptr(c), ptr(self.suh), ptr(a_had),
                                       ptr(self.svh), None, rows, self.size_k, self.size_n, self.k_bits,
                                       self.codebook, out, gpu.raw_stream())
+        self._add_bias(gpu, c, rows, out)
 
 
 class Exl3MultiLinear:
@@ -279,6 +312,7 @@ class MlpLayer:
         self.x_had = self.act_had = None      # rotated inputs of the fused call, allocated on first use
         # the one-call path takes one bit rate and codebook for the three linears
         self.uniform = gate.k_bits == up.k_bits == down.k_bits and gate.codebook == up.codebook == down.codebook
+        self.has_bias = any(l.bias is not None for l in (gate, up, down))
 
     @classmethod
     def load(cls, gpu: Gpu, ckpt, layer: int, max_rows: int = 1) -> "MlpLayer":
@@ -287,12 +321,10 @@ class MlpLayer:
 
     @classmethod
     def load_prefixed(cls, gpu: Gpu, ckpt, prefix: str, max_rows: int = 1) -> "MlpLayer":
-        """`{prefix}.gate_proj`, `.up_proj`, `.down_proj` (mlp.rs:58-112); a bias is refused
-        because it would not be applied."""
+        """`{prefix}.gate_proj`, `.up_proj`, `.down_proj` (mlp.rs:58-112).  The reference refuses
+        a bias here (mlp.rs:67-75); this loader keeps it, and `forward` then takes the four-call
+        path, where each linear adds its own."""
         parts = [f"{prefix}.gate_proj", f"{prefix}.up_proj", f"{prefix}.down_proj"]
-        for part in parts:
-            if find_linear(ckpt, part).bias is not None:
-                raise WeightsError(f"{part}: bias is present and is not applied")
         gate, up, down = (Exl3Linear.load(gpu, ckpt, part) for part in parts)
         if (gate.size_k, gate.size_n) != (up.size_k, up.size_n):
             raise WeightsError(f"{prefix}: gate is {gate.size_k}x{gate.size_n}, up is {up.size_k}x{up.size_n}")
@@ -305,7 +337,7 @@ class MlpLayer:
     def forward(self, gpu: Gpu, x: torch.Tensor, y: torch.Tensor, fused: bool = True, rows: int = 1) -> None:
         """x fp16 [rows][hidden] -> y fp32 [rows][hidden].  fused: one `berth_exl3_mlp` call (two
         launches up to 8 rows); otherwise the reference's four calls for one row (mlp.rs:118-150)."""
-        if fused and self.uniform:
+        if fused and self.uniform and not self.has_bias:
             if rows * self.intermediate > self.g.numel() or x.numel() < rows * self.hidden or \
                y.numel() < rows * self.hidden:
                 raise InputError(f"{self.gate.prefix}: buffer too small")

@@ -55,6 +55,7 @@ def load() -> C.CDLL:
         L.berth_ops_rms_norm.argtypes = [vp, vp, vp, ci, ci, C.c_float, C.c_float, C.c_float, ci, vp]
         L.berth_ops_rms_norm_res_in.argtypes = [vp, vp, vp, vp, ci, ci, C.c_float, C.c_float, C.c_float, ci, vp]
         L.berth_ops_add_f32.argtypes = [vp, vp, vp, ci, vp]
+        L.berth_ops_add_bias.argtypes = [vp, vp, ci, ci, ci, vp]
         L.berth_ops_rms_norm_f16.argtypes = [vp, vp, vp, ci, ci, C.c_float, C.c_float, C.c_float, vp]
         L.berth_ops_embed_tokens.argtypes = [vp, vp, vp, ci, ci, vp]
         L.berth_ops_embed_tokens_f16.argtypes = [vp, vp, vp, ci, ci, vp]
@@ -275,6 +276,13 @@ class ops:
         rc = load().berth_ops_add_f32(a, b, c, n, stream)
         if rc != 0:
             raise LaunchError(ops.last_error() or f"add_f32 launch failed ({rc})")
+
+    @staticmethod
+    def add_bias(c, bias, rows: int, n: int, c_fp32: bool, stream=None) -> None:
+        """c[rows][n] += bias[n] (fp32 bias) on a linear's output as written."""
+        rc = load().berth_ops_add_bias(c, bias, rows, n, int(c_fp32), stream)
+        if rc != 0:
+            raise LaunchError(ops.last_error() or f"add_bias launch failed ({rc})")
 
     @staticmethod
     def silu_mul(gate, up, out, numel: int, act_limit: float = 0.0, stream=None) -> None:

@@ -154,6 +154,11 @@ int berth_ops_rms_norm_res_in(const void* x, const void* weight, void* y, void* 
 /* replaces crates/berth-kernels/src/ops.rs:91-97,522-552 / csrc/ops/add.cu: c = a + b, fp32,
  * n elements; c may alias a. */
 int berth_ops_add_f32(const void* a, const void* b, void* c, int n, void* stream);
+/* No counterpart in the reference, whose engine refuses a linear that carries a bias
+ * (crates/berth-engine/src/mlp.rs:67-75, attn.rs:867-869; the tensor itself is classified at
+ * crates/berth-exl3/src/linear.rs:131-133,219-231).  c[rows][n] += bias[n]: c is a linear's output
+ * as written (fp16, or fp32 when c_fp32), bias fp32; the sum is formed in fp32 and rounded once. */
+int berth_ops_add_bias(void* c, const float* bias, int rows, int n, int c_fp32, void* stream);
 /* replaces crates/berth-kernels/src/ops.rs:108-118,600-640 / csrc/ops/norm.cu:80-112,163-190: the
  * same norm for fp16 rows with a bf16 weight, fp16 out, no residual. */
 int berth_ops_rms_norm_f16(const void* x, const void* weight, void* y, int rows, int dim, float epsilon,

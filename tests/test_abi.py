@@ -46,6 +46,20 @@ def test_reader_library_exports_every_declared_symbol():
         assert getattr(lib, name) is not None, name
 
 
+def test_reader_library_exports_every_declared_planner_symbol():
+    lib = C.CDLL(os.path.join(ROOT, "berth_amd", "lib", "libberth_exl3_reader.so"))
+    names = [n for n in _declared("berth_plan.h") if n.startswith("berth_plan_")]
+    assert "berth_plan_build" in names and "berth_plan_place" in names and len(names) >= 17
+    for name in names:
+        assert getattr(lib, name) is not None, name
+    # null arguments are refused with a message, not dereferenced
+    lib.berth_plan_last_error.restype = C.c_char_p
+    assert lib.berth_plan_build(None, None) == -1 and b"null argument" in lib.berth_plan_last_error()
+    assert lib.berth_plan_last_error_kind() == 90
+    assert lib.berth_plan_place(None, None, None, C.c_size_t(0), None, None, None, None) == -1
+    assert lib.berth_plan_is_routed_expert(None) == 0
+
+
 def test_linear_null_and_bad_sizes_do_not_touch_the_device():
     with pytest.raises(LaunchError, match="null"):
         K.exl3_linear(None, None, None, None, None, None, 1, 128, 256, 4, Codebook.MUL1, OutDtype.F16)
