@@ -563,6 +563,26 @@ thread_local std::string g_moe_err, g_moe_launch;
 
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
+// byte offsets inside the scratch of berth_moe_permute: the sorted rows' experts, the three
+// problem counts, one-row (VALU) problems and 32-row (MFMA) problems
+struct PermuteScratch {
+    size_t row_expert, counts, vprob, mprob, total;
+    int max_m;
+};
+PermuteScratch permute_scratch_layout(int T, int k, int E)
+{
+    const size_t P = (size_t)T * k, small = std::min<size_t>((size_t)E, P);
+    PermuteScratch s{};
+    size_t at = 0;
+    s.row_expert = at; at = align_up(at + P * 4);
+    s.counts = at; at = align_up(at + 16);
+    s.vprob = at; at = align_up(at + small * sizeof(GroupProblem));
+    s.mprob = at;
+    s.max_m = (int)(small + P / kGemmRows + 2);
+    s.total = align_up(at + (size_t)s.max_m * sizeof(GroupProblem));
+    return s;
+}
+
 struct MoeLayout {
     size_t idx, w, parts, offsets, perm, inv, row_expert, counts, vprob, mprob, bprob;
     size_t ah0, ah1, g, u, ahd, slot_out, sg, su, s_ahad, shared_out, total;
@@ -783,16 +803,16 @@ extern "C" int berth_moe_permute(const int32_t* idx, int32_t* offsets, int32_t* 
     // scratch holds the row maps, the counts and the problem lists
     const size_t P = (size_t)T * k;
     unsigned char* sb = (unsigned char*)scratch;
+    const PermuteScratch at = permute_scratch_layout(T, k, E);
     PermuteParams p{};
     p.idx = idx;
     p.offsets = offsets;
     p.perm = perm;
     p.inv = inv;
-    size_t at = 0;
-    p.row_expert = (int32_t*)(sb + at); at = align_up(at + P * 4);
-    p.counts = (int32_t*)(sb + at); at = align_up(at + 16);
-    p.vprob = (GroupProblem*)(sb + at); at = align_up(at + (std::min<size_t>(E, P)) * sizeof(GroupProblem));
-    p.mprob = (GroupProblem*)(sb + at);
+    p.row_expert = (int32_t*)(sb + at.row_expert);
+    p.counts = (int32_t*)(sb + at.counts);
+    p.vprob = (GroupProblem*)(sb + at.vprob);
+    p.mprob = (GroupProblem*)(sb + at.mprob);
     p.bprob = p.mprob;
     p.T = T;
     p.k = k;
@@ -809,13 +829,106 @@ extern "C" int berth_moe_permute(const int32_t* idx, int32_t* offsets, int32_t* 
 extern "C" size_t berth_moe_permute_scratch_bytes(int T, int k, int E)
 {
     if (T < 1 || k < 1 || E < 1) return 0;
-    const size_t P = (size_t)T * k;
-    size_t at = 0;
-    at = align_up(at + P * 4);
-    at = align_up(at + 16);
-    at = align_up(at + std::min<size_t>(E, P) * sizeof(GroupProblem));
-    at = align_up(at + (std::min<size_t>(E, P) + P / kGemmRows + 2) * sizeof(GroupProblem));
-    return at;
+    return permute_scratch_layout(T, k, E).total;
+}
+
+// One stage of the layer on its own: a grouped EXL3 linear (or the gate / up pair) over the
+// expert-sorted rows, driven by the problem lists berth_moe_permute left in its scratch.
+extern "C" int berth_moe_grouped_exl3(const void* a, const void* a_up, const int32_t* gather, int gather_div,
+                                      const void* experts, int lins_per_expert, int lin_base, int num_lins,
+                                      void* c0, void* c1, const void* permute_scratch, void* a_had, int T, int k,
+                                      int E, int size_k, int size_n, int k_bits, int codebook, int c_fp32,
+                                      void* stream_)
+{
+    MOE_TRY_BEGIN
+    hipStream_t stream = (hipStream_t)stream_;
+    if (!a || !experts || !c0 || !permute_scratch) throw std::runtime_error("moe grouped linear: null device pointer");
+    if (T < 1 || k < 1 || E < 1 || size_k < 1 || size_n < 1) throw std::runtime_error("moe: sizes must be positive");
+    if (k > E) throw std::runtime_error("moe: top-k exceeds the number of experts");
+    if (E > kMaxExperts) throw std::runtime_error("moe: at most 1024 experts");
+    if ((long)T * k > 65535) throw std::runtime_error("moe grouped linear: at most 65535 (token, slot) pairs per call");
+    if (num_lins != 1 && num_lins != 2) throw std::runtime_error("moe grouped linear: num_lins must be 1 or 2");
+    if ((num_lins == 2) != (c1 != nullptr)) throw std::runtime_error("moe grouped linear: c1 goes with the second linear");
+    if (num_lins == 2 && a_up) throw std::runtime_error("moe grouped linear: the silu input serves one linear");
+    if (lins_per_expert < 1 || lin_base < 0 || lin_base + num_lins > lins_per_expert)
+        throw std::runtime_error("moe grouped linear: lin_base + num_lins exceeds lins_per_expert");
+    if (gather && gather_div < 1) throw std::runtime_error("moe grouped linear: gather_div must be positive");
+    if (k_bits < 1 || k_bits > 8) throw std::runtime_error("moe grouped linear: K must be in 1..=8");
+    if (codebook < 0 || codebook > 2) throw std::runtime_error("moe grouped linear: codebook must be 0, 1, or 2");
+    if (c_fp32 != 0 && c_fp32 != 1) throw std::runtime_error("moe grouped linear: c_fp32 must be 0 or 1");
+    if (size_k % 128 || size_n % 128) throw std::runtime_error("moe grouped linear: sizes must be multiples of 128");
+    const int P = T * k;
+    const bool use_valu = T == 1 || P <= kValuPairs;        // what berth_moe_permute chose for these sizes
+    if (!use_valu && !a_had) throw std::runtime_error("moe grouped linear: a_had is required above 8 rows");
+    const unsigned char* sb = (const unsigned char*)permute_scratch;
+    const PermuteScratch at = permute_scratch_layout(T, k, E);
+
+    GroupedArgs g{};
+    g.a = a;
+    g.a_up = a_up;
+    g.gather = gather;
+    g.gather_div = gather ? gather_div : 1;
+    g.experts = experts;
+    g.shared = nullptr;
+    g.shared_expert = -1;
+    g.single_row = T == 1 ? 1 : 0;
+    g.lins_per_expert = lins_per_expert;
+    g.lin_base = lin_base;
+    g.num_lins = num_lins;
+    g.c0 = c0;
+    g.c1 = c1;
+    g.size_k = size_k;
+    g.size_n = size_n;
+    g.k_bits = k_bits;
+    g.codebook = codebook;
+    g.out_fp32 = c_fp32;
+    g.stream = stream;
+    if (use_valu) {
+        g.problems = sb + at.vprob;
+        g.num_problems = (const int*)(sb + at.counts);
+        g.max_problems = (int)std::min<size_t>((size_t)E, (size_t)P);
+        g_moe_launch = launch_gemv_grouped(g);
+    } else {
+        HadRowsParams h{};
+        h.a = (const _Float16*)a;
+        h.a_up = (const _Float16*)a_up;
+        h.gather = gather;
+        h.gather_div = g.gather_div;
+        h.row_expert = (const int32_t*)(sb + at.row_expert);
+        h.experts = (const ExpertLin*)experts;
+        h.shared_expert = -1;
+        h.lins_per_expert = lins_per_expert;
+        h.lin_base = lin_base;
+        h.out[0] = (_Float16*)a_had;
+        h.out[1] = (_Float16*)a_had + (size_t)P * size_k;
+        h.P = P;
+        h.K = size_k;
+        hipLaunchKernelGGL(moe_had_rows_kernel, dim3(P, num_lins), dim3(256), 0, stream, h);
+        hip_ok(hipGetLastError(), "moe_had_rows_kernel launch");
+        g.a_had = h.out[0];
+        g.a_had2 = num_lins == 2 ? h.out[1] : nullptr;
+        g.problems = sb + at.mprob;
+        g.num_problems = (const int*)(sb + at.counts) + 1;
+        g.max_problems = at.max_m;
+        g.mb = 1;
+        g_moe_launch = "moe_had_rows_kernel + " + launch_gemm_grouped(g);
+    }
+    MOE_TRY_END
+}
+
+// out[t] = shared_out[t] + sum_j w[t][j] * slot_out[inv[t * k + j]] in slot order
+extern "C" int berth_moe_combine(const void* slot_out, const void* shared_out, const float* w, const int32_t* inv,
+                                 void* out, int T, int H, int k, void* stream)
+{
+    MOE_TRY_BEGIN
+    if (!slot_out || !w || !inv || !out) throw std::runtime_error("moe combine: null device pointer");
+    if (T < 1 || H < 1 || k < 1) throw std::runtime_error("moe: sizes must be positive");
+    const size_t total = (size_t)T * H;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const float*)slot_out, (const float*)shared_out, w, inv, (float*)out, T, H, k);
+    hip_ok(hipGetLastError(), "moe_combine_kernel launch");
+    g_moe_launch = "moe_combine_kernel";
+    MOE_TRY_END
 }
 
 extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias, const void* experts,

@@ -79,6 +79,9 @@ def load() -> C.CDLL:
         L.berth_moe_route.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         L.berth_moe_permute.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, vp]
         L.berth_moe_permute_scratch_bytes.argtypes = [ci, ci, ci]
+        L.berth_moe_grouped_exl3.argtypes = [vp, vp, vp, ci, vp, ci, ci, ci, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci,
+                                             ci, vp]
+        L.berth_moe_combine.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, vp]
         L.berth_moe_permute_scratch_bytes.restype = C.c_size_t
         L.berth_moe_layer.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t,
                                       ci, ci, ci, ci, ci, ci, ci, ci, ci, vp]
@@ -318,6 +321,22 @@ class moe:
         rc = load().berth_moe_permute(idx, offsets, perm, inv, scratch, T, k, E, stream)
         if rc != 0:
             raise LaunchError(moe.last_error() or f"moe permute launch failed ({rc})")
+
+    @staticmethod
+    def grouped_exl3(a, a_up, gather, gather_div, experts_dev, lins_per_expert, lin_base, num_lins, c0, c1,
+                     permute_scratch, a_had, T, k, E, size_k, size_n, k_bits, codebook, c_fp32, stream=None) -> None:
+        """One grouped EXL3 linear (or the gate / up pair) over the rows `permute` sorted by expert."""
+        rc = load().berth_moe_grouped_exl3(a, a_up, gather, gather_div, experts_dev, lins_per_expert, lin_base,
+                                           num_lins, c0, c1, permute_scratch, a_had, T, k, E, size_k, size_n, k_bits,
+                                           int(codebook), int(c_fp32), stream)
+        if rc != 0:
+            raise LaunchError(moe.last_error() or f"moe grouped linear failed ({rc})")
+
+    @staticmethod
+    def combine(slot_out, shared_out, w, inv, out, T, H, k, stream=None) -> None:
+        rc = load().berth_moe_combine(slot_out, shared_out, w, inv, out, T, H, k, stream)
+        if rc != 0:
+            raise LaunchError(moe.last_error() or f"moe combine failed ({rc})")
 
     @staticmethod
     def permute_scratch_bytes(T, k, E) -> int:

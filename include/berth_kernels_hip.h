@@ -244,6 +244,25 @@ int berth_moe_route(const void* x, const void* wr, const float* bias, int32_t* i
 int berth_moe_permute(const int32_t* idx, int32_t* offsets, int32_t* perm, int32_t* inv,
                       void* scratch, int T, int k, int E, void* stream);
 size_t berth_moe_permute_scratch_bytes(int T, int k, int E);
+/* One stage on its own: a grouped EXL3 linear over the expert-sorted rows.  No counterpart in the
+ * reference; the per-expert weight lists play the role of b_list / suh_list / svh_list in its
+ * multi-linear launch (crates/berth-kernels/src/ops.rs:268-280, csrc/ops/mgemm.cu:194-228).
+ * Sorted row r (r < T*k) belongs to the expert berth_moe_permute assigned it; its input is row
+ * gather[r] / gather_div of `a` (gather NULL: row r), or silu(a[r]) * a_up[r] when a_up is given;
+ * its weights are experts[e * lins_per_expert + lin_base (+1)], a DEVICE array of berth_exl3_lin.
+ * num_lins 2 runs two consecutive linears on the same input (gate and up) into c0 and c1.
+ * Outputs are [T*k][size_n] in sorted order, fp16 or fp32 (c_fp32).  permute_scratch: the scratch
+ * berth_moe_permute filled for the same T, k, E (read only).  a_had: fp16 scratch
+ * [num_lins][T*k][size_k], needed above 8 rows (the MFMA path), else may be NULL. */
+int berth_moe_grouped_exl3(const void* a, const void* a_up, const int32_t* gather, int gather_div,
+                           const void* experts, int lins_per_expert, int lin_base, int num_lins, void* c0,
+                           void* c1, const void* permute_scratch, void* a_had, int T, int k, int E, int size_k,
+                           int size_n, int k_bits, int codebook, int c_fp32, void* stream);
+/* The last stage on its own: out[t] = shared_out[t] (or 0) + sum_j w[t][j] * slot_out[inv[t*k + j]],
+ * fp32 fma in slot order.  slot_out fp32 [T*k][H] in sorted order, shared_out fp32 [T][H] or NULL,
+ * w fp32 [T][k], inv int32 [T*k] from berth_moe_permute, out fp32 [T][H]. */
+int berth_moe_combine(const void* slot_out, const void* shared_out, const float* w, const int32_t* inv,
+                      void* out, int T, int H, int k, void* stream);
 /* Whole layer.  experts: DEVICE array of 3*E berth_exl3_lin (gate, up, down of
  * expert 0, then expert 1, ...).  shared: HOST array of 3 berth_exl3_lin holding
  * device pointers, or NULL.  out fp32 [T][H]; idx_out / w_out optional copies of

@@ -350,3 +350,92 @@ def test_moe_one_token_inline_routing_equals_the_routing_kernel():
         assert "moe_route_one_token_kernel" in res["0"][3] and "+route" not in res["0"][3], res["0"][3]
         for a, b in zip(res["1"][:3], res["0"][:3]):
             assert np.array_equal(a, b), (H, E, res["1"][3])
+
+
+@pytest.mark.parametrize("T,H,E,k,I,bits", [
+    (1, 256, 8, 2, 128, 4),          # one row per expert
+    (3, 256, 8, 2, 128, 4),          # six rows: still the dot-product kernel, several rows per problem
+    (64, 512, 16, 4, 256, 4),        # the MFMA path with rotated rows in a caller buffer
+    (33, 256, 4, 2, 128, 3),
+])
+def test_stage_entry_points_compose_to_the_layer(T, H, E, k, I, bits):
+    """route -> permute -> grouped gate/up -> grouped down -> combine, each through its own entry
+    point, against the same stages inside berth_moe_layer (same kernels: bit for bit) and the
+    oracle."""
+    gpu = Gpu(0)
+    wr, experts_np, experts, _, _ = _make_layer(gpu, 4100 + T, H, E, I, bits)
+    layer = MoeLayer(gpu, wr, experts, k)
+    x = (synth.activations(4200 + T, T, H).astype(np.float32) / np.sqrt(H)).astype(np.float16)
+    d_x = dev(x.view(np.uint16))
+    want_out = torch.zeros((T, H), dtype=torch.float32, device=DEV)
+    layer.forward(gpu, d_x, want_out, T)
+    torch.cuda.synchronize()
+    offs = K.moe.workspace_offsets(T, H, E, k, I, 0)
+    ws = layer._ws.cpu().numpy()
+    P = T * k
+
+    def inside(name, dtype, shape):
+        n = int(np.prod(shape)) * np.dtype(dtype).itemsize
+        return ws[offs[name]:offs[name] + n].view(dtype).reshape(shape).copy()
+
+    idx = torch.zeros((T, k), dtype=torch.int32, device=DEV)
+    w = torch.zeros((T, k), dtype=torch.float32, device=DEV)
+    parts = torch.zeros(T * ((H + 63) // 64) * E, dtype=torch.float32, device=DEV)
+    K.moe.route(d_x.data_ptr(), layer.router.data_ptr(), None, idx.data_ptr(), w.data_ptr(), None, parts.data_ptr(),
+                T, H, E, k, True)
+    off = torch.zeros(E + 1, dtype=torch.int32, device=DEV)
+    perm = torch.zeros(P, dtype=torch.int32, device=DEV)
+    inv = torch.zeros(P, dtype=torch.int32, device=DEV)
+    scratch = torch.zeros(K.moe.permute_scratch_bytes(T, k, E), dtype=torch.uint8, device=DEV)
+    K.moe.permute(idx.data_ptr(), off.data_ptr(), perm.data_ptr(), inv.data_ptr(), scratch.data_ptr(), T, k, E)
+    g = torch.zeros((P, I), dtype=torch.float16, device=DEV)
+    u = torch.zeros((P, I), dtype=torch.float16, device=DEV)
+    slot = torch.zeros((P, H), dtype=torch.float32, device=DEV)
+    a_had = torch.zeros(2 * P * max(H, I), dtype=torch.float16, device=DEV)
+    K.moe.grouped_exl3(d_x.data_ptr(), None, perm.data_ptr(), k, layer.table.data_ptr(), 3, 0, 2, g.data_ptr(),
+                       u.data_ptr(), scratch.data_ptr(), a_had.data_ptr(), T, k, E, H, I, bits, 2, False)
+    first = K.moe.last_launch()
+    K.moe.grouped_exl3(g.data_ptr(), u.data_ptr(), None, 1, layer.table.data_ptr(), 3, 2, 1, slot.data_ptr(), None,
+                       scratch.data_ptr(), a_had.data_ptr(), T, k, E, I, H, bits, 2, True)
+    out = torch.zeros((T, H), dtype=torch.float32, device=DEV)
+    K.moe.combine(slot.data_ptr(), None, w.data_ptr(), inv.data_ptr(), out.data_ptr(), T, H, k)
+    torch.cuda.synchronize()
+    assert ("exl3_gemm_kernel" in first) == (P > 8), first
+    assert np.array_equal(idx.cpu().numpy(), inside("idx", np.int32, (T, k)))
+    assert np.array_equal(perm.cpu().numpy(), inside("perm", np.int32, (P,)))
+    assert np.array_equal(inv.cpu().numpy(), inside("inv", np.int32, (P,)))
+    assert np.array_equal(g.cpu().numpy().view(np.uint16), inside("gate_out", np.uint16, (P, I)))
+    assert np.array_equal(u.cpu().numpy().view(np.uint16), inside("up_out", np.uint16, (P, I)))
+    assert np.array_equal(slot.cpu().numpy().view(np.uint32), inside("slot_out", np.uint32, (P, H)))
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), want_out.cpu().numpy().view(np.uint32))
+    want, oi, _ = O.moe_layer(x, wr, experts_np, k, I, bits, 2)
+    assert np.array_equal(idx.cpu().numpy(), oi)
+    assert np.abs(out.cpu().numpy() - want).max() <= 2e-3 * np.abs(want).max()
+
+
+def test_stage_entry_points_validate_before_launching():
+    P0 = 0x1000
+    bad = [
+        (dict(num_lins=3), "num_lins must be 1 or 2"),
+        (dict(num_lins=2, c1=None), "c1 goes with the second linear"),
+        (dict(a_up=P0, num_lins=2), "silu input serves one linear"),
+        (dict(lin_base=2, num_lins=2), "exceeds lins_per_expert"),
+        (dict(size_k=100), "multiples of 128"),
+        (dict(k_bits=9), "1..=8"),
+        (dict(T=64, a_had=None), "a_had is required above 8 rows"),
+        (dict(k=9, E=8), "top-k exceeds"),
+        (dict(gather=P0, gather_div=0), "gather_div must be positive"),
+    ]
+    for change, message in bad:
+        a = dict(a=P0, a_up=None, gather=None, gather_div=1, experts=P0, lins_per_expert=3, lin_base=0, num_lins=2,
+                 c0=P0, c1=P0, scratch=P0, a_had=P0, T=1, k=2, E=8, size_k=256, size_n=128, k_bits=4, codebook=2,
+                 c_fp32=False)
+        a.update(change)
+        with pytest.raises(K.LaunchError, match=message):
+            K.moe.grouped_exl3(a["a"], a["a_up"], a["gather"], a["gather_div"], a["experts"], a["lins_per_expert"],
+                               a["lin_base"], a["num_lins"], a["c0"], a["c1"], a["scratch"], a["a_had"], a["T"], a["k"],
+                               a["E"], a["size_k"], a["size_n"], a["k_bits"], a["codebook"], a["c_fp32"])
+    with pytest.raises(K.LaunchError, match="null device pointer"):
+        K.moe.combine(None, None, P0, P0, P0, 1, 128, 2)
+    with pytest.raises(K.LaunchError, match="sizes must be positive"):
+        K.moe.combine(P0, None, P0, P0, P0, 0, 128, 2)
