@@ -182,9 +182,11 @@ __device__ __forceinline__ void decode_lane(const uint32_t (&own)[BITS], uint32_
 // moves inside the 16-lane row and a select; no LDS traffic.
 __device__ __forceinline__ uint32_t fetch_prev(int lane, uint32_t last_own)
 {
+    // lanes whose source falls outside the row read 0 (bound_ctrl): those are exactly the lanes
+    // that take the other move's result, so neither move needs its destination set up first
     const int v = (int)last_own;
-    const int from_below = __builtin_amdgcn_update_dpp(v, v, 0x111, 0xF, 0xF, false);   // row_shr:1, lane i <- i-1
-    const int from_above = __builtin_amdgcn_update_dpp(v, v, 0x107, 0xF, 0xF, false);   // row_shl:7, lane i <- i+7
+    const int from_below = __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, true);    // row_shr:1, lane i <- i-1
+    const int from_above = __builtin_amdgcn_update_dpp(0, v, 0x107, 0xF, 0xF, true);    // row_shl:7, lane i <- i+7
     return (uint32_t)((lane & 7) ? from_below : from_above);
 }
 

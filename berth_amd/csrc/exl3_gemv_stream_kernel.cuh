@@ -214,6 +214,16 @@ template <int BITS> struct StreamRing {
     static constexpr int depth = BITS <= 4 ? BERTH_STREAM_RING : (BITS <= 6 ? (BERTH_STREAM_RING * 3) / 4 : BERTH_STREAM_RING / 2);
 };
 
+// a pointer every lane of the wave agrees on, moved to scalar registers
+template <typename T>
+__device__ __forceinline__ global_ptr<T> uniform_ptr(global_ptr<T> q)
+{
+    const uint64_t v = (uint64_t)q;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return (global_ptr<T>)(((uint64_t)hi << 32) | lo);
+}
+
 template <int BITS, int CB, bool SILU, int LUTMASK>
 __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams p)
 {
@@ -337,7 +347,10 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
     unsigned cb = div_magic(ufirst, p.mtr);
     unsigned r = ufirst - cb * TR;
     const int lane_dw = lane * BITS;
-    global_ptr<const uint32_t> pbase = as_global(lin.trellis) + (long)cb * (8 * tile_dw) + (long)r * row_dw;
+    // the walk's pointer is the same in every lane: held in scalar registers, so that stepping it
+    // costs no vector instruction and the loads take it as their scalar base
+    global_ptr<const uint32_t> pbase =
+        uniform_ptr(as_global(lin.trellis) + (long)cb * (8 * tile_dw) + (long)r * row_dw);
     unsigned p_r = r;                                       // tile row of the unit pbase points at
     unsigned p_left = uw0 < uw1 ? uw1 - uw0 - 1 : 0u;       // units after it that are still this wave's
     uint32_t own[RING][BITS];
