@@ -367,6 +367,9 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
             z[m] = ((red[0][m][t] + red[1][m][t]) + red[2][m][t]) + red[3][m][t];
     }
 
+    // the output scale is requested before the hand-over, whose waits it would otherwise queue behind
+    const half2_t sv = ((global_ptr<const half2_t>)as_global(lin.svh + nb * 128))[lane];
+
     if (p.S > 1) {
         // ---- cross-workgroup split-K: last arrival reduces in split order.
         // The partial sums travel as agent-scope atomic stores and loads, which go
@@ -424,7 +427,6 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
         for (int m = 0; m < MMAX; ++m) red[0][m][t] = z[m];
     }
     __syncthreads();
-    const half2_t sv = ((global_ptr<const half2_t>)as_global(lin.svh + nb * 128))[lane];
     for (int m = wave; m < rows; m += 4) {
         float v0 = red[0][m][2 * lane];
         float v1 = red[0][m][2 * lane + 1];

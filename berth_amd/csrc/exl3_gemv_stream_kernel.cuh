@@ -491,6 +491,8 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
     for (unsigned cbi = (unsigned)wave; cbi < ncb; cbi += kStreamWaves) {
         const unsigned cbx = cb_first + cbi;
         if (cbx * 128u >= (unsigned)width) continue;             // a narrower slice of a bundle: nothing there
+        // requested before the hand-over below, whose waits it would otherwise queue behind
+        const half2_t sv = ((global_ptr<const half2_t>)as_global(lin.svh + cbx * 128))[lane];
         const unsigned wf = piece_first[cbi], wl = piece_last[cbi];
         float z0 = 0.0f, z1 = 0.0f;
         for (unsigned wv = wf; wv <= wl; ++wv) {
@@ -538,7 +540,6 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
             }
         }
         // output Hadamard, svh, store
-        const half2_t sv = ((global_ptr<const half2_t>)as_global(lin.svh + cbx * 128))[lane];
         had128_wave(z0, z1, lane);
         z0 = (z0 * kRsqrt128) * (float)sv.x;
         z1 = (z1 * kRsqrt128) * (float)sv.y;
