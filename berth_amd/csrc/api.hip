@@ -51,6 +51,7 @@ Workspace& workspace_for_current_device()
         ws.cu_count = cus;
         ws.partial_bytes = kPartialBytes;
         ws.counter_slots = kCounters;
+        ws.counter_words = kCounters;
         ws.device = device;
     }
     return ws;
@@ -207,6 +208,7 @@ Workspace noalloc_scratch_for_current_device(hipStream_t stream)
     ws.cu_count = d.cu_count;
     ws.partial_bytes = kNoAllocPartialBytes;
     ws.counter_slots = kNoAllocCounters;
+    ws.counter_words = kNoAllocCounters;
     ws.strict = true;
     return ws;
 }

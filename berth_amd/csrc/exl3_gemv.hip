@@ -152,6 +152,7 @@ static std::string run_stream(const Workspace& ws, const StreamPlan& pl, StreamP
     p.counters = ws.counters;
     p.TR = p.K / 16;
     p.NB = p.N / 128;
+    p.cstride = counter_stride(ws, (long)pl.problems * p.NB);
     p.Gp = pl.Gp;
     p.q = pl.q;
     p.rem = pl.rem;
@@ -262,6 +263,7 @@ std::string launch_gemv(const LinearArgs& a, const Workspace* scratch)
     p.KB = a.size_k / 128;
     p.out_fp32 = a.out_fp32;
     if (p.NB > ws.counter_slots) throw std::runtime_error("exl3 gemv: size_n exceeds the split-K counter table");
+    p.cstride = counter_stride(ws, p.NB);
     pick_units(ws, p, p.NB, mmax);
     const int grid = p.NB * p.S;
     launch_bits(p, a.k_bits, a.codebook, mmax, dim3(grid), a.stream);
@@ -314,6 +316,7 @@ std::string launch_gemv_pair(const PairArgs& a)
     p.out_fp32 = 0;
     const long units = 2L * p.NB;
     if (units > kCounters) throw std::runtime_error("exl3 gemv: size_n exceeds the split-K counter table");
+    p.cstride = counter_stride(ws, units);
     pick_units(ws, p, units, mmax);
     dim3 grid((unsigned)(p.NB * p.S), 2);
     launch_bits(p, a.k_bits, a.codebook, mmax, grid, a.stream);
@@ -376,6 +379,7 @@ std::string launch_mgemm(const MgemmArgs& m)
     p.out_fp32 = m.c_fp32;
     const long units = (long)m.bszm_out * p.NB;
     if (units > kCounters) throw std::runtime_error("exl3_mgemm: too many (slice, column block) units");
+    p.cstride = counter_stride(ws, units);
     pick_units(ws, p, units, mmax);
     dim3 grid((unsigned)(m.bszm_out * p.NB * p.S));
     launch_bits(p, m.k_bits, m.codebook, mmax, grid, m.stream);
@@ -414,6 +418,7 @@ std::string launch_gemv_grouped(const GroupedArgs& g)
     p.out_fp32 = g.out_fp32;
     const long units = (long)g.max_problems * g.num_lins * p.NB;
     if (units > kCounters) throw std::runtime_error("moe grouped linear: too many (problem, column block) units");
+    p.cstride = counter_stride(ws, units);
     const int mmax = g.single_row ? 1 : 8;
     if (g.route_params) {
         if (!g.single_row || g.a_up || g.gather_div < 1)
@@ -428,17 +433,28 @@ std::string launch_gemv_grouped(const GroupedArgs& g)
         p.comb_inv = g.comb_inv;
         p.comb_shared = g.comb_shared;
         p.comb_out = g.comb_out;
-        p.comb_counters = ws.counters + units;
+        p.cstride = counter_stride(ws, units + p.NB);
+        p.comb_counters = ws.counters + (size_t)units * p.cstride;
         p.comb_k = g.comb_k;
     }
     pick_units(ws, p, units, mmax);
+    if (g.comb_out && g.comb_single) {
+        if (g.max_problems > kCombMaxProblems || g.comb_k > kCombMaxProblems || g.comb_shared_prob >= g.max_problems)
+            throw std::runtime_error("moe grouped linear: the single hand-over serves at most " +
+                                     std::to_string(kCombMaxProblems) + " problems");
+        const size_t part_floats = (size_t)units * p.S * 128;
+        if ((part_floats + (size_t)units * 64) * 4 > ws.partial_bytes)
+            throw std::runtime_error("moe grouped linear: split-K workspace too small for the single hand-over");
+        p.comb_sv = (uint32_t*)(ws.partials + part_floats);
+        p.comb_shared_prob = g.comb_shared_prob;
+    }
     dim3 grid((unsigned)(g.max_problems * p.NB * p.S), (unsigned)g.num_lins);
     launch_bits(p, g.k_bits, g.codebook, mmax, grid, g.stream);
     hip_ok(hipGetLastError(), "exl3_gemv_kernel grouped launch");
     return "exl3_gemv_kernel<" + std::to_string(g.k_bits) + "," + std::to_string(g.codebook) + "," +
            std::to_string(mmax) + "> grouped grid=" +
            std::to_string(grid.x) + "x" + std::to_string(grid.y) + " split_k=" + std::to_string(p.S) + (p.half_units ? "/half" : "") +
-           (g.comb_out ? " +combine" : "") + (g.route_params ? " +route" : "");
+           (g.comb_out ? (p.comb_sv ? " +combine(one hand-over)" : " +combine") : "") + (g.route_params ? " +route" : "");
 }
 
 }  // namespace berth

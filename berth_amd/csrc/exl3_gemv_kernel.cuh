@@ -69,7 +69,8 @@ struct GemvParams {
     void* c[2];                 // output per blockIdx.y, rows in problem order
     _Float16* a_had;            // optional (dense mode only)
     float* partials;            // [problem][lin][NB][S][MMAX][128]
-    unsigned* counters;         // [problem][lin][NB]
+    unsigned* counters;         // [problem][lin][NB], cstride words apart
+    int cstride;
     int K, N, NB, KB, S, out_fp32;
     int half_units;             // 1: a unit of the K walk is half a k-block (one row only)
     // one-token expert combine folded into the down projection (grouped mode, one
@@ -81,14 +82,25 @@ struct GemvParams {
     const int32_t* comb_inv;
     const float* comb_shared;
     float* comb_out;
-    unsigned* comb_counters;    // [NB], zero between launches
+    unsigned* comb_counters;    // [NB], cstride words apart, zero between launches
     int comb_k;
+    // Single hand-over form of the folded combine (comb_sv != nullptr; at most kCombMaxProblems
+    // problems, problem i's row is row i): the split-K parts of *all* problems of a column
+    // block are counted on one counter, and the last workgroup to arrive finishes every
+    // problem of the block (parts in split order, output rotation, output scale) and then
+    // runs the chain, so the rows never wait for a second counter.  comb_sv takes a copy of
+    // each problem's output scale [unit][64 half2] so that the finisher needs no expert
+    // record; comb_shared_prob is the problem whose row starts the chain (-1: comb_shared or 0).
+    uint32_t* comb_sv;
+    int comb_shared_prob;
     // grouped mode, one token, ROUTE instantiation: there is no problem list yet; problem i is
     // the selected expert with sorted position i, which every wave works out itself from the
     // router's segment sums (route.parts); the first workgroup's first wave stores the routing
     // results for the launches that follow.  route.k (+ 1 with an always-on expert) problems.
     RouteParams route;
 };
+
+constexpr int kCombMaxProblems = 16;
 
 // silu(g) * u with every step rounded to fp16: e = exp(-g); s = 1 + e; r = 1 / s;
 // t = g * r; out = t * u (crates/berth-kernels/csrc/ops/act.cu:35-69 and its fixture)
@@ -370,6 +382,116 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
     // the output scale is requested before the hand-over, whose waits it would otherwise queue behind
     const half2_t sv = ((global_ptr<const half2_t>)as_global(lin.svh + nb * 128))[lane];
 
+    if constexpr (SILU && MMAX == 1) {
+        if (p.comb_sv) {
+            // ---- one hand-over for split-K and combine (see GemvParams::comb_sv).  Every value
+            // below is formed by the operations, in the order, of the two-stage path further
+            // down (parts added in split order from 0.0f when S > 1, rotation, 1/sqrt(128), output
+            // scale, fma chain in slot order), so the two paths give the same bits.
+            __shared__ float crow[kCombMaxProblems][128];
+            const int count = min(*p.num_problems, kCombMaxProblems);
+            float* mine = p.partials + ((size_t)unit * p.S + s) * 128;
+            if (t < 128) __hip_atomic_store(mine + t, z[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (s == 0 && wave == 0)
+                __hip_atomic_store(p.comb_sv + (size_t)unit * 64 + lane, as_u32(sv), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            wait_own_stores();
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __syncthreads();
+            if (t == 0) {
+                unsigned old = __hip_atomic_fetch_add(p.comb_counters + (size_t)nb * p.cstride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                s_last = (old + 1 == (unsigned)(count * p.S)) ? 1u : 0u;
+            }
+            __syncthreads();
+            if (!s_last) return;
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+            if (t == 0) __hip_atomic_store(p.comb_counters + (size_t)nb * p.cstride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+            union Pair { unsigned long long u; float f[2]; };
+            const int col0 = nb * 128;
+            // operands of the chain, written by an earlier launch: lane j holds slot j's
+            float wj = 0.0f;
+            int rj = 0;
+            if (lane < p.comb_k) {
+                wj = p.comb_w[lane];
+                rj = p.comb_inv[lane];
+            }
+            float start = 0.0f;
+            if (t < 128 && p.comb_shared_prob < 0 && p.comb_shared) start = p.comb_shared[col0 + t];
+
+            // wave w finishes problems w, w + 4, w + 8, w + 12; all their parts are requested
+            // in batches of sixteen rows, then added in split order
+            const int mine_n = count > wave ? (count - wave + 3) >> 2 : 0;
+            const int total = mine_n * p.S;
+            uint32_t svj[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int j = wave + 4 * q;
+                svj[q] = j < count ? __hip_atomic_load(p.comb_sv + ((size_t)j * p.NB + nb) * 64 + lane, __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT)
+                                   : 0u;
+            }
+            float zz[4][2] = {};
+            int jl = 0, sp = 0;
+            for (int r0 = 0; r0 < total; r0 += 16) {
+                Pair part[16];
+                const int jl0 = jl, sp0 = sp;
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    part[u].u = 0ull;
+                    if (r0 + u < total) {
+                        const float* row = p.partials + ((size_t)((size_t)(wave + 4 * jl) * p.NB + nb) * p.S + sp) * 128;
+                        part[u].u = __hip_atomic_load((const unsigned long long*)(row + 2 * lane), __ATOMIC_RELAXED,
+                                                      __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    if (++sp == p.S) { sp = 0; ++jl; }
+                }
+                jl = jl0;
+                sp = sp0;
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    if (r0 + u < total) {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            if (jl == q) {
+                                zz[q][0] = p.S == 1 ? part[u].f[0] : zz[q][0] + part[u].f[0];
+                                zz[q][1] = p.S == 1 ? part[u].f[1] : zz[q][1] + part[u].f[1];
+                            }
+                    }
+                    if (++sp == p.S) { sp = 0; ++jl; }
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int j = wave + 4 * q;
+                if (j < count) {
+                    float v0 = zz[q][0], v1 = zz[q][1];
+                    had128_wave(v0, v1, lane);
+                    const half2_t sj = as_half2(svj[q]);
+                    v0 = (v0 * kRsqrt128) * (float)sj.x;
+                    v1 = (v1 * kRsqrt128) * (float)sj.y;
+                    crow[j][2 * lane] = v0;
+                    crow[j][2 * lane + 1] = v1;
+                    // the row itself, for callers that read the rows of the projection
+                    float2_t o = {v0, v1};
+                    *(float2_t*)((float*)cout + (size_t)j * n_stride + col0 + 2 * lane) = o;
+                }
+            }
+            __syncthreads();
+            if (t < 128) {
+                float a = p.comb_shared_prob >= 0 && p.comb_shared_prob < count ? crow[p.comb_shared_prob][t] : start;
+                for (int j = 0; j < p.comb_k; ++j) {
+                    const float wv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j));
+                    const int r = __builtin_amdgcn_readlane(rj, j);
+                    const float row = (unsigned)r < (unsigned)count ? crow[r][t] : 0.0f;
+                    a = __builtin_fmaf(wv, row, a);
+                }
+                p.comb_out[col0 + t] = a;
+            }
+            return;
+        }
+    }
+
     if (p.S > 1) {
         // ---- cross-workgroup split-K: last arrival reduces in split order.
         // The partial sums travel as agent-scope atomic stores and loads, which go
@@ -388,7 +510,7 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (t == 0) {
-            unsigned old = __hip_atomic_fetch_add(p.counters + unit, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            unsigned old = __hip_atomic_fetch_add(p.counters + (size_t)unit * p.cstride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             s_last = (old == (unsigned)(p.S - 1)) ? 1u : 0u;
         }
         __syncthreads();
@@ -417,7 +539,7 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
                         if (s0 + j < p.S) z[m] += part[j][m];
             }
         }
-        if (t == 0) __hip_atomic_store(p.counters + unit, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (t == 0) __hip_atomic_store(p.counters + (size_t)unit * p.cstride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // ---- output Hadamard, svh, store
@@ -450,10 +572,10 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
                 asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
                 unsigned old = 0;
                 if (lane == 0)
-                    old = __hip_atomic_fetch_add(p.comb_counters + nb, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    old = __hip_atomic_fetch_add(p.comb_counters + (size_t)nb * p.cstride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 old = (unsigned)__builtin_amdgcn_readfirstlane((int)old);
                 if (old + 1 != (unsigned)*p.num_problems) return;
-                if (lane == 0) __hip_atomic_store(p.comb_counters + nb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (lane == 0) __hip_atomic_store(p.comb_counters + (size_t)nb * p.cstride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                 const int h = nb * 128 + 2 * lane;
                 Pair acc2;

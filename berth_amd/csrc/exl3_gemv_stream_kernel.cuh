@@ -64,7 +64,8 @@ struct StreamParams {
     _Float16* a_had;            // optional; slab per rotation source
     const uint16_t* lut;        // [65536] fp16 bits of every state of this codebook (LUTMASK != 0)
     float* partials;            // [problem][column block][contributor][128]
-    unsigned* counters;         // [problem][column block], zero between launches
+    unsigned* counters;         // [problem][column block], cstride words apart, zero between launches
+    int cstride;
     int mode;                   // 0 by value, 1 uniform lists, 2 sliced lists
     int in_stride;              // elements between the inputs of consecutive problems (0: shared)
     int K, N, NB, TR;           // N: row stride of trellis and output in mode 0 / 1; TR = K / 16
@@ -518,10 +519,10 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
             wait_own_stores();
             unsigned old = 0;
             if (lane == 0)
-                old = __hip_atomic_fetch_add(p.counters + pslot + cbx, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                old = __hip_atomic_fetch_add(p.counters + (size_t)(pslot + cbx) * p.cstride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             old = (unsigned)__builtin_amdgcn_readfirstlane((int)old);
             if (old != count - 1) continue;
-            if (lane == 0) __hip_atomic_store(p.counters + pslot + cbx, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0) __hip_atomic_store(p.counters + (size_t)(pslot + cbx) * p.cstride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             z0 = z1 = 0.0f;
             for (unsigned j0 = 0; j0 < count; j0 += 8) {
                 Pair part[8];

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <cstdlib>
 #include <stdexcept>
 #include <string>
 
@@ -42,11 +43,30 @@ struct Workspace {
     unsigned* fault_dev = nullptr;
     volatile unsigned* fault_host = nullptr;
     size_t partial_bytes = 0;       // capacity of `partials`
-    int counter_slots = 0;          // capacity of `counters`
+    int counter_slots = 0;          // most counters a launch may use
+    size_t counter_words = 0;       // words behind `counters` (counters can be spread over them)
     bool strict = false;            // true: a launch that would not fit is refused instead of split less
 };
 constexpr size_t kPartialBytes = (size_t)256 << 20;
 constexpr int kCounters = 65536;
+// Words between the arrival counters of a one-row launch that needs `units` of them: as far
+// apart as the table allows, up to one counter per 128 bytes.  Neighbouring words send the
+// arrivals of a whole launch (hundreds within a microsecond) through one atomic unit: measured,
+// counters 32 bytes or more apart take 1.8 us off the four launches of a 27B layer set and
+// 2.9 us off the one-token MoE layer, and 32 bytes .. 16 KiB apart all measure the same.
+// Every launch leaves the counters it used at zero, so launches with different strides can
+// follow each other.  (BERTH_COUNTER_STRIDE caps the stride; 1 packs the counters.)
+inline int counter_stride(const Workspace& ws, long units)
+{
+    static const int cap = [] {
+        const char* e = std::getenv("BERTH_COUNTER_STRIDE");
+        const int v = e ? std::atoi(e) : 32;
+        return v < 1 ? 1 : (v > 32 ? 32 : v);
+    }();
+    int stride = 1;
+    while (stride * 2 <= cap && units * stride * 2 <= (long)ws.counter_words) stride *= 2;
+    return stride;
+}
 Workspace& workspace_for_current_device();
 // throws if a kernel of an earlier launch on this device reported a fault (and clears the report)
 void throw_pending_device_fault(const Workspace& ws);
@@ -112,6 +132,11 @@ struct GroupedArgs {
     const float* comb_shared = nullptr;
     float* comb_out = nullptr;
     int comb_k = 0;
+    // comb_single: split-K and combine share one hand-over (at most sixteen problems, problem i
+    // writing row i); comb_shared_prob is then the problem whose row starts the chain, or -1
+    // when comb_shared (a row written by an earlier launch, or null) does
+    int comb_single = 0;
+    int comb_shared_prob = -1;
 };
 std::string launch_gemv_grouped(const GroupedArgs& args);
 std::string launch_gemm_grouped(const GroupedArgs& args);

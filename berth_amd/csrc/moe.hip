@@ -69,13 +69,13 @@ __global__ __launch_bounds__(256) void moe_route_kernel(RouteParams p)
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     if (tid == 0) {
-        unsigned old = __hip_atomic_fetch_add(p.counters + grp, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        unsigned old = __hip_atomic_fetch_add(p.counters + grp * kRouteCounterStride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_last = (old == (unsigned)(p.nseg - 1)) ? 1u : 0u;
     }
     __syncthreads();
     if (!s_last) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    if (tid == 0) __hip_atomic_store(p.counters + grp, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) __hip_atomic_store(p.counters + grp * kRouteCounterStride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
     // ---- last workgroup of the token group: wave tt finishes token t0 + tt
     const int lane = tid & 63, tt = tid >> 6;
@@ -603,13 +603,15 @@ int moe_big_min()
     return v;
 }
 
-// One token: the down projection's last arrival per column block also combines the
-// block (BERTH_MOE_FOLD_COMBINE=0 keeps the separate combine launch).
-bool fold_combine_enabled()
+// One token: the down projection's last arrival per column block also combines the block.
+// BERTH_MOE_FOLD_COMBINE: 0 keeps the separate combine launch, 1 the two-stage form (split-K
+// hand-over per expert, then a second counter per column block); otherwise, with at most
+// sixteen problems, the single hand-over (one counter per column block for both).
+int fold_combine_mode()
 {
-    static const bool v = [] {
+    static const int v = [] {
         const char* e = std::getenv("BERTH_MOE_FOLD_COMBINE");
-        return !e || std::atoi(e) != 0;
+        return e ? std::atoi(e) : 2;
     }();
     return v;
 }
@@ -700,7 +702,6 @@ std::string run_route(const void* x, const void* wr, const float* bias, int32_t*
     p.nseg = (H + kRouteSeg - 1) / kRouteSeg;
     if (sort && T == 1) p.sort = *sort;
     const int groups = (T + kRouteTT - 1) / kRouteTT;
-    if (groups > kCounters) throw std::runtime_error("moe route: too many tokens for the counter table");
     if (T >= kRouteBigT) {
         const int group = route_big_group(E);
         dim3 grid(p.nseg, (T + group - 1) / group);
@@ -717,6 +718,7 @@ std::string run_route(const void* x, const void* wr, const float* bias, int32_t*
         hip_ok(hipGetLastError(), "moe_route_one_token_kernel launch");
         return std::string("moe_route_one_token_kernel grid=1") + (p.sort.perm ? " (with the sort of the one token)" : "");
     }
+    if ((long)groups * kRouteCounterStride > kCounters) throw std::runtime_error("moe route: too many tokens for the counter table");
     dim3 grid(p.nseg, groups);
     hipLaunchKernelGGL(moe_route_kernel, grid, dim3(256), 0, stream, p);
     hip_ok(hipGetLastError(), "moe_route_kernel launch");
@@ -1097,13 +1099,16 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
     g.out_fp32 = 1;
     // one token: the last expert to finish a column block of the down projection
     // also combines that block, so no combine launch follows
-    const bool fold_combine = T == 1 && L.max_v > 0 && L.max_m == 0 && fold_combine_enabled();
+    const bool fold_combine = T == 1 && L.max_v > 0 && L.max_m == 0 && fold_combine_mode() != 0;
     if (fold_combine) {
         g.comb_w = (const float*)w;
         g.comb_inv = (const int32_t*)(wsb + L.inv);
         g.comb_shared = shared_out;
         g.comb_out = (float*)out;
         g.comb_k = k;
+        // with the always-on expert among the problems its row (row k) starts the chain
+        g.comb_single = fold_combine_mode() != 1 && L.max_v <= kCombMaxProblems ? 1 : 0;
+        g.comb_shared_prob = fold ? k : -1;
     }
     if (L.max_v > 0) {
         g.problems = wsb + L.vprob;

@@ -25,6 +25,7 @@ struct GroupProblem {
 
 constexpr int kRouteSeg = 64;       // rows of the router weight per partial sum
 constexpr int kRouteTT = 4;         // tokens per route workgroup
+constexpr int kRouteCounterStride = 32;   // words between the arrival counters of neighbouring token groups
 constexpr int kMaxExperts = 1024;
 constexpr int kMaxTopK = 32;
 

@@ -250,52 +250,68 @@ def test_moe_config4_shape_zipf_shared():
     assert np.abs(out.cpu().numpy() - want).max() <= 2e-3 * np.abs(want).max()
 
 
+_ONE_TOKEN_CASES = {"plain": (2048, 128, 8, 768, 4, 0), "folded": (512, 16, 4, 256, 3, 256),
+                    "dense": (512, 16, 4, 256, 4, 384), "sixteen": (512, 32, 15, 256, 4, 256),
+                    "seventeen": (512, 32, 16, 256, 2, 256)}
+
+
 def _one_token_outputs():
-    """One token through three layers (no shared expert, shared expert of the routed
-    size, shared expert of another size), twice each: output bits and launch text."""
+    """One token through five layers (no shared expert, shared expert of the routed size,
+    shared expert of another size, sixteen and seventeen problems per launch), twice each:
+    output bits, the rows of the down projection and launch text."""
     gpu = Gpu(0)
     res = {}
-    for name, (H, E, k, I, bits, shared_I) in {"plain": (2048, 128, 8, 768, 4, 0), "folded": (512, 16, 4, 256, 3, 256),
-                                               "dense": (512, 16, 4, 256, 4, 384)}.items():
-        wr, _, experts, _, shared = _make_layer(gpu, 8100 + H + shared_I, H, E, I, bits, shared_I)
+    for name, (H, E, k, I, bits, shared_I) in _ONE_TOKEN_CASES.items():
+        wr, _, experts, _, shared = _make_layer(gpu, 8100 + H + shared_I + k, H, E, I, bits, shared_I)
         layer = MoeLayer(gpu, wr, experts, k, shared=shared)
-        outs = []
+        outs, rows = [], []
         for rep in range(2):
             x = (synth.activations(77 + rep, 1, H).astype(np.float32) / np.sqrt(H)).astype(np.float16)
             out = torch.zeros((1, H), dtype=torch.float32, device=DEV)
             layer.forward(gpu, dev(x.view(np.uint16)), out, 1)
             torch.cuda.synchronize()
             outs.append(out.cpu().numpy().view(np.uint32))
+            at = K.moe.workspace_offsets(1, H, E, k, I, shared_I)["slot_out"]
+            rows.append(layer._ws.cpu().numpy()[at:at + k * H * 4].view(np.uint32).copy())
         res[name] = np.stack(outs)
+        res[name + "_rows"] = np.stack(rows)
         res[name + "_launch"] = np.array(K.moe.last_launch())
     return res
 
 
 def test_moe_one_token_combine_inside_down_projection(tmp_path):
-    """With one token the last expert to finish a column block of the down projection
-    combines it; the result has the bits of the separate combine launch
-    (BERTH_MOE_FOLD_COMBINE=0, read once per process, so in a process of its own)."""
+    """With one token the last workgroup to finish a column block of the down projection
+    combines it.  By default split-K and combine share one hand-over (up to sixteen problems
+    per launch); BERTH_MOE_FOLD_COMBINE=1 keeps the two-stage form and =0 the separate combine
+    launch (read once per process, so each in a process of its own).  All three give the same
+    output bits and the same rows of the down projection."""
     import os
     import subprocess
     import sys
 
     here = _one_token_outputs()
-    for name in ("plain", "folded", "dense"):
+    for name in _ONE_TOKEN_CASES:
         launch = str(here[name + "_launch"])
         assert "+combine" in launch and "moe_combine_kernel" not in launch, launch
+        assert ("one hand-over" in launch) == (name != "seventeen"), launch
+        assert here[name].any() and here[name + "_rows"].any()
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    path = str(tmp_path / "separate.npz")
-    code = ("import numpy as np, tests.test_gpu_moe as T\n"
-            f"np.savez({path!r}, **T._one_token_outputs())\nprint('ok')\n")
-    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=600, cwd=root,
-                       env=dict(os.environ, BERTH_MOE_FOLD_COMBINE="0"))
-    assert r.returncode == 0 and "ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
-    there = np.load(path)
-    for name in ("plain", "folded", "dense"):
-        launch = str(there[name + "_launch"])
-        assert "moe_combine_kernel" in launch and "+combine" not in launch, launch
-        assert np.array_equal(here[name], there[name]), name
-        assert here[name].any()
+    for mode in ("0", "1"):
+        path = str(tmp_path / f"mode{mode}.npz")
+        code = ("import numpy as np, tests.test_gpu_moe as T\n"
+                f"np.savez({path!r}, **T._one_token_outputs())\nprint('ok')\n")
+        r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=600, cwd=root,
+                           env=dict(os.environ, BERTH_MOE_FOLD_COMBINE=mode))
+        assert r.returncode == 0 and "ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+        there = np.load(path)
+        for name in _ONE_TOKEN_CASES:
+            launch = str(there[name + "_launch"])
+            if mode == "0":
+                assert "moe_combine_kernel" in launch and "+combine" not in launch, launch
+            else:
+                assert "+combine" in launch and "one hand-over" not in launch, launch
+            assert np.array_equal(here[name], there[name]), (mode, name)
+            assert np.array_equal(here[name + "_rows"], there[name + "_rows"]), (mode, name)
 
 
 def test_moe_layer_with_128_row_problems():
