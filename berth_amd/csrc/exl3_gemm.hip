@@ -44,6 +44,20 @@ static int gemm_split(const Workspace& ws, long tiles, int KB, int mb)
     return (int)S;
 }
 
+// words between the counters of neighbouring tiles (see counter_stride); `tiles` bounds the
+// tile count of every launch the call makes
+static int gemm_counter_stride(long tiles)
+{
+    static const int cap = [] {
+        const char* e = std::getenv("BERTH_COUNTER_STRIDE");
+        const int v = e ? std::atoi(e) : 32;
+        return v < 1 ? 1 : (v > 32 ? 32 : v);
+    }();
+    int stride = 1;
+    while (stride * 2 <= cap && tiles * stride * 2 <= kCounters / 2) stride *= 2;
+    return stride;
+}
+
 std::string launch_gemm(const LinearArgs& a)
 {
     if (a.size_k % 128 != 0) throw std::runtime_error("exl3 linear: size_k must be a multiple of 128");
@@ -66,6 +80,7 @@ std::string launch_gemm(const LinearArgs& a)
     // 128-row tiles decode a weight once per 128 rows, but need enough tiles to spread
     // over the chip; narrow outputs (few column tiles) run as 32-row tiles instead
     const int nblocks = (a.size_n + 255) / 256;
+    p.cstride = gemm_counter_stride((long)nblocks * ((a.size_m + 31) / 32));
     const long tiles128 = (long)nblocks * ((a.size_m + 127) / 128);
     const int mb_plain = (a.size_m <= 32 || tiles128 * 4 < ws.cu_count) ? 1 : 4;
     const int KB = a.size_k / 128;
@@ -160,6 +175,7 @@ std::string launch_gemm_grouped(const GroupedArgs& g)
     p.counters = ws.counters;
     const int nblocks = (g.size_n + 255) / 256;
     const long tiles = (long)g.max_problems * g.num_lins * nblocks;
+    p.cstride = gemm_counter_stride(tiles);
     p.S = gemm_split(ws, tiles, g.size_k / 128, mb);
     if (g.max_problems > 65535) throw std::runtime_error("moe grouped linear: too many problems");
     std::string desc;

@@ -48,7 +48,8 @@ struct GemmParams {
     // split-K
     int S;
     float* partials;            // [unit][S][4 waves][MB][2][16][64]
-    unsigned* counters;         // [unit]
+    unsigned* counters;         // [unit], cstride words apart ("arrived"; "written" kGemmWrittenBase further on)
+    int cstride;
     // balanced dense launches (exl3_gemm_balanced_kernel): the launch's (tile, k-block) units,
     // tile-major, are dealt out evenly to gridDim.x workgroups
     int units;                  // tiles * K/128; 0: not a balanced launch
@@ -292,8 +293,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
         // the wait is short and cannot block) and adds the parts in k order.  If it holds
         // part 0 itself it starts from its registers and never writes them out.
         constexpr size_t kPerWg = (size_t)4 * MB * 2 * 16 * 64;
-        unsigned* arrived = p.counters + kr.counter;
-        unsigned* written = p.counters + kGemmWrittenBase + kr.counter;
+        unsigned* arrived = p.counters + kr.counter * p.cstride;
+        unsigned* written = arrived + kGemmWrittenBase;
         if (threadIdx.x == 0) {
             unsigned old = __hip_atomic_fetch_add(arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             s_last = (old == (unsigned)(kr.parts - 1)) ? 1u : 0u;

@@ -182,8 +182,8 @@ __device__ __forceinline__ void gemm_tile_wide(const GemmParams& p, const int ti
     if (kr.parts > 1) {
         constexpr size_t kPerWave = (size_t)MB * 2 * 16 * 64;
         constexpr size_t kPerWg = 8 * kPerWave;
-        unsigned* arrived = p.counters + kr.counter;
-        unsigned* written = p.counters + kGemmWrittenBase + kr.counter;
+        unsigned* arrived = p.counters + kr.counter * p.cstride;
+        unsigned* written = arrived + kGemmWrittenBase;
         if (threadIdx.x == 0) {
             unsigned old = __hip_atomic_fetch_add(arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             s_last = (old == (unsigned)(kr.parts - 1)) ? 1u : 0u;
