@@ -74,10 +74,20 @@ __device__ __forceinline__ void wait_own_stores() { asm volatile("s_waitcnt vmcn
 template <int LINES>
 __device__ __forceinline__ void touch_kernel_arguments()
 {
-    static_assert(LINES == 3 || LINES == 6, "instantiated line counts");
+    static_assert(LINES == 3 || LINES == 6 || LINES == 10, "instantiated line counts");
     const auto ka = __builtin_amdgcn_kernarg_segment_ptr();
     int t0, t1, t2, t3, t4, t5;
-    if constexpr (LINES == 6)
+    if constexpr (LINES == 10) {
+        int t6, t7, t8, t9;
+        asm volatile("s_load_dword %0, %10, 0x0\n\ts_load_dword %1, %10, 0x40\n\ts_load_dword %2, %10, 0x80\n\t"
+                     "s_load_dword %3, %10, 0xc0\n\ts_load_dword %4, %10, 0x100\n\ts_load_dword %5, %10, 0x140\n\t"
+                     "s_load_dword %6, %10, 0x180\n\ts_load_dword %7, %10, 0x1c0\n\ts_load_dword %8, %10, 0x200\n\t"
+                     "s_load_dword %9, %10, 0x240\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7),
+                       "=&s"(t8), "=&s"(t9)
+                     : "s"(ka));
+    } else if constexpr (LINES == 6)
         asm volatile("s_load_dword %0, %6, 0x0\n\ts_load_dword %1, %6, 0x40\n\ts_load_dword %2, %6, 0x80\n\t"
                      "s_load_dword %3, %6, 0xc0\n\ts_load_dword %4, %6, 0x100\n\ts_load_dword %5, %6, 0x140\n\t"
                      "s_waitcnt lgkmcnt(0)"

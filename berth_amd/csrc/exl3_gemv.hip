@@ -424,6 +424,13 @@ std::string launch_gemv_grouped(const GroupedArgs& g)
         if (!g.single_row || g.a_up || g.gather_div < 1)
             throw std::runtime_error("moe grouped linear: the inline routing serves the one-token gate / up launch");
         p.route = *(const RouteParams*)g.route_params;
+        if (g.resolved_out && (g.resolved_lin < 0 || g.resolved_lin >= g.lins_per_expert))
+            throw std::runtime_error("moe grouped linear: resolved linear index out of range");
+        p.resolved_out = (ExpertLin*)g.resolved_out;
+        p.resolved_lin = g.resolved_lin;
+    } else if (g.resolved) {
+        if (!g.single_row) throw std::runtime_error("moe grouped linear: resolved records serve one-row problems");
+        p.resolved = (const ExpertLin*)g.resolved;
     }
     if (g.comb_out) {
         if (!g.single_row || g.num_lins != 1 || !g.out_fp32 || !g.a_up || !g.comb_w || !g.comb_inv || g.comb_k < 1)
@@ -454,7 +461,8 @@ std::string launch_gemv_grouped(const GroupedArgs& g)
     return "exl3_gemv_kernel<" + std::to_string(g.k_bits) + "," + std::to_string(g.codebook) + "," +
            std::to_string(mmax) + "> grouped grid=" +
            std::to_string(grid.x) + "x" + std::to_string(grid.y) + " split_k=" + std::to_string(p.S) + (p.half_units ? "/half" : "") +
-           (g.comb_out ? (p.comb_sv ? " +combine(one hand-over)" : " +combine") : "") + (g.route_params ? " +route" : "");
+           (g.comb_out ? (p.comb_sv ? " +combine(one hand-over)" : " +combine") : "") + (g.route_params ? " +route" : "") +
+           (g.resolved ? " resolved" : "");
 }
 
 }  // namespace berth

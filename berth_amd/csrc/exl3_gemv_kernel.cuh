@@ -20,6 +20,8 @@
 //     fp16 arithmetic as the stand-alone SiLU kernel.
 #pragma once
 
+#include <stddef.h>
+
 #include "exl3_decode.cuh"
 #include "hadamard.cuh"
 #include "moe_route.cuh"
@@ -93,6 +95,14 @@ struct GemvParams {
     // record; comb_shared_prob is the problem whose row starts the chain (-1: comb_shared or 0).
     uint32_t* comb_sv;
     int comb_shared_prob;
+    // Grouped one-row launches.  ROUTE instantiation: where the wave that stores the routing
+    // results also leaves the records of linear `resolved_lin` of the experts in sorted order,
+    // then of the always-on expert (null: nowhere).  Other instantiations: `resolved` non-null
+    // replaces the problem list and the expert table (problem i is row i, linear resolved[i];
+    // the grid holds exactly the problems there are).
+    const ExpertLin* resolved;
+    int resolved_lin;
+    ExpertLin* resolved_out;
     // grouped mode, one token, ROUTE instantiation: there is no problem list yet; problem i is
     // the selected expert with sorted position i, which every wave works out itself from the
     // router's segment sums (route.parts); the first workgroup's first wave stores the routing
@@ -271,8 +281,10 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
     __shared__ float red[4][MMAX][128];
     __shared__ unsigned s_last;
 
-    static_assert(sizeof(GemvParams) > 5 * 64, "the argument block spans at least six lines");
-    touch_kernel_arguments<6>();
+    // every field the other instantiations read sits in the first six lines of the argument block
+    static_assert(offsetof(GemvParams, resolved) + 8 <= 6 * 64 && sizeof(GemvParams) > 9 * 64 &&
+                  sizeof(GemvParams) <= 10 * 64, "the argument block's lines as they are touched here");
+    touch_kernel_arguments<ROUTE ? 10 : 6>();
     const int lane = threadIdx.x & 63;
     // wave-uniform on purpose: everything derived from it (k-block, addresses) stays in SGPRs
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -291,9 +303,56 @@ __global__ __launch_bounds__(256, 4) void exl3_gemv_kernel(GemvParams p)
     };
     if constexpr (ROUTE) {
         static_assert(MMAX == 1 && !SILU, "the inline routing serves the one-token gate / up launch");
-        const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && wave == 0;
-        const int expert = route_finish_one_token(p.route, lane, prob, writer);
+        // One wave works the routing out and the others take its answer: a quarter of the reads
+        // of the segment sums, which every workgroup of the launch wants at the same moment
+        // (measured: 1.2 us off the layer against all four waves doing it side by side).
+        __shared__ int s_expert;
+        if (wave == 0) {
+            // The first workgroup's first wave stores the routing results.  It also leaves, for
+            // the launch that follows, the record of linear `resolved_lin` of the expert at
+            // each sorted position (then of the always-on expert), so that that launch reaches
+            // its weights with one dependent read instead of two.  It asks for the records of
+            // all experts (at most 128: lane l holds experts l and l + 64) ahead of the
+            // routing, so that its stores do not wait for a read that depends on the routing.
+            const bool writer = blockIdx.x == 0 && blockIdx.y == 0;
+            const bool resolve = writer && p.resolved_out;
+            unsigned rec[2][6];
+            if (resolve) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const int e2 = min(lane + 64 * i, p.route.E - 1);
+                    const unsigned* src = (const unsigned*)(p.experts + e2 * p.lins_per_expert + p.resolved_lin);
+#pragma unroll
+                    for (int q = 0; q < 6; ++q) rec[i][q] = src[q];
+                }
+            }
+            const RouteOneToken r = route_one_token(p.route, lane, writer);
+            const int e = route_expert_at(p.route, r, lane, prob);
+            if (lane == 0) s_expert = e;
+            if (resolve) {
+                unsigned got[6];
+#pragma unroll
+                for (int q = 0; q < 6; ++q) {
+                    const unsigned lo = (unsigned)__shfl((int)rec[0][q], r.sel & 63, 64);
+                    const unsigned hi = (unsigned)__shfl((int)rec[1][q], r.sel & 63, 64);
+                    got[q] = r.sel >= 64 ? hi : lo;
+                }
+                if (lane < p.route.k) {
+                    unsigned* dst = (unsigned*)(p.resolved_out + r.rank);
+#pragma unroll
+                    for (int q = 0; q < 6; ++q) dst[q] = got[q];
+                }
+                if (lane == 0 && p.shared_expert >= 0) p.resolved_out[p.route.k] = p.shared[p.resolved_lin];
+            }
+        }
+        __syncthreads();
+        const int expert = __builtin_amdgcn_readfirstlane(s_expert);
         lin = expert_lin(expert);
+        row0 = prob;
+        rows = 1;
+    } else if (p.resolved) {
+        // one-row problems whose linears an earlier launch resolved: problem i is row i
+        lin = p.resolved[prob];
         row0 = prob;
         rows = 1;
     } else if (p.problems) {

@@ -137,6 +137,13 @@ struct GroupedArgs {
     // when comb_shared (a row written by an earlier launch, or null) does
     int comb_single = 0;
     int comb_shared_prob = -1;
+    // with route_params: where the launch's first workgroup leaves {trellis, suh, svh} of linear
+    // `resolved_lin` of the experts in sorted order (then the always-on one), or null.
+    // `resolved` (single_row, no route_params): those records, read instead of the problem
+    // list and the expert table; the launch then holds exactly max_problems problems.
+    void* resolved_out = nullptr;
+    int resolved_lin = 0;
+    const void* resolved = nullptr;
 };
 std::string launch_gemv_grouped(const GroupedArgs& args);
 std::string launch_gemm_grouped(const GroupedArgs& args);

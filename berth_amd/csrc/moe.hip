@@ -585,7 +585,7 @@ PermuteScratch permute_scratch_layout(int T, int k, int E)
 
 struct MoeLayout {
     size_t idx, w, parts, offsets, perm, inv, row_expert, counts, vprob, mprob, bprob;
-    size_t ah0, ah1, g, u, ahd, slot_out, sg, su, s_ahad, shared_out, total;
+    size_t ah0, ah1, g, u, ahd, slot_out, sg, su, s_ahad, shared_out, vlin, total;
     int max_v, max_m, max_b, nseg;
 };
 
@@ -626,6 +626,15 @@ bool inline_route_enabled()
 
 // The always-on expert runs as one more expert of the grouped launches (rows P ..
 // P + T - 1, token order) when it has the routed experts' intermediate size.
+// One token with the inline routing: the gate / up launch leaves the down projection's
+// {trellis, suh, svh} records in sorted order, and the down launch reads those instead of the
+// problem list and the expert table (BERTH_MOE_RESOLVED=0: off).
+bool resolved_records_enabled()
+{
+    const char* e = std::getenv("BERTH_MOE_RESOLVED");
+    return !e || std::atoi(e) != 0;
+}
+
 bool shared_is_folded(int I, int shared_I) { return shared_I > 0 && shared_I == I; }
 
 MoeLayout moe_layout(int T, int H, int E, int k, int I, int shared_I)
@@ -672,6 +681,7 @@ MoeLayout moe_layout(int T, int H, int E, int k, int I, int shared_I)
         L.s_ahad = take((size_t)T * std::max(H, shared_I) * 2);
         L.shared_out = take(shared_I ? (size_t)T * H * 4 : 0);
     }
+    L.vlin = take((size_t)std::max(L.max_v, 1) * sizeof(ExpertLin));
     L.total = at;
     return L;
 }
@@ -971,6 +981,7 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
     RouteParams inline_route{};
     const bool route_inline = T == 1 && E % 2 == 0 && E <= kRouteOneMaxE && L.nseg <= kRouteOneMaxSeg && L.max_v > 0 &&
                               inline_route_enabled();
+    const bool use_resolved = route_inline && resolved_records_enabled();
     if (route_inline) {
         RouteParams& r = inline_route;
         r.x = (const _Float16*)x;
@@ -1017,8 +1028,13 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
         g.num_problems = (const int*)(wsb + L.counts);
         g.max_problems = L.max_v;
         g.route_params = route_inline ? &inline_route : nullptr;
+        if (use_resolved) {
+            g.resolved_out = wsb + L.vlin;
+            g.resolved_lin = 2;
+        }
         desc += " + " + launch_gemv_grouped(g);
         g.route_params = nullptr;
+        g.resolved_out = nullptr;
     }
     if (L.max_m > 0) {
         HadRowsParams h{};
@@ -1114,7 +1130,9 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
         g.problems = wsb + L.vprob;
         g.num_problems = (const int*)(wsb + L.counts);
         g.max_problems = L.max_v;
+        g.resolved = use_resolved ? wsb + L.vlin : nullptr;
         desc += " + " + launch_gemv_grouped(g);
+        g.resolved = nullptr;
     }
     if (L.max_m > 0) {
         HadRowsParams h{};

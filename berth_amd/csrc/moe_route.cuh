@@ -180,11 +180,16 @@ __device__ __forceinline__ void route_sort_one_token(const PermuteParams& q, int
 
 // One token, at most 128 experts: the routing's last part by one wave, from the segment sums
 // parts[seg][e] that moe_route_segments_kernel left in memory: logits (segments added in
-// order, bias), top-k, and the sorted position of every selected expert.  Returns the expert
-// whose sorted position is `want_rank` (the always-on expert E for want_rank == k).  Every
-// wave that calls this gets the same bits; the wave with `writer` set also stores the
-// routing results (logits, idx, w, and what the sort of the one token writes).
-__device__ __forceinline__ int route_finish_one_token(const RouteParams& p, int lane, int want_rank, bool writer)
+// order, bias), top-k, and the sorted position of every selected expert (lane j < k: expert of
+// slot j and its sorted position).  Every wave that calls this gets the same bits; the wave
+// with `writer` set also stores the routing results (logits, idx, w, and what the sort of the
+// one token writes).
+struct RouteOneToken {
+    int sel;
+    int rank;
+};
+
+__device__ __forceinline__ RouteOneToken route_one_token(const RouteParams& p, int lane, bool writer)
 {
     float lg[kRoutePer];
 #pragma unroll
@@ -212,16 +217,23 @@ __device__ __forceinline__ int route_finish_one_token(const RouteParams& p, int 
             lg[i] = v;
         }
     }
-    const int sel = route_topk_n<2>(lg, lane, p, 0, writer);
-    if (writer && p.sort.perm) route_sort_one_token(p.sort, lane, sel);
-    if (want_rank >= p.k) return p.E;
-    int rank = 0;
+    RouteOneToken r;
+    r.sel = route_topk_n<2>(lg, lane, p, 0, writer);
+    if (writer && p.sort.perm) route_sort_one_token(p.sort, lane, r.sel);
+    r.rank = 0;
     for (int j = 0; j < p.k; ++j) {
-        const int other = __builtin_amdgcn_readlane(sel, j);
-        rank += other < sel ? 1 : 0;
+        const int other = __builtin_amdgcn_readlane(r.sel, j);
+        r.rank += other < r.sel ? 1 : 0;
     }
-    const unsigned long long holder = __builtin_amdgcn_ballot_w64(lane < p.k && rank == want_rank);
-    return __builtin_amdgcn_readlane(sel, (int)__builtin_ctzll(holder));
+    return r;
+}
+
+// the expert whose sorted position is `want_rank` (the always-on expert E for want_rank == k)
+__device__ __forceinline__ int route_expert_at(const RouteParams& p, const RouteOneToken& r, int lane, int want_rank)
+{
+    if (want_rank >= p.k) return p.E;
+    const unsigned long long holder = __builtin_amdgcn_ballot_w64(lane < p.k && r.rank == want_rank);
+    return __builtin_amdgcn_readlane(r.sel, (int)__builtin_ctzll(holder));
 }
 
 }  // namespace berth

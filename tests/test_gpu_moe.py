@@ -350,8 +350,8 @@ def test_moe_one_token_inline_routing_equals_the_routing_kernel():
         x = (synth.activations(8801 + H, 1, H).astype(np.float32) / np.sqrt(H)).astype(np.float16)
         d_x = dev(x.view(np.uint16))
         res = {}
-        for mode in ("1", "0"):
-            os.environ["BERTH_MOE_INLINE_ROUTE"] = mode
+        for mode, env in (("1", {}), ("unresolved", {"BERTH_MOE_RESOLVED": "0"}), ("0", {"BERTH_MOE_INLINE_ROUTE": "0"})):
+            os.environ.update(env)
             try:
                 out = torch.zeros((1, H), dtype=torch.float32, device=DEV)
                 idx = torch.full((1, k), -1, dtype=torch.int32, device=DEV)
@@ -361,11 +361,15 @@ def test_moe_one_token_inline_routing_equals_the_routing_kernel():
                 res[mode] = (out.cpu().numpy().view(np.uint32), idx.cpu().numpy(), w.cpu().numpy().view(np.uint32),
                              K.moe.last_launch())
             finally:
-                del os.environ["BERTH_MOE_INLINE_ROUTE"]
-        assert "moe_route_segments_kernel" in res["1"][3] and "+route" in res["1"][3], res["1"][3]
+                for name in env:
+                    del os.environ[name]
+        # the down launch takes its linears from the records the gate / up launch left, unless told not to
+        assert "moe_route_segments_kernel" in res["1"][3] and "+route" in res["1"][3] and "resolved" in res["1"][3], res["1"][3]
+        assert "+route" in res["unresolved"][3] and "resolved" not in res["unresolved"][3], res["unresolved"][3]
         assert "moe_route_one_token_kernel" in res["0"][3] and "+route" not in res["0"][3], res["0"][3]
-        for a, b in zip(res["1"][:3], res["0"][:3]):
-            assert np.array_equal(a, b), (H, E, res["1"][3])
+        for other in ("unresolved", "0"):
+            for a, b in zip(res["1"][:3], res[other][:3]):
+                assert np.array_equal(a, b), (H, E, other, res["1"][3])
 
 
 @pytest.mark.parametrize("T,H,E,k,I,bits", [
