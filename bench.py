@@ -34,7 +34,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per GEMV launch of the default workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs scaled by a 1 GiB copy (profiles/exl3_gemv_4bpw_batch1_27b_linear_set.md)
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {4: int((42325 + 258) * 1024)}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {4: int((42378 + 258) * 1024)}
 # vector instructions per weight of the GEMV launches of the default workload, from a rocprofv3
 # --pmc SQ_INSTS_VALU run of this file (same profile): wave instructions * 64 lanes / weights
 VALU_INSTR_PER_WEIGHT = 4.9
