@@ -2,9 +2,8 @@
 // once per tile and shared through LDS.
 //
 // The 128-row kernel keeps decoded weights in the registers of the wave that decoded
-// them, so a weight is decoded once per 128 rows and each SIMD has one MFMA-issuing
-// wave (a wave issues a 32x32x16 MFMA every 32 cycles at best; the matrix pipe takes
-// one every 16).  Here a workgroup has eight waves:
+// them, so a weight is decoded once per 128 rows.  Here a weight is decoded once per 256
+// rows, by one of the eight waves of a workgroup, and the other waves take it from LDS:
 //
 //   decode   wave w, lane l decodes, per 64 rows of K ("macro-step"), the 32 weights of
 //            one octet lane: tile row w/2 of the four, tile column 8*(w%2) + l/8; its four
