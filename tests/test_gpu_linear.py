@@ -455,6 +455,31 @@ def test_lm_head_shape_6bpw_slices_match_oracle():
         assert close(got[c0:c0 + 256], want.reshape(-1))[0] == 0, c0
 
 
+@pytest.mark.parametrize("rows", [1, 3])
+def test_very_wide_output_uses_closer_counters(rows):
+    """More column blocks than the arrival-counter table holds at one counter per 128 bytes
+    (K 256, N 128 x 5000, 2 bpw): the launch packs its counters closer together.  Windows at both
+    ends and in the middle against the oracle, and the same call again gives the same bits (the
+    counters were left at zero)."""
+    Kk, N, bits = 256, 128 * 5000, 2
+    tr, suh, svh = synth.linear(4242, Kk, N, bits)
+    x = synth.activations(4243, rows, Kk)
+    d_tr, d_suh, d_svh, d_x = dev(tr), dev(suh.view(np.uint16)), dev(svh.view(np.uint16)), dev(x.view(np.uint16))
+    a_had = torch.zeros(rows * Kk, dtype=torch.float16, device=DEV)
+    outs = []
+    for _ in range(2):
+        c = torch.zeros(rows * N, dtype=torch.float16, device=DEV)
+        K.exl3_linear(d_x.data_ptr(), d_tr.data_ptr(), c.data_ptr(), d_suh.data_ptr(), a_had.data_ptr(),
+                      d_svh.data_ptr(), rows, Kk, N, bits, Codebook.MUL1, OutDtype.F16)
+        torch.cuda.synchronize()
+        outs.append(host_f16(c).reshape(rows, N))
+    assert np.array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
+    for c0 in (0, 128 * 2500, N - 256):
+        sub = np.ascontiguousarray(tr[:, c0 // 16:c0 // 16 + 16, :])
+        want, _ = O.linear(x, sub, suh, svh[c0:c0 + 256], Kk, 256, bits, 2, out_fp32=False)
+        assert close(outs[0][:, c0:c0 + 256], want.reshape(rows, 256))[0] == 0, c0
+
+
 @pytest.mark.parametrize("name,kernel", [("gate_proj", "exl3_gemm_wide_kernel<4,2,256x256>"),
                                          ("down_proj", "exl3_gemm_balanced_kernel<4,2,128x256>"),
                                          ("q_proj", "exl3_gemm_balanced_kernel<4,2,128x256>"),
