@@ -7,6 +7,7 @@
 
 #include "../../include/berth_kernels_hip.h"
 
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 #include <initializer_list>
@@ -33,10 +34,11 @@ Workspace& workspace_for_current_device()
         hip_ok(hipMalloc(&partials, kPartialBytes), "split-K workspace");
         hip_ok(hipMalloc(&counters, kCounters * sizeof(unsigned)), "split-K counters");
         hip_ok(hipMemset(counters, 0, kCounters * sizeof(unsigned)), "split-K counter memset");
-        void* tables = nullptr;
-        hip_ok(hipMalloc(&tables, 3 * 65536 * sizeof(uint16_t)), "state tables");
-        build_state_tables((uint16_t*)tables);
-        ws.state_tables = (uint16_t*)tables;
+        void* accum = nullptr;
+        hip_ok(hipMalloc(&accum, (size_t)kAccumSlots * 1024), "column-block accumulators");
+        hip_ok(hipMemset(accum, 0, (size_t)kAccumSlots * 1024), "column-block accumulator memset");
+        ws.accum = (unsigned long long*)accum;
+        ws.accum_slots = kAccumSlots;
         int cus = 0;
         hip_ok(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device), "multiProcessorCount");
         ws.partials = (float*)partials;
@@ -57,24 +59,66 @@ Workspace& workspace_for_current_device()
     return ws;
 }
 
+std::string describe_device_fault(unsigned code)
+{
+    if (code >= 0x40000000u)
+        return "an earlier streaming GEMV launch on this device gave up waiting for the other contributors of column block " +
+               std::to_string(code - 0x40000001u) + " and wrote NaN there";
+    return "an earlier launch on this device gave up waiting for the split-K partial sums of tile " +
+           std::to_string(code - 1u) + " and left it unwritten";
+}
+
 void throw_pending_device_fault(const Workspace& ws)
 {
     if (!ws.fault_host) return;
     const unsigned code = *ws.fault_host;
     if (code == 0u) return;
     *ws.fault_host = 0u;
-    throw std::runtime_error(
-        "an earlier launch on this device gave up waiting for the split-K partial sums of tile " +
-        std::to_string(code - 1u) +
-        " and left it unwritten (the library's workspace serves one launch at a time per device: launches "
-        "that overlap on two streams mix their counters); this call launched nothing");
+    throw std::runtime_error(describe_device_fault(code) +
+                             " (the library's workspace serves one launch at a time per device: launches "
+                             "that overlap on two streams mix their counters); this call launched nothing");
 }
 
-unsigned spin_limit()
+namespace {
+int env_int(const char* name, int fallback)
 {
-    const char* e = std::getenv("BERTH_SPIN_LIMIT");
-    const long v = e ? std::strtol(e, nullptr, 0) : 0;
-    return v > 0 ? (unsigned)v : (1u << 20);
+    const char* e = std::getenv(name);
+    return e && *e ? (int)std::strtol(e, nullptr, 0) : fallback;
+}
+int clamp(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+Knobs read_knobs()
+{
+    Knobs k{};
+    k.gemv_stream = env_int("BERTH_GEMV_STREAM", 1);
+    k.gemv_stream_min_units = std::max(2, env_int("BERTH_GEMV_STREAM_MIN_UNITS", 3));
+    k.gemv_stream_shrink = env_int("BERTH_GEMV_STREAM_SHRINK", 0);
+    k.gemv_stream_wgs = env_int("BERTH_GEMV_STREAM_WGS", 0);
+    k.gemv_stream_lut = env_int("BERTH_GEMV_STREAM_LUT", -1);
+    k.gemv_wg_per_cu = env_int("BERTH_GEMV_WG_PER_CU", 0);
+    k.gemv_half_units = env_int("BERTH_GEMV_HALF_UNITS", 1);
+    k.gemv_max_rows = clamp(env_int("BERTH_GEMV_MAX_ROWS", 8), 1, 8);
+    k.gemm_wg_per_cu = env_int("BERTH_GEMM_WG_PER_CU", 0);
+    k.gemm_balanced = env_int("BERTH_GEMM_BALANCED", 1);
+    k.gemm_rows256 = env_int("BERTH_GEMM_ROWS256", 1);
+    k.counter_stride = clamp(env_int("BERTH_COUNTER_STRIDE", 32), 1, 32);
+    k.moe_big_min = env_int("BERTH_MOE_BIG_MIN", 0);
+    k.moe_fold_combine = env_int("BERTH_MOE_FOLD_COMBINE", 2);
+    k.moe_inline_route = env_int("BERTH_MOE_INLINE_ROUTE", 1);
+    k.moe_resolved = env_int("BERTH_MOE_RESOLVED", 1);
+    const int spins = env_int("BERTH_SPIN_LIMIT", 0);
+    k.spin_limit = spins > 0 ? (unsigned)spins : (1u << 20);
+    return k;
+}
+std::mutex g_knobs_mu;
+Knobs g_knobs = read_knobs();
+}  // namespace
+
+const Knobs& knobs() { return g_knobs; }
+void reload_knobs()
+{
+    std::lock_guard<std::mutex> lock(g_knobs_mu);
+    g_knobs = read_knobs();
 }
 
 namespace {
@@ -103,15 +147,7 @@ void check_shape(const char* who, const LinearArgs& a)
 }
 
 // rows up to this count take the VALU kernel, more rows the MFMA kernel
-int gemv_max_rows()
-{
-    static const int v = [] {
-        const char* e = std::getenv("BERTH_GEMV_MAX_ROWS");
-        const int x = e ? std::atoi(e) : 8;
-        return x < 1 ? 1 : (x > 8 ? 8 : x);
-    }();
-    return v;
-}
+int gemv_max_rows() { return knobs().gemv_max_rows; }
 
 std::string dispatch_linear(const LinearArgs& a)
 {
@@ -148,14 +184,21 @@ extern "C" int berth_exl3_linear(const void* a, const void* trellis, void* c, co
 }
 
 // ---- the entry point that allocates nothing -------------------------------------
-// Split-K scratch of berth_exl3_linear_noalloc: partial sums, then the arrival counters.
-// Every GPU the library runs on holds its own copy until the process ends.  In host code
-// the array's name is only a handle for hipGetSymbolAddress; the device address it
-// returns, kept per device, is what kernels and fills get.
+// Scratch of berth_exl3_linear_noalloc: split-K partial sums, their arrival counters, and the
+// streaming kernel's column-block accumulators.  Every GPU the library runs on holds its own
+// copy until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; the device address it returns, kept per device, is what kernels get.
+// The array has no initialiser, so it is zero when the code object is loaded, and every launch
+// leaves the counters and accumulators it used at zero again: nothing has to clear it, and
+// the entry point launches nothing but its GEMV (a first call inside a stream capture records
+// that one kernel).
 namespace {
 constexpr size_t kNoAllocPartialBytes = (size_t)8 << 20;
 constexpr int kNoAllocCounters = 65536;
-constexpr size_t kNoAllocBytes = kNoAllocPartialBytes + (size_t)kNoAllocCounters * sizeof(unsigned);
+constexpr int kNoAllocAccumSlots = 2048;
+constexpr size_t kNoAllocCounterOff = kNoAllocPartialBytes;
+constexpr size_t kNoAllocAccumOff = kNoAllocCounterOff + (size_t)kNoAllocCounters * sizeof(unsigned);
+constexpr size_t kNoAllocBytes = kNoAllocAccumOff + (size_t)kNoAllocAccumSlots * 1024;
 }  // namespace
 static __device__ __align__(256) unsigned char scratch[kNoAllocBytes];
 
@@ -163,19 +206,12 @@ namespace {
 struct NoAllocDevice {
     unsigned char* ptr = nullptr;   // device address of this device's copy of `scratch`
     int cu_count = 0;
-    bool cleared = false;           // the counters have been zeroed once on this device
 };
 std::mutex g_noalloc_mu;
 NoAllocDevice g_noalloc[kMaxDevices];
 
-__global__ void fill_zero_u32_kernel(unsigned* p, int n)
-{
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = 0u;
-}
-
 // the scratch of the current device as a Workspace; looks the address up on first use
-Workspace noalloc_scratch_for_current_device(hipStream_t stream)
+Workspace noalloc_scratch_for_current_device()
 {
     int device = 0;
     hip_ok(hipGetDevice(&device), "hipGetDevice");
@@ -191,25 +227,25 @@ Workspace noalloc_scratch_for_current_device(hipStream_t stream)
         d.ptr = ptr;
         d.cu_count = cus;
     }
-    unsigned* counters = (unsigned*)(d.ptr + kNoAllocPartialBytes);
-    if (!d.cleared) {
-        // Counters must start at zero; every launch leaves them at zero again (the last
-        // arrival resets its counter).  A fill kernel, not a memset: callers may be capturing.
-        hipLaunchKernelGGL(fill_zero_u32_kernel, dim3((kNoAllocCounters + 255) / 256), dim3(256), 0, stream, counters,
-                           kNoAllocCounters);
-        hip_ok(hipGetLastError(), "scratch counter fill");
-        d.cleared = true;
-    }
     Workspace ws;
     ws.partials = (float*)d.ptr;
-    ws.counters = counters;
-    ws.state_tables = nullptr;
+    ws.counters = (unsigned*)(d.ptr + kNoAllocCounterOff);
+    ws.accum = (unsigned long long*)(d.ptr + kNoAllocAccumOff);
+    ws.accum_slots = kNoAllocAccumSlots;
     ws.device = device;
     ws.cu_count = d.cu_count;
     ws.partial_bytes = kNoAllocPartialBytes;
     ws.counter_slots = kNoAllocCounters;
     ws.counter_words = kNoAllocCounters;
     ws.strict = true;
+    // the fault word of the library's workspace, if that exists already (no allocation here)
+    {
+        std::lock_guard<std::mutex> ws_lock(g_ws_mu);
+        if (g_ws[device].device >= 0) {
+            ws.fault_dev = g_ws[device].fault_dev;
+            ws.fault_host = g_ws[device].fault_host;
+        }
+    }
     return ws;
 }
 }  // namespace
@@ -231,7 +267,7 @@ extern "C" int berth_exl3_linear_noalloc(const void* a, const void* trellis, voi
             throw std::runtime_error("exl3 linear (no allocation): at most 8 rows (more rows need the library's workspace)");
         if (size_n / 128 > kNoAllocCounters)
             throw std::runtime_error("exl3 linear (no allocation): size_n exceeds the scratch's counter table");
-        const Workspace ws = noalloc_scratch_for_current_device((hipStream_t)stream);
+        const Workspace ws = noalloc_scratch_for_current_device();
         g_exl3_launch = launch_gemv(args, &ws);
         return 0;
     } catch (const std::exception& err) {
@@ -263,6 +299,27 @@ extern "C" int berth_kernels_init(int device)
         (void)hipGetLastError();
         return -1;
     }
+}
+
+// Reads the BERTH_* environment knobs again (they are otherwise read once per process).  Not
+// for use while another thread is launching.
+extern "C" void berth_kernels_reload_env(void) { reload_knobs(); }
+
+// Host-only query for sync points: 0 if no kernel on `device` has reported a fault since the
+// last report, else the fault code (and the report is cleared).  A bounded wait inside a
+// kernel that gives up stores its code in a host-visible word and leaves its part of the
+// output unwritten (MFMA split-K) or NaN (streaming GEMV); launches on the device also check
+// the word and fail, but a caller that synchronises and then launches nothing more, or
+// launches only kernels of other libraries, learns of it here.  Returns -1 on a bad device.
+extern "C" long long berth_kernels_pending_fault(int device)
+{
+    if (device < 0 || device >= kMaxDevices) return -1;
+    std::lock_guard<std::mutex> lock(g_ws_mu);
+    const Workspace& ws = g_ws[device];
+    if (ws.device < 0 || !ws.fault_host) return 0;
+    const unsigned code = *ws.fault_host;
+    if (code) *ws.fault_host = 0u;
+    return (long long)code;
 }
 
 // Diagnostics: the per-device internals (allocated on first use), for tools that inspect or
@@ -787,11 +844,10 @@ extern "C" int berth_ops_silu_mul(const void* gate, const void* up, void* out, i
 }
 
 // crates/berth-kernels/csrc/ops/mgemm.cu:125-272,296-340: same checks in the same order
-extern "C" int berth_ops_mgemm(const void* a, const void* b_list, void* c, const void* suh_list,
-                               void* a_had, const void* svh_list, int size_m, int size_k, int size_n,
-                               int k_bits, int codebook, int c_fp32, int bszm_in, int bszm_out,
-                               const int* size_n_list, const void* c_ptrs, const int* n_stride_list,
-                               const int* had_src_list, int num_had_src, void* stream)
+static int mgemm_entry(const void* a, const void* b_list, void* c, const void* suh_list, void* a_had,
+                       const void* svh_list, int size_m, int size_k, int size_n, int k_bits, int codebook, int c_fp32,
+                       int bszm_in, int bszm_out, const int* size_n_list, const void* c_ptrs, const int* n_stride_list,
+                       const int* had_src_list, int num_had_src, void* stream, bool host_lists)
 {
     try {
         g_ops_err.clear();
@@ -820,6 +876,7 @@ extern "C" int berth_ops_mgemm(const void* a, const void* b_list, void* c, const
         MgemmArgs m{a, b_list, c, suh_list, a_had, svh_list, size_m, size_k, size_n, k_bits, codebook, c_fp32,
                     bszm_in, bszm_out, size_n_list, c_ptrs, n_stride_list, had_src_list, num_had_src,
                     (hipStream_t)stream};
+        m.host_lists = host_lists;
         g_ops_launch = launch_mgemm(m);
         return 1;
     } catch (const std::exception& err) {
@@ -828,6 +885,26 @@ extern "C" int berth_ops_mgemm(const void* a, const void* b_list, void* c, const
         (void)hipGetLastError();
         return -1;
     }
+}
+
+extern "C" int berth_ops_mgemm(const void* a, const void* b_list, void* c, const void* suh_list,
+                               void* a_had, const void* svh_list, int size_m, int size_k, int size_n,
+                               int k_bits, int codebook, int c_fp32, int bszm_in, int bszm_out,
+                               const int* size_n_list, const void* c_ptrs, const int* n_stride_list,
+                               const int* had_src_list, int num_had_src, void* stream)
+{
+    return mgemm_entry(a, b_list, c, suh_list, a_had, svh_list, size_m, size_k, size_n, k_bits, codebook, c_fp32, bszm_in,
+                       bszm_out, size_n_list, c_ptrs, n_stride_list, had_src_list, num_had_src, stream, false);
+}
+
+extern "C" int berth_ops_mgemm_hostlists(const void* a, const void* b_list, void* c, const void* suh_list,
+                                         void* a_had, const void* svh_list, int size_m, int size_k, int size_n,
+                                         int k_bits, int codebook, int c_fp32, int bszm_in, int bszm_out,
+                                         const int* size_n_list, const void* c_ptrs, const int* n_stride_list,
+                                         const int* had_src_list, int num_had_src, void* stream)
+{
+    return mgemm_entry(a, b_list, c, suh_list, a_had, svh_list, size_m, size_k, size_n, k_bits, codebook, c_fp32, bszm_in,
+                       bszm_out, size_n_list, c_ptrs, n_stride_list, had_src_list, num_had_src, stream, true);
 }
 
 extern "C" const char* berth_ops_last_error(void) { return g_ops_err.c_str(); }

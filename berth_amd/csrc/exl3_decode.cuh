@@ -74,9 +74,22 @@ __device__ __forceinline__ void wait_own_stores() { asm volatile("s_waitcnt vmcn
 template <int LINES>
 __device__ __forceinline__ void touch_kernel_arguments()
 {
-    static_assert(LINES == 3 || LINES == 6 || LINES == 10, "instantiated line counts");
+    static_assert(LINES == 3 || LINES == 6 || LINES == 10 || LINES == 16, "instantiated line counts");
     const auto ka = __builtin_amdgcn_kernarg_segment_ptr();
     int t0, t1, t2, t3, t4, t5;
+    if constexpr (LINES == 16) {
+        int t6, t7, t8, t9, t10, t11, t12, t13, t14, t15;
+        asm volatile("s_load_dword %0, %16, 0x0\n\ts_load_dword %1, %16, 0x40\n\ts_load_dword %2, %16, 0x80\n\t"
+                     "s_load_dword %3, %16, 0xc0\n\ts_load_dword %4, %16, 0x100\n\ts_load_dword %5, %16, 0x140\n\t"
+                     "s_load_dword %6, %16, 0x180\n\ts_load_dword %7, %16, 0x1c0\n\ts_load_dword %8, %16, 0x200\n\t"
+                     "s_load_dword %9, %16, 0x240\n\ts_load_dword %10, %16, 0x280\n\ts_load_dword %11, %16, 0x2c0\n\t"
+                     "s_load_dword %12, %16, 0x300\n\ts_load_dword %13, %16, 0x340\n\ts_load_dword %14, %16, 0x380\n\t"
+                     "s_load_dword %15, %16, 0x3c0\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7),
+                       "=&s"(t8), "=&s"(t9), "=&s"(t10), "=&s"(t11), "=&s"(t12), "=&s"(t13), "=&s"(t14), "=&s"(t15)
+                     : "s"(ka));
+    } else
     if constexpr (LINES == 10) {
         int t6, t7, t8, t9;
         asm volatile("s_load_dword %0, %10, 0x0\n\ts_load_dword %1, %10, 0x40\n\ts_load_dword %2, %10, 0x80\n\t"

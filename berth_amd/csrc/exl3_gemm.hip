@@ -30,11 +30,7 @@ static void gemm_bits(const GemmParams& p, int bits, int cb, int mb, hipStream_t
 // workgroups share a tile), at least two k-blocks per workgroup, inside the workspace
 static int gemm_split(const Workspace& ws, long tiles, int KB, int mb)
 {
-    static const int per_cu = [] {
-        const char* e = std::getenv("BERTH_GEMM_WG_PER_CU");
-        int v = e ? std::atoi(e) : 0;
-        return v > 0 ? v : 1;
-    }();
+    const int per_cu = knobs().gemm_wg_per_cu > 0 ? knobs().gemm_wg_per_cu : 1;
     long S = ((long)ws.cu_count * per_cu + tiles - 1) / tiles;
     if (S > KB / 2) S = KB / 2;
     if (S < 1) S = 1;
@@ -48,11 +44,7 @@ static int gemm_split(const Workspace& ws, long tiles, int KB, int mb)
 // tile count of every launch the call makes
 static int gemm_counter_stride(long tiles)
 {
-    static const int cap = [] {
-        const char* e = std::getenv("BERTH_COUNTER_STRIDE");
-        const int v = e ? std::atoi(e) : 32;
-        return v < 1 ? 1 : (v > 32 ? 32 : v);
-    }();
+    const int cap = knobs().counter_stride;
     int stride = 1;
     while (stride * 2 <= cap && tiles * stride * 2 <= kCounters / 2) stride *= 2;
     return stride;
@@ -86,15 +78,9 @@ std::string launch_gemm(const LinearArgs& a)
     const int KB = a.size_k / 128;
     std::string desc;
     p.tile0 = 0;
-    static const int balance = [] {
-        const char* e = std::getenv("BERTH_GEMM_BALANCED");
-        return e ? std::atoi(e) : 1;
-    }();
+    const int balance = knobs().gemm_balanced;
     // 0: never 256-row tiles; 1 (default): where they are faster; 2: wherever they are possible
-    static const int rows256 = [] {
-        const char* e = std::getenv("BERTH_GEMM_ROWS256");
-        return e ? std::atoi(e) : 1;
-    }();
+    const int rows256 = knobs().gemm_rows256;
     // 128-row tiles rarely divide over the compute units (272 tiles on 256 units leave most of
     // the chip idle for the second half of the launch): deal the (tile, k-block) units out evenly.
     // 128-row tiles: one workgroup per compute unit, two when a workgroup still gets 16 k-blocks

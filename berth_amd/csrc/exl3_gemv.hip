@@ -43,23 +43,6 @@ void launch_gemv_stream_cb0(const StreamParams& p, int bits, int lutmask, dim3 g
 void launch_gemv_stream_cb1(const StreamParams& p, int bits, int lutmask, dim3 grid, hipStream_t stream);
 void launch_gemv_stream_cb2(const StreamParams& p, int bits, int lutmask, dim3 grid, hipStream_t stream);
 
-// ---- state -> weight tables of the three codebooks (one launch each at workspace set-up)
-template <int CB>
-__global__ void state_table_kernel(uint16_t* table)
-{
-    const uint32_t s = blockIdx.x * blockDim.x + threadIdx.x;
-    if (s < 65536u) table[s] = (uint16_t)(decode_pair<CB>(s, s) & 0xffffu);
-}
-
-void build_state_tables(uint16_t* tables)
-{
-    hipLaunchKernelGGL(state_table_kernel<0>, dim3(256), dim3(256), 0, 0, tables);
-    hipLaunchKernelGGL(state_table_kernel<1>, dim3(256), dim3(256), 0, 0, tables + 65536);
-    hipLaunchKernelGGL(state_table_kernel<2>, dim3(256), dim3(256), 0, 0, tables + 2 * 65536);
-    hip_ok(hipGetLastError(), "state_table_kernel launch");
-    hip_ok(hipStreamSynchronize(0), "state tables");
-}
-
 // ---- the one-row streaming kernel: the static split and when it applies
 //
 // Of a problem's U = (N/128) * (K/16) units every wave of its Gp workgroups takes q (the
@@ -70,32 +53,19 @@ void build_state_tables(uint16_t* tables)
 // for the operands the kernel divides.
 struct StreamPlan {
     bool ok = false;
-    int problems = 0, Gp = 0, maxc = 0;
+    int problems = 0, Gp = 0;
     unsigned q = 0, rem = 0, mq = 0, mq1 = 0, mtr = 0;
 };
 
-static int env_int(const char* name, int fallback)
-{
-    const char* e = std::getenv(name);
-    return e ? (int)std::strtol(e, nullptr, 0) : fallback;
-}
-
-// Knobs, read at every call (tests switch them inside one process):
-//   BERTH_GEMV_STREAM            0: never take the streaming kernel
-//   BERTH_GEMV_STREAM_MIN_UNITS  fewest tile rows per wave for which it is taken (default 4)
-//   BERTH_GEMV_STREAM_SHRINK     1: a smaller weight takes it with fewer workgroups instead of
-//                                falling back (default 0: the many-workgroup kernel is faster there)
-//   BERTH_GEMV_STREAM_WGS        cap on the workgroups per problem
-//   BERTH_GEMV_STREAM_LUT        table mask of the hybrid decode (bit pp: pair pp of every dword
-//                                comes from the table); 0: arithmetic only; unset: by size (below)
-// The 128 KiB table costs every workgroup a copy through its compute unit's load path (1.2 us
-// measured) and pays back about an eighth of the decode time at 4 bits per weight, where
-// the window halves feed the table addresses directly (335 MB weight: 103.6 -> 92.4 us); at
-// other bit rates the addresses cost a shift each and the gain was 1 % (27B lm_head, 6 bpw).
-// So: 4 bpw weights of at least 1 MiB per workgroup.
+// Hybrid decode (BERTH_GEMV_STREAM_LUT: bit pp set = pair pp of every dword comes from a
+// 128 KiB state -> weight table in LDS that the workgroup builds at its start; 0: arithmetic
+// only; unset: by size).  Building the table costs about two tile rows of decode per wave and
+// a table weight still costs 2.5 vector instructions against 4.4, with the random 2-byte LDS
+// reads as the next bound: it pays for long launches only (4 bpw, at least 1 MiB of weights
+// per workgroup: 335 MB weight 103.6 -> 92.4 us), not for the 10-30 us launches of a layer set.
 static int stream_lut_mask(int bits, unsigned long long bytes_per_workgroup)
 {
-    const int forced = env_int("BERTH_GEMV_STREAM_LUT", -1);
+    const int forced = knobs().gemv_stream_lut;
     if (forced >= 0) return forced;
     return bits == 4 && bytes_per_workgroup >= (1ull << 20) ? 0xA : 0;
 }
@@ -105,16 +75,16 @@ static unsigned magic(unsigned d) { return (unsigned)((1ull << 32) / d) + 1u; }
 static StreamPlan plan_stream(const Workspace& ws, int problems, int K, int N)
 {
     StreamPlan pl;
-    if (!env_int("BERTH_GEMV_STREAM", 1) || problems < 1 || problems > ws.cu_count) return pl;
+    const Knobs& kn = knobs();
+    if (!kn.gemv_stream || problems < 1 || problems > ws.cu_count || !ws.accum) return pl;
     const unsigned TR = (unsigned)K / 16, NB = (unsigned)N / 128, KB = (unsigned)K / 128;
     const unsigned long long U = (unsigned long long)NB * TR;
     if (U >= (1ull << 31)) return pl;
-    const unsigned min_units = (unsigned)std::max(2, env_int("BERTH_GEMV_STREAM_MIN_UNITS", 4));
+    const unsigned min_units = (unsigned)kn.gemv_stream_min_units;
     int Gp = ws.cu_count / problems;
-    const int cap = env_int("BERTH_GEMV_STREAM_WGS", 0);
-    if (cap > 0 && Gp > cap) Gp = cap;
+    if (kn.gemv_stream_wgs > 0 && Gp > kn.gemv_stream_wgs) Gp = kn.gemv_stream_wgs;
     if (U / ((unsigned)Gp * kStreamWaves) < min_units) {
-        if (!env_int("BERTH_GEMV_STREAM_SHRINK", 0)) return pl;
+        if (!kn.gemv_stream_shrink) return pl;
         Gp = (int)(U / (min_units * kStreamWaves));
         if (Gp < 1) return pl;
     }
@@ -125,13 +95,13 @@ static StreamPlan plan_stream(const Workspace& ws, int problems, int K, int N)
     const unsigned L = kStreamWaves * (q + 1);                 // most units of one workgroup
     if ((L + TR - 1) / TR + 1 > (unsigned)kStreamMaxCb) return pl;
     if (KB > (unsigned)kStreamXsBlocks && (L + 16 >= TR || L / 8 + 2 > (unsigned)kStreamXsBlocks)) return pl;
-    const unsigned maxc = (TR + kStreamWaves * q - 1) / (kStreamWaves * q) + 1;   // workgroups that can share a column block
-    if ((unsigned long long)problems * NB > (unsigned long long)ws.counter_slots) return pl;
-    if ((unsigned long long)problems * NB * maxc * 128 * sizeof(float) > ws.partial_bytes) return pl;
+    // workgroups that can share a column block: bounded by the accumulator word's count field
+    const unsigned sharers = (TR + kStreamWaves * q - 1) / (kStreamWaves * q) + 1;
+    if (sharers > (unsigned)kFixedMaxSharers) return pl;
+    if ((unsigned long long)problems * NB > (unsigned long long)ws.accum_slots) return pl;
     pl.ok = true;
     pl.problems = problems;
     pl.Gp = Gp;
-    pl.maxc = (int)maxc;
     pl.q = q;
     pl.rem = rem;
     pl.mq = magic(q);
@@ -143,23 +113,23 @@ static StreamPlan plan_stream(const Workspace& ws, int problems, int K, int N)
 static std::string run_stream(const Workspace& ws, const StreamPlan& pl, StreamParams& p, int bits, int cb,
                               hipStream_t stream)
 {
-    int mask = ws.state_tables ? stream_lut_mask(bits, (unsigned long long)pl.q * kStreamWaves * 256 * bits) : 0;
+    throw_pending_device_fault(ws);
+    int mask = stream_lut_mask(bits, (unsigned long long)pl.q * kStreamWaves * 256 * bits);
 #ifndef BERTH_STREAM_EXTRA_MASKS
     if (mask != 0) mask = 0xA;          // the one hybrid mask that is instantiated
 #endif
-    p.lut = ws.state_tables ? ws.state_tables + (size_t)cb * 65536 : nullptr;
-    p.partials = ws.partials;
-    p.counters = ws.counters;
+    p.accum = ws.accum;
+    p.fault = ws.fault_dev;
+    p.spin_limit = spin_limit();
     p.TR = p.K / 16;
     p.NB = p.N / 128;
-    p.cstride = counter_stride(ws, (long)pl.problems * p.NB);
     p.Gp = pl.Gp;
+    p.mgp = magic((unsigned)pl.Gp);
     p.q = pl.q;
     p.rem = pl.rem;
     p.mq = pl.mq;
     p.mq1 = pl.mq1;
     p.mtr = pl.mtr;
-    p.maxc = pl.maxc;
     const dim3 grid((unsigned)(pl.problems * pl.Gp));
     switch (cb) {
     case 0: launch_gemv_stream_cb0(p, bits, mask, grid, stream); break;
@@ -176,7 +146,7 @@ static std::string run_stream(const Workspace& ws, const StreamPlan& pl, StreamP
 
 static int wg_per_cu()
 {
-    const int x = env_int("BERTH_GEMV_WG_PER_CU", 0);
+    const int x = knobs().gemv_wg_per_cu;
     return x > 0 ? x : 6;
 }
 
@@ -208,10 +178,7 @@ static int pick_split(const Workspace& ws, long units, int KB, int mmax, bool tr
 // bound sits below them, and the split stays within one batch of the finisher's loads.
 static void pick_units(const Workspace& ws, GemvParams& p, long units, int mmax)
 {
-    static const int allow = [] {
-        const char* e = std::getenv("BERTH_GEMV_HALF_UNITS");
-        return e ? std::atoi(e) : 1;
-    }();
+    const int allow = knobs().gemv_half_units;
     p.half_units = 0;
     if (allow && mmax == 1 && units * p.KB <= (long)ws.cu_count * 6) {
         const int S = pick_split(ws, units, 2 * p.KB, mmax, true);
@@ -333,6 +300,50 @@ std::string launch_mgemm(const MgemmArgs& m)
     Workspace& ws = workspace_for_current_device();
     const bool sliced = m.had_src_list != nullptr;
     const int mmax = m.size_m == 1 ? 1 : 8;
+    if (m.host_lists) {
+        // the lists are host memory: the problems travel by value in the kernel arguments
+        const StreamPlan pl = m.size_m == 1 && m.bszm_out <= kStreamMaxSlices
+                                  ? plan_stream(ws, m.bszm_out, m.size_k, m.size_n) : StreamPlan{};
+        if (!pl.ok)
+            throw std::runtime_error("exl3_mgemm (host lists): serves one row, at most " + std::to_string(kStreamMaxSlices) +
+                                     " slices and weights large enough for the streaming kernel; pass device lists to "
+                                     "berth_ops_mgemm otherwise");
+        StreamParams sp{};
+        sp.a = (const _Float16*)m.a;
+        sp.a_had = (_Float16*)m.a_had;
+        sp.mode = 3;
+        sp.in_stride = (!sliced && m.bszm_in > 1) ? m.size_k : 0;
+        sp.K = m.size_k;
+        sp.N = m.size_n;
+        sp.out_fp32 = m.c_fp32;
+        const uint64_t* b = (const uint64_t*)m.b_list;
+        const uint64_t* su = (const uint64_t*)m.suh_list;
+        const uint64_t* sv = (const uint64_t*)m.svh_list;
+        for (int i = 0; i < m.bszm_out; ++i) {
+            StreamSlice& sl = sp.slice[i];
+            sl.trellis = (const uint32_t*)b[i];
+            sl.svh = (const _Float16*)sv[i];
+            if (sliced) {
+                const int src = m.had_src_list[i];
+                if (src < 0 || src >= m.num_had_src) throw std::runtime_error("exl3_mgemm (host lists): had_src_list entry out of range");
+                if (m.size_n_list[i] < 0 || m.size_n_list[i] > m.size_n || m.size_n_list[i] % 128 != 0)
+                    throw std::runtime_error("exl3_mgemm (host lists): size_n_list entry must be a multiple of 128 within size_n");
+                sl.suh = (const _Float16*)su[src];
+                sl.c = (void*)((const uint64_t*)m.c_ptrs)[i];
+                sl.width = m.size_n_list[i];
+                sl.n_stride = m.n_stride_list[i];
+                sl.had_slab = src;
+            } else {
+                sl.suh = (const _Float16*)su[i];
+                sl.c = (char*)m.c + (size_t)i * m.size_n * (m.c_fp32 ? 4 : 2);
+                sl.width = m.size_n;
+                sl.n_stride = m.size_n;
+                sl.had_slab = i;
+            }
+        }
+        return std::string(sliced ? "sliced x" : "uniform x") + std::to_string(m.bszm_out) + " by value " +
+               run_stream(ws, pl, sp, m.k_bits, m.codebook, m.stream);
+    }
     if (m.size_m == 1) {
         const StreamPlan pl = plan_stream(ws, m.bszm_out, m.size_k, m.size_n);
         if (pl.ok) {

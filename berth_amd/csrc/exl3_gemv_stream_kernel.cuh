@@ -13,26 +13,32 @@
 //     evenly: wave W takes q units, the first `rem` waves one more.  No second round, no
 //     tail of half-empty compute units: the grid is at most the number of compute units
 //     and every wave does the same amount of decode.
-//   * A wave keeps a ring of RING tile rows in registers; a tile row is reloaded with the
-//     tile row RING units ahead as soon as it has been decoded.  The walk crosses column
+//   * A wave keeps a ring of two tile rows in registers; a tile row is reloaded with the
+//     tile row two units ahead as soon as it has been decoded.  The walk crosses column
 //     block boundaries without draining the ring.
 //   * The workgroup rotates the activation of the k-blocks its units touch once, into
 //     LDS (every wave takes some k-blocks), and writes a_had for the k-blocks whose
-//     column-block-0 units it owns.
-//   * Decode is a hybrid: of the four weight pairs of a dword, those selected by LUTMASK
-//     come from a 128 KiB state -> fp16 table in LDS (copied from device memory with
-//     LDS-direct loads while the first tile rows are in flight), the others from the
-//     codebook arithmetic.  The table read costs address + read + pack (2.5 vector
-//     instructions per weight with the dot product) against 4.25 for the arithmetic;
-//     the LDS read rate bounds how many can go that way.
+//     column-block-0 units it owns.  Those loads go out first of all, ahead of the split
+//     arithmetic of the wave and of its first tile row: the barrier behind the rotation
+//     is what the whole workgroup waits for.
+//   * Decode is optionally a hybrid: of the four weight pairs of a dword, those selected
+//     by LUTMASK come from a 128 KiB state -> fp16 table in LDS, which the workgroup builds
+//     in place while its first loads are in flight, the others from the codebook
+//     arithmetic.  The table read costs address + read + pack (2.5 vector instructions
+//     per weight with the dot product) against 4.4 for the arithmetic; the LDS read rate
+//     bounds how many can go that way.
 //   * Partial sums: a wave writes one 128-column partial per column block it touched
-//     into LDS; a column block that lies entirely inside the workgroup's units is
-//     finished there; otherwise the workgroup's partial goes to the library workspace
-//     and the last workgroup to arrive adds the partials in workgroup order.  Every
-//     summation order is fixed by the static split.
+//     into LDS, and the pieces of a column block are added in wave order.  A column block
+//     that lies entirely inside the workgroup's units is finished there.  Otherwise every
+//     workgroup that shares it adds its part, converted to 64-bit fixed point, onto the
+//     block's accumulator words with one atomic add that returns the old value: integer
+//     sums do not depend on the order of the adds, and the add that completes the count
+//     has learnt the total in that same round trip and finishes the block.  So results
+//     repeat bit for bit, and the hand-over is one memory round trip.
 #pragma once
 
 #include "exl3_gemv_kernel.cuh"
+
 
 #include <utility>
 
@@ -48,6 +54,16 @@ __host__ __device__ constexpr int stream_lds_bytes(int lutmask)
     return (lutmask ? 131072 : 0) + kStreamXsBlocks * 256 + kStreamPieces * 512 + 128;
 }
 
+// one problem of a bundle whose lists the host knows (mode 3)
+struct StreamSlice {
+    const uint32_t* trellis;
+    const _Float16* suh;
+    const _Float16* svh;
+    void* c;
+    int width, n_stride, had_slab, pad;
+};
+constexpr int kStreamMaxSlices = 16;
+
 struct StreamParams {
     const _Float16* a;          // input row(s): fp16 [K] (per problem when in_stride != 0)
     const _Float16* a_up;       // optional: the input is silu(a) * a_up
@@ -62,38 +78,23 @@ struct StreamParams {
     const int* n_stride_list;
     const int* had_src_list;
     _Float16* a_had;            // optional; slab per rotation source
-    const uint16_t* lut;        // [65536] fp16 bits of every state of this codebook (LUTMASK != 0)
-    float* partials;            // [problem][column block][contributor][128]
-    unsigned* counters;         // [problem][column block], cstride words apart, zero between launches
-    int cstride;
-    int mode;                   // 0 by value, 1 uniform lists, 2 sliced lists
+    int mode;                   // 0 by value, 1 uniform lists, 2 sliced lists, 3 slices by value
     int in_stride;              // elements between the inputs of consecutive problems (0: shared)
     int K, N, NB, TR;           // N: row stride of trellis and output in mode 0 / 1; TR = K / 16
     int out_fp32;
     int Gp;                     // workgroups per problem (gridDim.x = problems * Gp)
+    unsigned mgp;               // floor(2^32 / Gp) + 1
     unsigned q, rem;            // units per wave; the first `rem` waves of a problem take q + 1
     unsigned mq, mq1, mtr;      // floor(2^32 / d) + 1 for d = q, q + 1, TR (exact for the operands used)
-    int maxc;                   // contributor slots per column block in `partials`
-#ifdef BERTH_STREAM_TRACE
-    unsigned long long* trace;  // [wave][8] timestamps (instrumented builds only)
-#endif
+    unsigned long long* accum;  // [problem][column block][128] fixed-point sums, zero between launches
+    unsigned* fault;            // host-visible word for a finisher that gives up its bounded wait
+    unsigned spin_limit;
+    StreamSlice slice[kStreamMaxSlices];    // mode 3: the problems, by value
 };
 
 __device__ __forceinline__ unsigned div_magic(unsigned n, unsigned m) { return __umulhi(n, m); }
 
-// phase timestamps of an instrumented build (a measurement aid; compiled out otherwise)
-#ifdef BERTH_STREAM_TRACE
-#define BERTH_STREAM_STAMP(i)                                                                      \
-    do {                                                                                           \
-        if (lane == 0)                                                                             \
-            p.trace[((size_t)blockIdx.x * kStreamWaves + wave) * 8 + (i)] = wall_clock64(); \
-    } while (0)
-#else
-#define BERTH_STREAM_STAMP(i) do { } while (0)
-#endif
-
 typedef __attribute__((address_space(3))) const uint16_t* lds_u16_ptr;
-typedef __attribute__((address_space(3))) void* lds_void_ptr;
 
 // LDS byte address 2 * s of the table entry of the 16-bit state in the low / high half of r
 __device__ __forceinline__ uint32_t lut_addr_lo(uint32_t r)
@@ -196,6 +197,28 @@ struct HybridDecode {
     }
 };
 
+
+// Cross-workgroup sums of a column block travel as 64-bit words of three fields: bits 16..63
+// the value as a signed integer in units of 2^-18, bits 8..15 the number of contributions that
+// did not fit (magnitude 2^23 or more, or not a number), bits 0..7 the number of contributions.
+// Integer addition is associative, so the sharers' atomic adds give the same bits in whatever
+// order they land, and the add that returns the full count has learnt the total in the same
+// round trip.  At most 64 sharers add to a word, so neither the counts nor the value wrap; a
+// word with a contribution that did not fit yields a NaN.
+constexpr int kFixedBits = 18;
+constexpr int kFixedMaxSharers = 64;
+__device__ __forceinline__ unsigned long long to_fixed_tagged(float z)
+{
+    const double d = (double)z * (double)(1 << kFixedBits);
+    if (!(__builtin_fabs(d) < 2199023255552.0)) return 0x101ull;          // 2^41
+    return ((unsigned long long)(long long)__builtin_rint(d) << 16) | 1ull;
+}
+__device__ __forceinline__ float from_fixed_tagged(unsigned long long t)
+{
+    if ((t >> 8) & 0xffull) return __builtin_nanf("");
+    return (float)((double)((long long)t >> 16) * (1.0 / (double)(1 << kFixedBits)));
+}
+
 // f(0); if more: f(1); ... each call nested inside the previous one's branch
 template <int J, int N, class F>
 __device__ __forceinline__ void nested_tail(unsigned count, F&& f)
@@ -208,11 +231,15 @@ __device__ __forceinline__ void nested_tail(unsigned count, F&& f)
     }
 }
 
+// Tile rows a wave keeps in flight.  Two: with sixteen waves per compute unit that is what the
+// memory's latency takes at the rate the decode consumes them; deeper rings only lengthen the
+// queues that everything else (the first loads of the launch, the hand-over at its end) waits in
+// (27B layer set at 4 bits per weight, four launches: 67.1 us with four, 65.3 with two).
 #ifndef BERTH_STREAM_RING
-#define BERTH_STREAM_RING 4
+#define BERTH_STREAM_RING 2
 #endif
 template <int BITS> struct StreamRing {
-    static constexpr int depth = BITS <= 4 ? BERTH_STREAM_RING : (BITS <= 6 ? (BERTH_STREAM_RING * 3) / 4 : BERTH_STREAM_RING / 2);
+    static constexpr int depth = BERTH_STREAM_RING;
 };
 
 // a pointer every lane of the wave agrees on, moved to scalar registers
@@ -234,24 +261,32 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
     constexpr int kRedOff = kXsOff + kStreamXsBlocks * 256;
     constexpr int kMetaOff = kRedOff + kStreamPieces * 512;
     constexpr int RING = StreamRing<BITS>::depth;
-    constexpr int kRowLoads = BITS % 4 == 0 ? BITS / 4 : (BITS % 2 == 0 ? BITS / 2 : BITS);   // load instructions per tile row
     uint32_t* const xs = (uint32_t*)(lds + kXsOff);
     float* const red = (float*)(lds + kRedOff);
     unsigned* const piece_first = (unsigned*)(lds + kMetaOff);
     unsigned* const piece_last = piece_first + 16;
 
-    static_assert(sizeof(StreamParams) > 2 * 64 && sizeof(StreamParams) <= 6 * 64, "argument lines touched below");
-    touch_kernel_arguments<3>();
+    static_assert(sizeof(StreamParams) > 15 * 64 && sizeof(StreamParams) <= 16 * 64, "argument lines touched below");
+    touch_kernel_arguments<16>();
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int prob = blockIdx.x / p.Gp;
-    const int gl = blockIdx.x - prob * p.Gp;
+    const unsigned prob = div_magic(blockIdx.x, p.mgp);
+    const unsigned gl = blockIdx.x - prob * (unsigned)p.Gp;
 
     // ---- this problem's tensors
     ExpertLin lin = p.lin[p.mode == 0 ? prob : 0];
     int n_stride = p.N, had_slab = 0, width = p.N;
     void* cout = p.c[p.mode == 0 ? prob : 0];
-    if (p.mode) {
+    if (p.mode == 3) {
+        const StreamSlice& sl = p.slice[prob];
+        lin.trellis = sl.trellis;
+        lin.suh = sl.suh;
+        lin.svh = sl.svh;
+        cout = sl.c;
+        width = sl.width;
+        n_stride = sl.n_stride;
+        had_slab = sl.had_slab;
+    } else if (p.mode) {
         lin.trellis = (const uint32_t*)p.b_list[prob];
         lin.svh = (const _Float16*)p.svh_list[prob];
         if (p.mode == 2) {
@@ -262,83 +297,55 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
             cout = (void*)p.c_ptrs[prob];
         } else {
             lin.suh = (const _Float16*)p.suh_list[prob];
-            had_slab = prob;
+            had_slab = (int)prob;
             cout = (char*)p.c[0] + (size_t)prob * p.N * (p.out_fp32 ? 4 : 2);
         }
     }
     const bool write_had = p.a_had && (p.mode != 0 || prob == 0);
 
-    // ---- the static split: units of this workgroup and of this wave
+    // ---- the static split, workgroup level: units [u0, u1)
     // (a slice narrower than the bundle's width ends early: its units stop at its last column block)
     const unsigned TR = (unsigned)p.TR;
     const unsigned u_end = (unsigned)(width >> 7) * TR;
-    const unsigned W0 = (unsigned)gl * kStreamWaves;
+    const unsigned W0 = gl * kStreamWaves;
     const unsigned u0 = min(W0 * p.q + min(W0, p.rem), u_end);
     const unsigned u1 = min((W0 + kStreamWaves) * p.q + min(W0 + kStreamWaves, p.rem), u_end);
     if (u0 >= u1) return;
-    const unsigned Ww = W0 + (unsigned)wave;
-    const unsigned uw0 = min(Ww * p.q + min(Ww, p.rem), u_end);
-    const unsigned uw1 = min((Ww + 1) * p.q + min(Ww + 1, p.rem), u_end);
     const unsigned cb_first = div_magic(u0, p.mtr);
-    const unsigned cb_last = div_magic(u1 - 1, p.mtr);
-    const unsigned ncb = cb_last - cb_first + 1;
-
-    BERTH_STREAM_STAMP(0);
-    if (threadIdx.x < 16) {
-        piece_first[threadIdx.x] = 0xffffffffu;
-        piece_last[threadIdx.x] = 0u;
-    }
-
-    // ---- rotate the k-blocks this workgroup's units touch.  Region A: the k-blocks of the
-    // first column block's units (or all of K); region B, behind it: those of the second
-    // column block's units, which start at k-block 0, when the two do not cover all of K.
+    // The k-blocks these units touch are a cyclic run of nk k-blocks from that of the first
+    // unit (the walk wraps from the last tile row of a column block to tile row 0 of the
+    // next); k-block a_lo + i, taken modulo K / 128, is held in slot i of the LDS region.
     const unsigned KB = TR >> 3;
-    unsigned a_lo, n_a, n_b;
-    {
-        const unsigned r_lo = u0 - cb_first * TR;
-        if (ncb == 1) {
-            a_lo = r_lo >> 3;
-            n_a = ((u1 - 1 - cb_first * TR) >> 3) - a_lo + 1;
-            n_b = 0;
-        } else {
-            a_lo = r_lo >> 3;
-            n_a = KB - a_lo;
-            n_b = ncb == 2 ? ((u1 - 1 - cb_last * TR) >> 3) + 1 : KB;
-            if (n_b >= a_lo) { a_lo = 0; n_a = KB; n_b = 0; }      // together they cover all of K
-        }
+    const unsigned r_lo = u0 - cb_first * TR;
+    unsigned a_lo = r_lo >> 3;
+    unsigned nk = ((r_lo & 7u) + (u1 - u0) + 7u) >> 3;
+    if (nk >= KB) {
+        nk = KB;
+        a_lo = 0;
     }
-    // the activation and scales of this wave's k-blocks (at most 64 / 16 = 4) are requested
-    // ahead of the ring; the rotation itself runs once they are there, with the ring in flight
+    // ---- first of all the activation and the scales of this wave's share of those k-blocks
+    // (slots wave, wave + 16, ...): the rotation is what the whole workgroup waits for
     constexpr int kRot = kStreamXsBlocks / kStreamWaves;
     const global_ptr<const half2_t> xin = (global_ptr<const half2_t>)as_global(p.a + (size_t)prob * p.in_stride);
     const global_ptr<const half2_t> uin = (global_ptr<const half2_t>)as_global(p.a_up + (size_t)prob * p.in_stride);
     const global_ptr<const half2_t> sin = (global_ptr<const half2_t>)as_global(lin.suh);
     half2_t rot_x[kRot], rot_s[kRot], rot_u[kRot];
+    unsigned rot_kb[kRot];
 #pragma unroll
     for (int t = 0; t < kRot; ++t) {
         const unsigned i = (unsigned)wave + t * kStreamWaves;
-        const unsigned ic = i < n_a + n_b ? i : 0u;                     // past the end: any valid k-block, unused
-        const unsigned kb = ic < n_a ? a_lo + ic : ic - n_a;
+        unsigned kb = a_lo + (i < nk ? i : 0u);                         // past the end: any valid k-block, unused
+        kb = kb >= KB ? kb - KB : kb;
+        rot_kb[t] = kb;
         rot_x[t] = xin[kb * 64 + lane];
         rot_s[t] = sin[kb * 64 + lane];
         if (SILU) rot_u[t] = uin[kb * 64 + lane];
     }
-    // ---- the table: 128 KiB from device memory straight into LDS, 8 KiB per wave
-    if constexpr (LUTMASK != 0) {
-        const global_ptr<const unsigned char> src = (global_ptr<const unsigned char>)as_global((const unsigned char*)p.lut);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int off = (wave * 8 + i) * 1024;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + off + lane * 16),
-                                             (lds_void_ptr)(lds + off), 16, 0, 0);
-        }
-    }
-    // A compute unit serves its waves' vector memory requests in arrival order: the bulk loads
-    // of the ring must not get ahead of another wave's few loads above, on which the whole
-    // workgroup waits.  So every wave has issued those before any wave issues its ring.
-    __builtin_amdgcn_s_barrier();
-    BERTH_STREAM_STAMP(1);
-    // ---- ring prologue: the first RING tile rows of this wave
+
+    // ---- this wave's units [uw0, uw1) and its first tile row
+    const unsigned Ww = W0 + (unsigned)wave;
+    const unsigned uw0 = min(Ww * p.q + min(Ww, p.rem), u_end);
+    const unsigned uw1 = min((Ww + 1) * p.q + min(Ww + 1, p.rem), u_end);
     constexpr int tile_dw = 8 * BITS;
     const long row_dw = (long)(n_stride >> 4) * tile_dw;
     const long wrap_dw = (long)(8 * tile_dw) - (long)(TR - 1) * row_dw;
@@ -355,22 +362,49 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
     unsigned p_r = r;                                       // tile row of the unit pbase points at
     unsigned p_left = uw0 < uw1 ? uw1 - uw0 - 1 : 0u;       // units after it that are still this wave's
     uint32_t own[RING][BITS];
-#pragma unroll
-    for (int j = 0; j < RING; ++j) {
+    auto prologue_row = [&](int j) {
         load_tile_dwords<BITS>(pbase + lane_dw, own[j]);
         const long step = p_left == 0 ? 0 : (p_r == TR - 1 ? wrap_dw : row_dw);
         pbase += step;
         p_r = p_left == 0 ? p_r : (p_r == TR - 1 ? 0u : p_r + 1);
         p_left = p_left == 0 ? 0u : p_left - 1;
         __builtin_amdgcn_sched_barrier(0);
+    };
+    // Only the first tile row goes out ahead of the rotation: whole rings of sixteen waves are
+    // more than the compute unit's request queue holds, the later waves would sit in the
+    // issue of their loads until the burst has drained at the memory's rate, and the barrier
+    // below waits for the slowest wave.
+    prologue_row(0);
+    // the output scale of the column block this wave finishes at the end: asked for now, so
+    // that the hand-over does not wait for it
+    const unsigned cb_last = div_magic(u1 - 1, p.mtr);
+    const unsigned ncb = cb_last - cb_first + 1;
+    half2_t sv_mine = {};
+    if ((unsigned)wave < ncb && (cb_first + (unsigned)wave) * 128u < (unsigned)width)
+        sv_mine = ((global_ptr<const half2_t>)as_global(lin.svh + (cb_first + (unsigned)wave) * 128))[lane];
+    if (threadIdx.x < 16) {
+        piece_first[threadIdx.x] = 0xffffffffu;
+        piece_last[threadIdx.x] = 0u;
     }
 
-    BERTH_STREAM_STAMP(2);
-    half2_t rotated[kRot];
+    // ---- the table: built in place while the first tile rows and the activation are on
+    // their way (the vector ALU has nothing else to do until they arrive).  Thread t writes
+    // the entries of states 2 (t + 1024 j), + 1 as one dword: consecutive lanes, consecutive
+    // dwords.
+    if constexpr (LUTMASK != 0) {
+        uint32_t* const tab = (uint32_t*)lds;
+#pragma unroll 8
+        for (int j = 0; j < 32; ++j) {
+            const uint32_t s2 = 2u * (threadIdx.x + 1024u * (unsigned)j);
+            tab[threadIdx.x + 1024u * (unsigned)j] = decode_pair<CB>(s2, s2 + 1u);
+        }
+    }
+    // ---- rotate; a_had: the workgroup that owns tile row 8 * kb of column block 0 writes k-block kb
+    const global_ptr<half2_t> hout = (global_ptr<half2_t>)as_global(p.a_had + (size_t)had_slab * p.K);
 #pragma unroll
     for (int t = 0; t < kRot; ++t) {
         const unsigned i = (unsigned)wave + t * kStreamWaves;
-        if (i >= n_a + n_b) break;
+        if (i >= nk) break;
         half2_t x = rot_x[t];
         if (SILU) {
             x.x = silu_mul_h(x.x, rot_u[t].x);
@@ -379,30 +413,21 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
         float v0 = (float)x.x * (float)rot_s[t].x;
         float v1 = (float)x.y * (float)rot_s[t].y;
         had128_wave(v0, v1, lane);
-        rotated[t].x = (_Float16)(v0 * kRsqrt128);
-        rotated[t].y = (_Float16)(v1 * kRsqrt128);
-        xs[i * 64 + lane] = as_u32(rotated[t]);
-    }
-    // The table has to be complete at the barrier; the ring stays in flight.  Vector memory
-    // operations complete in issue order, so "all but the ring's loads" covers the table copy.
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(RING * kRowLoads) : "memory");
-    if (write_had) {
-        // a_had: the workgroup that owns tile row 8 * kb of column block 0 writes k-block kb
-        const global_ptr<half2_t> hout = (global_ptr<half2_t>)as_global(p.a_had + (size_t)had_slab * p.K);
-#pragma unroll
-        for (int t = 0; t < kRot; ++t) {
-            const unsigned i = (unsigned)wave + t * kStreamWaves;
-            if (i >= n_a + n_b) break;
-            const unsigned kb = i < n_a ? a_lo + i : i - n_a;
-            if (u0 <= 8 * kb && 8 * kb < u1) hout[kb * 64 + lane] = rotated[t];
-        }
+        half2_t rotated;
+        rotated.x = (_Float16)(v0 * kRsqrt128);
+        rotated.y = (_Float16)(v1 * kRsqrt128);
+        xs[i * 64 + lane] = as_u32(rotated);
+        if (write_had && u0 <= 8 * rot_kb[t] && 8 * rot_kb[t] < u1) hout[rot_kb[t] * 64 + lane] = rotated;
     }
     __syncthreads();
-    BERTH_STREAM_STAMP(3);
+    // the rest of the ring goes out behind the barrier: a wave whose loads wait for room in
+    // the compute unit's request queue then holds up nobody but itself
+#pragma unroll
+    for (int j = 1; j < RING; ++j) prologue_row(j);
 
     // ---- the walk
     // LDS byte offset of the rotated activation of tile row r of the current column block
-    const unsigned xoff_wrap = kXsOff + (n_b ? n_a * 256u : 0u) - (n_b ? 0u : a_lo * 256u);   // tile row 0 of a later column block
+    const unsigned xoff_wrap = kXsOff + (a_lo ? (KB - a_lo) * 256u : 0u);     // tile row 0 of a later column block
     unsigned xoff = kXsOff + (r << 5) - a_lo * 256u;
     if (cb != cb_first) xoff = xoff_wrap + (r << 5);
     unsigned piece = (unsigned)wave + (cb - cb_first);
@@ -475,25 +500,34 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
     // whole rings: straight-line, one exit, so that the wait before each tile row's use
     // is exactly "all but the RING - 1 loads issued after it"
     const unsigned groups = left / RING;
+    // A wave runs its tile rows at the highest user priority and steps it down over the
+    // second half of its run (to 2 at a half, 1 at three quarters, 0 for the last eighth).
+    // Measured on the four launches of a 27B layer set, interleaved runs on one machine:
+    // 66.4 us without, 64.9 with a constant 3, 63.3 with quarter steps, 62.9 with these;
+    // the opposite ramp and two ramps per run are no better than none.
+    const unsigned g1 = groups >> 1, g2 = groups - (groups >> 2), g3 = groups - (groups >> 3);
+    __builtin_amdgcn_s_setprio(3);
     for (unsigned g = 0; g < groups; ++g) {
+        if (g == g1) __builtin_amdgcn_s_setprio(2);
+        if (g == g2) __builtin_amdgcn_s_setprio(1);
+        if (g == g3) __builtin_amdgcn_s_setprio(0);
 #pragma unroll
         for (int j = 0; j < RING; ++j) stage(own[j], true);
     }
+    __builtin_amdgcn_s_setprio(0);
     // the remaining tile rows (fewer than RING), nested so that each is reached one way only
     const unsigned tail = left - groups * RING;
     nested_tail<0, RING - 1>(tail, [&](auto J) { stage(own[decltype(J)::value], false); });
-    BERTH_STREAM_STAMP(4);
     if (r != 0 && uw0 < uw1) flush(piece);
     __syncthreads();
-    BERTH_STREAM_STAMP(5);
 
     // ---- finish the column blocks: wave w takes column blocks cb_first + w, + 16, ...
     const long pslot = (long)prob * p.NB;
+    static_assert(kStreamMaxCb <= kStreamWaves, "one pass: wave w finishes column block cb_first + w");
     for (unsigned cbi = (unsigned)wave; cbi < ncb; cbi += kStreamWaves) {
         const unsigned cbx = cb_first + cbi;
         if (cbx * 128u >= (unsigned)width) continue;             // a narrower slice of a bundle: nothing there
-        // requested before the hand-over below, whose waits it would otherwise queue behind
-        const half2_t sv = ((global_ptr<const half2_t>)as_global(lin.svh + cbx * 128))[lane];
+        const half2_t sv = sv_mine;
         const unsigned wf = piece_first[cbi], wl = piece_last[cbi];
         float z0 = 0.0f, z1 = 0.0f;
         for (unsigned wv = wf; wv <= wl; ++wv) {
@@ -509,36 +543,36 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
             const unsigned big = p.rem * (p.q + 1);
             const unsigned wa = ua < big ? div_magic(ua, p.mq1) : p.rem + div_magic(ua - big, p.mq);
             const unsigned wb = ub < big ? div_magic(ub, p.mq1) : p.rem + div_magic(ub - big, p.mq);
-            const unsigned gf = wa >> 4, count = (wb >> 4) - gf + 1;
-            float* slab = p.partials + ((pslot + cbx) * p.maxc) * 128;
-            union Pair { unsigned long long u; float f[2]; } mine;
-            mine.f[0] = z0;
-            mine.f[1] = z1;
-            __hip_atomic_store((unsigned long long*)(slab + ((unsigned)gl - gf) * 128 + 2 * lane), mine.u, __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-            wait_own_stores();
-            unsigned old = 0;
-            if (lane == 0)
-                old = __hip_atomic_fetch_add(p.counters + (size_t)(pslot + cbx) * p.cstride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            old = (unsigned)__builtin_amdgcn_readfirstlane((int)old);
-            if (old != count - 1) continue;
-            if (lane == 0) __hip_atomic_store(p.counters + (size_t)(pslot + cbx) * p.cstride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            z0 = z1 = 0.0f;
-            for (unsigned j0 = 0; j0 < count; j0 += 8) {
-                Pair part[8];
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    const unsigned j = j0 + t < count ? j0 + t : count - 1;
-                    part[t].u = __hip_atomic_load((const unsigned long long*)(slab + j * 128 + 2 * lane), __ATOMIC_RELAXED,
-                                                  __HIP_MEMORY_SCOPE_AGENT);
+            const unsigned count = (wb >> 4) - (wa >> 4) + 1;
+            unsigned long long* const word = p.accum + ((size_t)(pslot + cbx) * 128 + 2 * lane);
+            const unsigned long long f0 = to_fixed_tagged(z0), f1 = to_fixed_tagged(z1);
+            unsigned long long t0 = __hip_atomic_fetch_add(word, f0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + f0;
+            unsigned long long t1 = __hip_atomic_fetch_add(word + 1, f1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + f1;
+            // the sharer whose add completed column 0 finishes the column block
+            if ((unsigned)__builtin_amdgcn_readfirstlane((int)((unsigned)t0 & 0xffu)) != count) continue;
+            // usually every column is complete by then; one that another sharer's add had not
+            // reached yet is read again (that sharer's add is in flight: the wait is short)
+            unsigned spins = 0;
+            while (true) {
+                const bool done = ((unsigned)t0 & 0xffu) == count && ((unsigned)t1 & 0xffu) == count;
+                if (__builtin_amdgcn_ballot_w64(!done) == 0ull) break;
+                if (++spins > p.spin_limit) {
+                    // a contributor is missing (a stale accumulator, two launches mixed on one
+                    // device): say so, and leave no plausible numbers behind
+                    if (p.fault && lane == 0)
+                        __hip_atomic_store(p.fault, 0x40000001u + (unsigned)cbx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    t0 = t1 = 0x100ull;
+                    break;
                 }
-#pragma unroll
-                for (int t = 0; t < 8; ++t)
-                    if (j0 + t < count) {
-                        z0 += part[t].f[0];
-                        z1 += part[t].f[1];
-                    }
+                if (!done) {
+                    t0 = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    t1 = __hip_atomic_load(word + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
             }
+            __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(word + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            z0 = from_fixed_tagged(t0);
+            z1 = from_fixed_tagged(t1);
         }
         // output Hadamard, svh, store
         had128_wave(z0, z1, lane);
@@ -553,7 +587,6 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
             *(half2_t*)((_Float16*)cout + at) = o;
         }
     }
-    BERTH_STREAM_STAMP(6);
 }
 
 }  // namespace berth

@@ -34,7 +34,8 @@ inline void raise_dynamic_lds_limit(const void* kernel, int bytes, bool (&done)[
 struct Workspace {
     float* partials = nullptr;      // kPartialBytes
     unsigned* counters = nullptr;   // kCounters entries, zero between launches
-    uint16_t* state_tables = nullptr;   // [3 codebooks][65536] fp16 bits of every trellis state, or null
+    unsigned long long* accum = nullptr;   // zero between launches: fixed-point column-block sums of the streaming GEMV
+    int accum_slots = 0;            // column blocks (1 KiB each) behind `accum`
     int device = -1;
     int cu_count = 0;
     // One word of host-pinned memory that kernels can write (device address fault_dev, host
@@ -49,6 +50,32 @@ struct Workspace {
 };
 constexpr size_t kPartialBytes = (size_t)256 << 20;
 constexpr int kCounters = 65536;
+constexpr int kAccumSlots = 16384;     // column blocks of a streaming launch (16 MiB of accumulators)
+// The BERTH_* environment knobs, read once per process into one record; no launch calls
+// getenv.  berth_kernels_reload_env() reads them again (tests that switch a knob inside one
+// process call it after changing the environment).
+struct Knobs {
+    int gemv_stream;            // BERTH_GEMV_STREAM            0: never take the streaming kernel
+    int gemv_stream_min_units;  // BERTH_GEMV_STREAM_MIN_UNITS  fewest tile rows per wave for which it is taken
+    int gemv_stream_shrink;     // BERTH_GEMV_STREAM_SHRINK     1: fewer workgroups instead of falling back
+    int gemv_stream_wgs;        // BERTH_GEMV_STREAM_WGS        cap on the workgroups per problem (0: none)
+    int gemv_stream_lut;        // BERTH_GEMV_STREAM_LUT        table mask of the hybrid decode (-1: by size)
+    int gemv_wg_per_cu;         // BERTH_GEMV_WG_PER_CU         workgroups per compute unit of the 1..8-row kernel
+    int gemv_half_units;        // BERTH_GEMV_HALF_UNITS        0: never walk half k-blocks
+    int gemv_max_rows;          // BERTH_GEMV_MAX_ROWS          rows up to this count take the VALU kernel (1..8)
+    int gemm_wg_per_cu;         // BERTH_GEMM_WG_PER_CU
+    int gemm_balanced;          // BERTH_GEMM_BALANCED
+    int gemm_rows256;           // BERTH_GEMM_ROWS256
+    int counter_stride;         // BERTH_COUNTER_STRIDE         cap on the words between arrival counters (1..32)
+    int moe_big_min;            // BERTH_MOE_BIG_MIN
+    int moe_fold_combine;       // BERTH_MOE_FOLD_COMBINE
+    int moe_inline_route;       // BERTH_MOE_INLINE_ROUTE
+    int moe_resolved;           // BERTH_MOE_RESOLVED
+    unsigned spin_limit;        // BERTH_SPIN_LIMIT             polls of a bounded wait before it gives up
+};
+const Knobs& knobs();
+void reload_knobs();
+
 // Words between the arrival counters of a one-row launch that needs `units` of them: as far
 // apart as the table allows, up to one counter per 128 bytes.  Neighbouring words send the
 // arrivals of a whole launch (hundreds within a microsecond) through one atomic unit: measured,
@@ -58,11 +85,7 @@ constexpr int kCounters = 65536;
 // follow each other.  (BERTH_COUNTER_STRIDE caps the stride; 1 packs the counters.)
 inline int counter_stride(const Workspace& ws, long units)
 {
-    static const int cap = [] {
-        const char* e = std::getenv("BERTH_COUNTER_STRIDE");
-        const int v = e ? std::atoi(e) : 32;
-        return v < 1 ? 1 : (v > 32 ? 32 : v);
-    }();
+    const int cap = knobs().counter_stride;
     int stride = 1;
     while (stride * 2 <= cap && units * stride * 2 <= (long)ws.counter_words) stride *= 2;
     return stride;
@@ -71,9 +94,7 @@ Workspace& workspace_for_current_device();
 // throws if a kernel of an earlier launch on this device reported a fault (and clears the report)
 void throw_pending_device_fault(const Workspace& ws);
 // polls a split-K finisher spends on its wait before it gives up (BERTH_SPIN_LIMIT, default 2^20)
-unsigned spin_limit();
-// fills tables[cb][s] with the fp16 weight of state s for the three codebooks (synchronous)
-void build_state_tables(uint16_t* tables);
+inline unsigned spin_limit() { return knobs().spin_limit; }
 
 struct LinearArgs {
     const void* a;
@@ -163,6 +184,7 @@ struct MgemmArgs {
     const int* had_src_list;
     int num_had_src;
     hipStream_t stream;
+    bool host_lists = false;    // the seven lists are host memory (one row, the streaming kernel only)
 };
 std::string launch_mgemm(const MgemmArgs& args);
 

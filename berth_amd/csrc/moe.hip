@@ -594,46 +594,24 @@ struct MoeLayout {
 // default: at the measured shapes 32-row problems alone are faster, because the
 // 128-row tile spends more time per k-block than four 32-row tiles running side by
 // side.
-int moe_big_min()
-{
-    static const int v = [] {
-        const char* e = std::getenv("BERTH_MOE_BIG_MIN");
-        return e ? std::atoi(e) : 0;
-    }();
-    return v;
-}
+int moe_big_min() { return knobs().moe_big_min; }
 
 // One token: the down projection's last arrival per column block also combines the block.
 // BERTH_MOE_FOLD_COMBINE: 0 keeps the separate combine launch, 1 the two-stage form (split-K
 // hand-over per expert, then a second counter per column block); otherwise, with at most
 // sixteen problems, the single hand-over (one counter per column block for both).
-int fold_combine_mode()
-{
-    static const int v = [] {
-        const char* e = std::getenv("BERTH_MOE_FOLD_COMBINE");
-        return e ? std::atoi(e) : 2;
-    }();
-    return v;
-}
+int fold_combine_mode() { return knobs().moe_fold_combine; }
 
 // One token with a small router: the routing's last part runs inside the gate / up launch
 // (BERTH_MOE_INLINE_ROUTE=0 keeps the single-workgroup routing kernel).
-bool inline_route_enabled()
-{
-    const char* e = std::getenv("BERTH_MOE_INLINE_ROUTE");
-    return !e || std::atoi(e) != 0;
-}
+bool inline_route_enabled() { return knobs().moe_inline_route != 0; }
 
 // The always-on expert runs as one more expert of the grouped launches (rows P ..
 // P + T - 1, token order) when it has the routed experts' intermediate size.
 // One token with the inline routing: the gate / up launch leaves the down projection's
 // {trellis, suh, svh} records in sorted order, and the down launch reads those instead of the
 // problem list and the expert table (BERTH_MOE_RESOLVED=0: off).
-bool resolved_records_enabled()
-{
-    const char* e = std::getenv("BERTH_MOE_RESOLVED");
-    return !e || std::atoi(e) != 0;
-}
+bool resolved_records_enabled() { return knobs().moe_resolved != 0; }
 
 bool shared_is_folded(int I, int shared_I) { return shared_I > 0 && shared_I == I; }
 

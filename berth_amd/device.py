@@ -278,6 +278,13 @@ class Exl3MultiLinear:
         self.size_n_list, self.n_stride_list, self.had_src_list = i32([width] * len(b)), i32(stride), i32(src)
         self.a_had = torch.zeros(len(sources) * self.size_k, dtype=torch.float16, device=gpu.device)
         self._c_key, self._c_ptrs = None, None
+        # the same lists on the host: one-row launches pass them by value (berth_ops_mgemm_hostlists)
+        self._h = {"b": np.array(b, dtype=np.uint64), "svh": np.array(svh, dtype=np.uint64),
+                   "suh": np.array([s.suh.data_ptr() for s in sources], dtype=np.uint64),
+                   "size_n": np.array([width] * len(b), dtype=np.int32), "stride": np.array(stride, dtype=np.int32),
+                   "src": np.array(src, dtype=np.int32)}
+        self._h_c = None
+        self.host_lists = self.slices <= 16
 
     def forward(self, gpu: Gpu, a: torch.Tensor, outs: list[torch.Tensor], out: OutDtype, rows: int = 1) -> None:
         """a fp16 [rows][K]; outs[i] [rows][N_i] of `out` for source i."""
@@ -290,7 +297,21 @@ class Exl3MultiLinear:
         if key != self._c_key:
             ptrs = [outs[s].data_ptr() + n0 * esz for s, n0 in zip(self._src, self._n0)]
             self._c_ptrs = torch.tensor(ptrs, dtype=torch.int64, device=gpu.device)
+            self._h_c = np.array(ptrs, dtype=np.uint64)
             self._c_key = key
+        if rows == 1 and self.host_lists:
+            h = self._h
+            try:
+                K.ops.exl3_mgemm_hostlists(ptr(a), h["b"].ctypes.data, ptr(outs[0]), h["suh"].ctypes.data, ptr(self.a_had),
+                                           h["svh"].ctypes.data, 1, self.size_k, self.width, self.k_bits, self.codebook,
+                                           out, 1, self.slices, h["size_n"].ctypes.data, self._h_c.ctypes.data,
+                                           h["stride"].ctypes.data, h["src"].ctypes.data, len(self.sources),
+                                           gpu.raw_stream())
+                return
+            except K.LaunchError as err:
+                if "host lists" not in str(err):
+                    raise
+                self.host_lists = False         # too small for the streaming kernel: device lists from now on
         K.ops.exl3_mgemm(ptr(a), ptr(self.b_list), ptr(outs[0]), ptr(self.suh_list), ptr(self.a_had),
                          ptr(self.svh_list), rows, self.size_k, self.width, self.k_bits, self.codebook, out,
                          1, self.slices, ptr(self.size_n_list), ptr(self._c_ptrs), ptr(self.n_stride_list),

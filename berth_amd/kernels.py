@@ -73,6 +73,7 @@ def load() -> C.CDLL:
         L.berth_exl3_mlp.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         L.berth_exl3_unpack_signs.restype = C.c_int
         L.berth_ops_mgemm.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, ci, ci, vp, vp, vp, vp, ci, vp]
+        L.berth_ops_mgemm_hostlists.argtypes = L.berth_ops_mgemm.argtypes
         for name in ("berth_exl3_last_error", "berth_exl3_last_launch", "berth_prefill_last_error",
                      "berth_prefill_last_launch", "berth_ops_last_error", "berth_ops_last_launch"):
             getattr(L, name).restype = C.c_char_p
@@ -91,6 +92,10 @@ def load() -> C.CDLL:
         L.berth_moe_last_error.restype = C.c_char_p
         L.berth_moe_last_launch.restype = C.c_char_p
         L.berth_kernels_workspace.argtypes = [C.POINTER(vp), C.POINTER(C.c_size_t), C.POINTER(vp), C.POINTER(ci)]
+        L.berth_kernels_pending_fault.restype = C.c_longlong
+        L.berth_kernels_pending_fault.argtypes = [ci]
+        L.berth_kernels_reload_env.restype = None
+        L.berth_kernels_reload_env.argtypes = []
         L.berth_device_cc.argtypes = [ci]
         L.berth_device_sms.argtypes = [ci]
         _lib = L
@@ -151,6 +156,18 @@ def last_launch() -> str:
 
 def last_error() -> str:
     return _s(load().berth_exl3_last_error())
+
+
+def reload_env() -> None:
+    """Makes the library read the BERTH_* environment knobs again (it reads them once per
+    process): call after changing os.environ inside a running process."""
+    load().berth_kernels_reload_env()
+
+
+def pending_fault(device: int = 0) -> int:
+    """0, or the code of a fault a kernel on `device` reported since the last report (cleared
+    by this call): berth_kernels_pending_fault."""
+    return int(load().berth_kernels_pending_fault(device))
 
 
 def device_cc(device: int = 0) -> int:
@@ -226,6 +243,19 @@ class ops:
         if rc > 0:
             return rc
         raise LaunchError(ops.last_error() or f"exl3_mgemm launch failed ({rc})")
+
+    @staticmethod
+    def exl3_mgemm_hostlists(a, b_list, c, suh_list, a_had, svh_list, size_m, size_k, size_n, k_bits,
+                             codebook: Codebook, out: OutDtype, bszm_in, bszm_out, size_n_list=None, c_ptrs=None,
+                             n_stride_list=None, had_src_list=None, num_had_src=0, stream=None) -> int:
+        """berth_ops_mgemm_hostlists: exl3_mgemm with the seven lists as host arrays (addresses of
+        ctypes / numpy buffers); one row, at most 16 slices, streaming-kernel sizes."""
+        rc = load().berth_ops_mgemm_hostlists(a, b_list, c, suh_list, a_had, svh_list, size_m, size_k, size_n, k_bits,
+                                              int(codebook), int(out), bszm_in, bszm_out, size_n_list, c_ptrs,
+                                              n_stride_list, had_src_list, num_had_src, stream)
+        if rc > 0:
+            return rc
+        raise LaunchError(ops.last_error() or f"exl3_mgemm (host lists) launch failed ({rc})")
 
     @staticmethod
     def rms_norm(x, weight, y, rows: int, dim: int, epsilon: float, constant_bias: float = 1.0,

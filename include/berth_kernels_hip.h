@@ -88,6 +88,21 @@ int berth_kernels_init(int device);
  * kernel on the device returns -1 with that report instead of launching. */
 int berth_kernels_workspace(void** partials, size_t* partial_bytes, void** counters, int* counter_slots);
 
+/* No counterpart in the reference.  Host-only query for the caller's synchronisation points:
+ * 0 when no kernel on `device` has reported a fault since the last report, else the fault
+ * code, and the report is cleared (-1: no such device).  A bounded wait inside a kernel that
+ * gives up stores its code in a host-visible word; launches on the device check the word too
+ * and fail with the report, but a caller that synchronises and launches nothing of this library
+ * afterwards learns of it only here.  Codes below 0x40000000: 1 + the tile an MFMA split-K
+ * finisher left unwritten; from 0x40000001: 0x40000001 + the column block a streaming GEMV
+ * finisher filled with NaN. */
+long long berth_kernels_pending_fault(int device);
+
+/* No counterpart in the reference.  The BERTH_* environment knobs are read once per process;
+ * this reads them again (for tests that switch a knob inside one process).  Not to be called
+ * while another thread is launching. */
+void berth_kernels_reload_env(void);
+
 /* crates/berth-kernels/csrc/linear.cu:301-332.  cc is the gfx target number
  * (950 on MI355X); sms is the compute-unit count. */
 int berth_device_cc(int device);
@@ -190,6 +205,19 @@ int berth_ops_mgemm(const void* a, const void* b_list, void* c, const void* suh_
                     int codebook, int c_fp32, int bszm_in, int bszm_out, const int* size_n_list,
                     const void* c_ptrs, const int* n_stride_list, const int* had_src_list,
                     int num_had_src, void* stream);
+/* No counterpart in the reference: berth_ops_mgemm with its lists in HOST memory (b_list,
+ * suh_list, svh_list and c_ptrs arrays of device addresses as uint64, the three int lists as
+ * ints; a, c and a_had stay device pointers).  For callers that built the lists themselves and
+ * still hold them: the problems then travel by value in the kernel arguments, which takes the
+ * two dependent device reads (list entry, then the source's scale pointer) out of the head of
+ * the launch (1.5 - 2.5 us of a 12 - 30 us launch).  Serves one row, at most 16 slices, and
+ * weights large enough for the one-row streaming kernel; anything else returns -1 and the
+ * caller passes device lists to berth_ops_mgemm.  Same return values and error slot. */
+int berth_ops_mgemm_hostlists(const void* a, const void* b_list, void* c, const void* suh_list, void* a_had,
+                              const void* svh_list, int size_m, int size_k, int size_n, int k_bits,
+                              int codebook, int c_fp32, int bszm_in, int bszm_out, const int* size_n_list,
+                              const void* c_ptrs, const int* n_stride_list, const int* had_src_list,
+                              int num_had_src, void* stream);
 const char* berth_ops_last_error(void);    /* ops.rs:145 */
 const char* berth_ops_last_launch(void);   /* ops.rs:146 */
 

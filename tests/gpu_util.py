@@ -1,4 +1,7 @@
 """Helpers shared by the GPU parity tests."""
+import contextlib
+import os
+
 import numpy as np
 import torch
 
@@ -28,3 +31,23 @@ def close(got, want, rtol=2e-3, atol=1e-3):
     lim = atol + rtol * np.abs(want)
     bad = err > lim
     return int(bad.sum()), float((err / lim).max())
+
+
+@contextlib.contextmanager
+def knobs(**kv):
+    """Sets BERTH_* environment knobs for the body and makes the library read them (it reads
+    the environment once per process, then only when told to)."""
+    from berth_amd import kernels as K
+    old = {k: os.environ.get(k) for k in kv}
+    for k, v in kv.items():
+        os.environ[k] = str(v)
+    K.reload_env()
+    try:
+        yield
+    finally:
+        for k, v in old.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+        K.reload_env()

@@ -15,7 +15,7 @@ from berth_amd import kernels as K
 from berth_amd import synth
 from berth_amd.kernels import Codebook, LaunchError, OutDtype
 from oracle import oracle as O
-from tests.gpu_util import DEV, close, dev
+from tests.gpu_util import DEV, close, dev, knobs
 from tests.test_gpu_runtime import Runtime
 
 pytestmark = pytest.mark.gpu
@@ -51,8 +51,7 @@ def test_finisher_gives_up_reports_and_recovers():
     bogus = np.array([1000], dtype=np.uint32)
     rt.ok(rt.copy_from_host(None, counters.value + 4 * WRITTEN_BASE, bogus.ctypes.data, 4))
 
-    os.environ["BERTH_SPIN_LIMIT"] = "300"
-    try:
+    with knobs(BERTH_SPIN_LIMIT=300):
         c.fill_(777.0)
         launch = _launch(d, c, a_had, None, rows, Kk, N)     # the launch itself is accepted and every kernel exits
         assert "exl3_gemm_kernel" in launch
@@ -60,8 +59,6 @@ def test_finisher_gives_up_reports_and_recovers():
         with pytest.raises(LaunchError, match="gave up waiting for the split-K partial sums of tile 0"):
             _launch(d, c, a_had, None, rows, Kk, N)
         assert K.prefill_lin.last_launch() == ""
-    finally:
-        del os.environ["BERTH_SPIN_LIMIT"]
     both = np.zeros(2, dtype=np.uint32)
     rt.ok(rt.copy_to_host(None, both[:1].ctypes.data, counters.value, 4))
     rt.ok(rt.copy_to_host(None, both[1:].ctypes.data, counters.value + 4 * WRITTEN_BASE, 4))

@@ -10,7 +10,7 @@ from berth_amd import synth
 from berth_amd.device import Exl3Linear, Gpu
 from berth_amd.moe import MoeLayer
 from oracle import oracle as O
-from tests.gpu_util import DEV, close, dev
+from tests.gpu_util import DEV, close, dev, knobs
 
 pytestmark = pytest.mark.gpu
 
@@ -351,8 +351,7 @@ def test_moe_one_token_inline_routing_equals_the_routing_kernel():
         d_x = dev(x.view(np.uint16))
         res = {}
         for mode, env in (("1", {}), ("unresolved", {"BERTH_MOE_RESOLVED": "0"}), ("0", {"BERTH_MOE_INLINE_ROUTE": "0"})):
-            os.environ.update(env)
-            try:
+            with knobs(**env):
                 out = torch.zeros((1, H), dtype=torch.float32, device=DEV)
                 idx = torch.full((1, k), -1, dtype=torch.int32, device=DEV)
                 w = torch.zeros((1, k), dtype=torch.float32, device=DEV)
@@ -360,9 +359,6 @@ def test_moe_one_token_inline_routing_equals_the_routing_kernel():
                 torch.cuda.synchronize()
                 res[mode] = (out.cpu().numpy().view(np.uint32), idx.cpu().numpy(), w.cpu().numpy().view(np.uint32),
                              K.moe.last_launch())
-            finally:
-                for name in env:
-                    del os.environ[name]
         # the down launch takes its linears from the records the gate / up launch left, unless told not to
         assert "moe_route_segments_kernel" in res["1"][3] and "+route" in res["1"][3] and "resolved" in res["1"][3], res["1"][3]
         assert "+route" in res["unresolved"][3] and "resolved" not in res["unresolved"][3], res["unresolved"][3]

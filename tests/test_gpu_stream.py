@@ -21,24 +21,9 @@ from berth_amd import kernels as K
 from berth_amd import synth
 from berth_amd.kernels import Codebook, OutDtype
 from oracle import oracle as O
-from tests.gpu_util import DEV, close, dev, host_f16, host_u16
+from tests.gpu_util import DEV, close, dev, host_f16, host_u16, knobs
 
 pytestmark = pytest.mark.gpu
-
-
-@contextlib.contextmanager
-def knobs(**kv):
-    old = {k: os.environ.get(k) for k in kv}
-    for k, v in kv.items():
-        os.environ[k] = str(v)
-    try:
-        yield
-    finally:
-        for k, v in old.items():
-            if v is None:
-                os.environ.pop(k, None)
-            else:
-                os.environ[k] = v
 
 
 def forced(wgs=0, lut="0xA", min_units=2):

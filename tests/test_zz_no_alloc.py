@@ -10,7 +10,7 @@ from berth_amd import kernels as K
 from berth_amd import synth
 from berth_amd.kernels import Codebook, OutDtype
 from oracle import oracle as O
-from tests.gpu_util import DEV, close, dev, host_u16
+from tests.gpu_util import DEV, close, dev, host_u16, knobs
 
 pytestmark = pytest.mark.gpu
 
@@ -65,11 +65,7 @@ def test_no_alloc_refuses_what_does_not_fit():
     # With the default split (about six workgroups per compute unit) the partial sums of a launch
     # stay under 6.3 MB on 256 compute units; a finer split of eight rows of a wide, deep weight
     # exceeds the 8 MiB and is refused before anything is launched (the pointers are never used).
-    import os
-    os.environ["BERTH_GEMV_WG_PER_CU"] = "16"
-    try:
+    with knobs(BERTH_GEMV_WG_PER_CU=16):
         with pytest.raises(K.LaunchError, match="bytes of split-K scratch"):
             K.exl3_linear_noalloc(bad, bad, bad, bad, bad, bad, 8, 16384, 16384, 2, Codebook.MUL1, OutDtype.F32)
-    finally:
-        del os.environ["BERTH_GEMV_WG_PER_CU"]
     assert K.last_launch() == ""
