@@ -26,8 +26,6 @@ LIBRARIES = {
                                 "exl3_gemm_cb2.hip",
                                 "exl3_reconstruct.hip", "elementwise.hip", "moe.hip"],
     "libberth_hip.so": ["berth_hip.hip"],
-    # measurement probe used by bench.py only
-    "libberth_probe.so": ["probe/valu_rate.hip"],
 }
 
 
@@ -61,15 +59,30 @@ def build_all(jobs: int = 8, only: str | None = None) -> list[str]:
         built.append(build_code_object())
         built.append(build_reader())
         built.append(build_host_check())
+        built.append(build_bench_native())
     return built
+
+
+def build_bench_native() -> str:
+    """bench.py's native helpers (bench_native.hip at the repository root: the vector-ALU rate
+    probe and the eager launch loop over the C ABI), linked against the kernels library."""
+    root = os.path.dirname(HERE)
+    out = os.path.join(root, "libberth_bench.so")
+    cmd = [HIPCC, *FLAGS, "-shared", "-I" + root, os.path.join(root, "bench_native.hip"), "-o", out,
+           "-L" + LIB, "-lberth_kernels_hip", "-Wl,-rpath,$ORIGIN/berth_amd/lib"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"bench helper build failed:\n{r.stderr[-4000:]}")
+    return out
 
 
 def build_code_object() -> str:
     """A stand-alone gfx950 code object (hipcc --genco) with the test kernels the runtime
-    library's module path is exercised with (tests/test_gpu_runtime.py)."""
-    out = os.path.join(LIB, "runtime_probe.hsaco")
+    library's module path is exercised with (tests/runtime_probe.hip, tests/test_gpu_runtime.py)."""
+    tests = os.path.join(os.path.dirname(HERE), "tests")
+    out = os.path.join(tests, "runtime_probe.hsaco")
     cmd = [HIPCC, "--genco", "--offload-arch=gfx950", "-O3", "-ffp-contract=off",
-           os.path.join(CSRC, "probe", "runtime_probe.hip"), "-o", out]
+           os.path.join(tests, "runtime_probe.hip"), "-o", out]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"code object build failed:\n{r.stderr[-4000:]}")

@@ -13,7 +13,7 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-CODE_OBJECT = os.path.join(ROOT, "berth_amd", "lib", "runtime_probe.hsaco")
+CODE_OBJECT = os.path.join(ROOT, "tests", "runtime_probe.hsaco")
 
 
 class Runtime:
