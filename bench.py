@@ -200,6 +200,32 @@ class NativeCalls:
             call.i[j] = v
         self._calls.append(call)
 
+    def mlp(self, layer, x, y):
+        """berth_exl3_mlp on one row (MlpLayer's buffers)."""
+        import ctypes
+        from berth_amd.device import ptr
+        from berth_amd.kernels import Exl3Lin
+        layer.forward(self.gpu, x, y, fused=True)           # allocates the layer's rotated-input buffers
+        lins = (Exl3Lin * 3)(*[Exl3Lin(ptr(l.trellis), ptr(l.suh), ptr(l.svh)) for l in (layer.gate, layer.up, layer.down)])
+        self._keep.append(lins)
+        call = self._type()
+        call.kind = 3
+        for j, v in enumerate((ptr(x), ctypes.addressof(lins), ptr(layer.g), ptr(layer.u), ptr(layer.x_had),
+                               ptr(layer.act_had), ptr(y))):
+            call.p[j] = v
+        for j, v in enumerate((1, layer.hidden, layer.intermediate, layer.gate.k_bits, int(layer.gate.codebook))):
+            call.i[j] = v
+        self._calls.append(call)
+
+    def silu_mul(self, gate, up, out, numel: int):
+        from berth_amd.device import ptr
+        call = self._type()
+        call.kind = 4
+        for j, v in enumerate((ptr(gate), ptr(up), ptr(out))):
+            call.p[j] = v
+        call.i[0] = numel
+        self._calls.append(call)
+
     def run(self, steps: int):
         import ctypes
         if self._array is None:
@@ -555,18 +581,30 @@ def mlp_block_bench(gpu, layers, bits: int, steps: int):
     x = gpu.upload((synth.activations(11, 1, H).astype(np.float32) / np.sqrt(H)).astype(np.float16).view(np.uint16))
     y = torch.zeros(H, dtype=torch.float32, device=gpu.device)
     nbytes = 2 * linear_bytes(H, I, bits, 1, 2) + linear_bytes(I, H, bits, 1, 4)
-    res = {"config": f"hidden {H}, intermediate {I}, {bits} bpw, mul1, batch 1", "bytes": nbytes}
+    res = {"config": f"hidden {H}, intermediate {I}, {bits} bpw, mul1, batch 1", "bytes": nbytes,
+           "launch": "eager, issued by the compiled host loop"}
     for name, fused in (("one_call", True), ("four_calls", False)):
-        for i in range(len(mlps)):
-            mlps[i].forward(gpu, x, y, fused=fused)
+        calls = NativeCalls(gpu, 1 if fused else 4)
+        for m in mlps:
+            if fused:
+                calls.mlp(m, x, y)
+            else:
+                calls.linear(m.gate, x, m.g, False)
+                calls.linear(m.up, x, m.u, False)
+                calls.silu_mul(m.g, m.u, m.u, I)
+                calls.linear(m.down, m.u, y, True)
+        calls.run(len(mlps))
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for i in range(steps):
-            mlps[i % len(mlps)].forward(gpu, x, y, fused=fused)
-        e1.record()
-        torch.cuda.synchronize()
-        dt = e0.elapsed_time(e1) * 1e-3 / steps
+        best = None
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            calls.run(steps)
+            e1.record()
+            torch.cuda.synchronize()
+            dt = e0.elapsed_time(e1) * 1e-3 / steps
+            best = dt if best is None else min(best, dt)
+        dt = best
         res[name] = {"us_per_block": round(dt * 1e6, 2), "GBps": round(nbytes / dt / 1e9, 1),
                      "frac_of_hbm_peak": round(nbytes / dt / 1e9 / HBM_PEAK_GBS, 4)}
     return res

@@ -98,7 +98,8 @@ extern "C" int berth_probe_valu(double sustain_ms, double* out)
 
 // One prepared call of the C ABI.  kind 0: berth_exl3_linear(p[0..5], i[0..5], stream);
 // kind 1: berth_ops_mgemm_hostlists, kind 2: berth_ops_mgemm (p[0..5], i[0..7], p[6..9], i[8], stream);
-// kind 3: berth_exl3_mlp(p[0], lins = p[1] (host), p[2..6], i[0..4], stream).
+// kind 3: berth_exl3_mlp(p[0], lins = p[1] (host), p[2..6], i[0..4], stream);
+// kind 4: berth_ops_silu_mul(p[0..2], numel = i[0], act_limit 0, stream).
 struct BenchCall {
     int kind;
     int i[12];
@@ -133,6 +134,7 @@ extern "C" int berth_bench_run(const BenchCall* calls, int per_step, int distinc
                 rc = berth_exl3_mlp(c.p[0], (const berth_exl3_lin*)c.p[1], (void*)c.p[2], (void*)c.p[3], (void*)c.p[4],
                                     (void*)c.p[5], (void*)c.p[6], c.i[0], c.i[1], c.i[2], c.i[3], c.i[4], stream);
                 break;
+            case 4: rc = berth_ops_silu_mul(c.p[0], c.p[1], (void*)c.p[2], (int64_t)c.i[0], 0.0f, stream); break;
             default: break;
             }
             if (rc != 0) return 1 + s * per_step + j;
