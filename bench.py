@@ -217,6 +217,34 @@ class NativeCalls:
             call.i[j] = v
         self._calls.append(call)
 
+    def mlp_block(self, layer, x32, res, res_out, norm_w, y):
+        """berth_exl3_mlp_block on one row (epsilon 1e-6, bias 1, scale 1, bf16 norm weight)."""
+        import ctypes
+        from berth_amd.device import ptr
+        from berth_amd.kernels import Exl3Lin, RmsNorm
+        layer.forward_block(self.gpu, x32, res, res_out, norm_w, y)      # allocates the layer's scratch
+        lins = (Exl3Lin * 3)(*[Exl3Lin(ptr(l.trellis), ptr(l.suh), ptr(l.svh)) for l in (layer.gate, layer.up, layer.down)])
+        norm = RmsNorm(ptr(norm_w), 1e-6, 1.0, 1.0, 1)
+        self._keep += [lins, norm]
+        call = self._type()
+        call.kind = 5
+        for j, v in enumerate((ptr(x32), ptr(res), ptr(res_out), ctypes.addressof(norm), ctypes.addressof(lins),
+                               ptr(layer.h_norm), ptr(layer.g), ptr(layer.u), ptr(layer.x_had), ptr(layer.act_had), ptr(y))):
+            call.p[j] = v
+        for j, v in enumerate((1, layer.hidden, layer.intermediate, layer.gate.k_bits, int(layer.gate.codebook))):
+            call.i[j] = v
+        self._calls.append(call)
+
+    def raw(self, kind: int, pointers, ints):
+        from berth_amd.device import ptr
+        call = self._type()
+        call.kind = kind
+        for j, t in enumerate(pointers):
+            call.p[j] = ptr(t)
+        for j, v in enumerate(ints):
+            call.i[j] = v
+        self._calls.append(call)
+
     def silu_mul(self, gate, up, out, numel: int):
         from berth_amd.device import ptr
         call = self._type()
@@ -583,10 +611,23 @@ def mlp_block_bench(gpu, layers, bits: int, steps: int):
     nbytes = 2 * linear_bytes(H, I, bits, 1, 2) + linear_bytes(I, H, bits, 1, 4)
     res = {"config": f"hidden {H}, intermediate {I}, {bits} bpw, mul1, batch 1", "bytes": nbytes,
            "launch": "eager, issued by the compiled host loop"}
-    for name, fused in (("one_call", True), ("four_calls", False)):
-        calls = NativeCalls(gpu, 1 if fused else 4)
+    # the block with the glue either side of it: residual add + RMS norm ahead, residual add behind
+    x32 = torch.randn(H, device=gpu.device, dtype=torch.float32)
+    resid = torch.randn(H, device=gpu.device, dtype=torch.float32)
+    res_out = torch.zeros_like(resid)
+    h16 = torch.zeros(H, dtype=torch.float16, device=gpu.device)
+    norm_w = torch.zeros(H, dtype=torch.int16, device=gpu.device)          # bf16 zeros: weight + 1 = 1
+    for name, fused in (("one_call", True), ("four_calls", False), ("block_one_call", "block"),
+                        ("block_norm_mlp_add_calls", "glue")):
+        calls = NativeCalls(gpu, {True: 1, False: 4, "block": 1, "glue": 3}[fused])
         for m in mlps:
-            if fused:
+            if fused == "block":
+                calls.mlp_block(m, x32, resid, res_out, norm_w, y)
+            elif fused == "glue":
+                calls.raw(6, (x32, norm_w, h16, res_out), (1, H))           # rms_norm_res_in (in place on res_out)
+                calls.mlp(m, h16, y)
+                calls.raw(7, (y, res_out, y), (H,))                         # add_f32
+            elif fused:
                 calls.mlp(m, x, y)
             else:
                 calls.linear(m.gate, x, m.g, False)

@@ -99,7 +99,10 @@ extern "C" int berth_probe_valu(double sustain_ms, double* out)
 // One prepared call of the C ABI.  kind 0: berth_exl3_linear(p[0..5], i[0..5], stream);
 // kind 1: berth_ops_mgemm_hostlists, kind 2: berth_ops_mgemm (p[0..5], i[0..7], p[6..9], i[8], stream);
 // kind 3: berth_exl3_mlp(p[0], lins = p[1] (host), p[2..6], i[0..4], stream);
-// kind 4: berth_ops_silu_mul(p[0..2], numel = i[0], act_limit 0, stream).
+// kind 4: berth_ops_silu_mul(p[0..2], numel = i[0], act_limit 0, stream);
+// kind 5: berth_exl3_mlp_block(p[0..2], norm = p[3] (host), lins = p[4] (host), p[5..10], i[0..4], stream);
+// kind 6: berth_ops_rms_norm_res_in(p[0..3], rows = i[0], dim = i[1], epsilon 1e-6, bias 1, scale 1, bf16 weight, stream);
+// kind 7: berth_ops_add_f32(p[0..2], n = i[0], stream).
 struct BenchCall {
     int kind;
     int i[12];
@@ -135,6 +138,17 @@ extern "C" int berth_bench_run(const BenchCall* calls, int per_step, int distinc
                                     (void*)c.p[5], (void*)c.p[6], c.i[0], c.i[1], c.i[2], c.i[3], c.i[4], stream);
                 break;
             case 4: rc = berth_ops_silu_mul(c.p[0], c.p[1], (void*)c.p[2], (int64_t)c.i[0], 0.0f, stream); break;
+            case 5:
+                rc = berth_exl3_mlp_block(c.p[0], c.p[1], (void*)c.p[2], (const berth_rms_norm*)c.p[3],
+                                          (const berth_exl3_lin*)c.p[4], (void*)c.p[5], (void*)c.p[6], (void*)c.p[7],
+                                          (void*)c.p[8], (void*)c.p[9], (void*)c.p[10], c.i[0], c.i[1], c.i[2], c.i[3],
+                                          c.i[4], stream);
+                break;
+            case 6:
+                rc = berth_ops_rms_norm_res_in(c.p[0], c.p[1], (void*)c.p[2], (void*)c.p[3], c.i[0], c.i[1], 1e-6f, 1.0f, 1.0f,
+                                               1, stream);
+                break;
+            case 7: rc = berth_ops_add_f32(c.p[0], c.p[1], (void*)c.p[2], c.i[0], stream); break;
             default: break;
             }
             if (rc != 0) return 1 + s * per_step + j;

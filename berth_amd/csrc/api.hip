@@ -535,6 +535,82 @@ extern "C" int berth_exl3_mlp(const void* x, const berth_exl3_lin* lins, void* g
     }
 }
 
+// The FFN block of a decoder layer around berth_exl3_mlp: the residual add and RMS norm ahead
+// of it (crates/berth-kernels/src/ops.rs:430-500, rms_norm_res_in) and the residual add behind
+// it (ops.rs:522-552, add_f32), as crates/berth-engine/src/mlp.rs:118-150 is called from the
+// block.  One row whose linears take the streaming kernel: two launches, the norm formed while
+// the gate / up launch rotates its input, the sum added where the down launch writes its output.
+extern "C" int berth_exl3_mlp_block(const void* x, const void* residual, void* residual_out, const berth_rms_norm* norm,
+                                    const berth_exl3_lin* lins, void* h_norm, void* gate_out, void* up_out, void* a_had,
+                                    void* act_had, void* y, int size_m, int hidden, int intermediate, int k_bits,
+                                    int codebook, void* stream)
+{
+    try {
+        g_exl3_err.clear();
+        g_exl3_launch.clear();
+        if (!x || !residual || !residual_out || !norm || !norm->weight || !lins || !h_norm || !gate_out || !up_out ||
+            !a_had || !act_had || !y)
+            throw std::runtime_error("exl3 mlp block: null device pointer");
+        for (int i = 0; i < 3; ++i)
+            if (!lins[i].trellis || !lins[i].suh || !lins[i].svh) throw std::runtime_error("exl3 mlp block: null device pointer");
+        if (size_m < 1 || hidden < 1 || intermediate < 1) throw std::runtime_error("exl3 mlp block: sizes must be positive");
+        if (residual_out == residual || residual_out == x)
+            throw std::runtime_error("exl3 mlp block: residual_out must not alias residual or x");
+        if (norm->weight_bf16 != 0 && norm->weight_bf16 != 1)
+            throw std::runtime_error("exl3 mlp block: weight_bf16 must be 0 or 1");
+        hipStream_t st = (hipStream_t)stream;
+        LinearArgs down{up_out, lins[2].trellis, y, lins[2].suh, act_had, lins[2].svh, size_m, intermediate, hidden,
+                        k_bits, codebook, 1, st};
+        LinearArgs gate{x, lins[0].trellis, gate_out, lins[0].suh, a_had, lins[0].svh, size_m, hidden, intermediate,
+                        k_bits, codebook, 0, st};
+        check_shape("exl3 mlp block", gate);
+        check_shape("exl3 mlp block", down);
+        const int n = size_m * hidden;
+        const bool fuse_norm = size_m == 1 && gemv_stream_applies(2, hidden, intermediate, false);
+        const bool fuse_add = size_m == 1 && gemv_stream_applies(1, intermediate, hidden, false);
+        std::string desc;
+        if (fuse_norm) {
+            const NormInput ni{(const float*)x, (const float*)residual, (float*)residual_out, norm->weight, norm->epsilon,
+                               norm->constant_bias, norm->constant_scale, norm->weight_bf16};
+            PairArgs pair{nullptr, {lins[0].trellis, lins[1].trellis}, {lins[0].suh, lins[1].suh},
+                          {lins[0].svh, lins[1].svh}, {gate_out, up_out}, a_had, 1, hidden, intermediate, k_bits, codebook, st};
+            pair.norm = &ni;
+            desc = launch_gemv_pair(pair);
+        } else {
+            // the same arithmetic as separate launches
+            desc = launch_add_f32(residual, x, residual_out, n, st);
+            desc += " ; " + launch_rms_norm(residual_out, norm->weight, h_norm, nullptr, size_m, hidden, norm->epsilon,
+                                            norm->constant_bias, norm->constant_scale, norm->weight_bf16, st);
+        }
+        if (size_m <= 8) {
+            if (!fuse_norm) {
+                PairArgs pair{h_norm, {lins[0].trellis, lins[1].trellis}, {lins[0].suh, lins[1].suh},
+                              {lins[0].svh, lins[1].svh}, {gate_out, up_out}, a_had, size_m, hidden, intermediate, k_bits,
+                              codebook, st};
+                desc += " ; " + launch_gemv_pair(pair);
+            }
+            down.a = gate_out;
+            down.a_up = up_out;
+            if (fuse_add) down.out_add = (const float*)residual_out;
+            desc += " ; " + launch_gemv(down) + (fuse_add ? " +residual" : "");
+        } else {
+            if (berth_exl3_mlp(h_norm, lins, gate_out, up_out, a_had, act_had, y, size_m, hidden, intermediate, k_bits,
+                               codebook, stream) != 0)
+                throw std::runtime_error(g_exl3_err);
+            desc += " ; " + g_exl3_launch;
+        }
+        if (!fuse_add) desc += " ; " + launch_add_f32(y, residual_out, y, n, st);
+        g_exl3_launch = desc;
+        return 0;
+    } catch (const std::exception& err) {
+        const std::string what = err.what();
+        g_exl3_err = what;
+        g_exl3_launch.clear();
+        (void)hipGetLastError();
+        return -1;
+    }
+}
+
 extern "C" int berth_exl3_unpack_signs(const void* packed, void* out, int64_t packed_bytes, void* stream)
 {
     try {

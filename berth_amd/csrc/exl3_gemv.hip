@@ -110,6 +110,14 @@ static StreamPlan plan_stream(const Workspace& ws, int problems, int K, int N)
     return pl;
 }
 
+bool gemv_stream_applies(int problems, int size_k, int size_n, bool whole_rows)
+{
+    if (size_k % 128 != 0 || size_n % 128 != 0) return false;
+    const StreamPlan pl = plan_stream(workspace_for_current_device(), problems, size_k, size_n);
+    if (!pl.ok) return false;
+    return !whole_rows || (unsigned)kStreamWaves * pl.q >= (unsigned)size_k / 16;
+}
+
 static std::string run_stream(const Workspace& ws, const StreamPlan& pl, StreamParams& p, int bits, int cb,
                               hipStream_t stream)
 {
@@ -209,9 +217,14 @@ std::string launch_gemv(const LinearArgs& a, const Workspace* scratch)
             sp.K = a.size_k;
             sp.N = a.size_n;
             sp.out_fp32 = a.out_fp32;
+            if (a.out_add) {
+                if (!a.out_fp32) throw std::runtime_error("exl3 gemv: a row is added to an fp32 output only");
+                sp.out_add = a.out_add;
+            }
             return run_stream(ws, pl, sp, a.k_bits, a.codebook, a.stream);
         }
     }
+    if (a.out_add) throw std::runtime_error("exl3 gemv: the added output row needs the one-row streaming kernel");
 
     GemvParams p{};
     p.a = (const _Float16*)a.a;
@@ -259,9 +272,20 @@ std::string launch_gemv_pair(const PairArgs& a)
             sp.K = a.size_k;
             sp.N = a.size_n;
             sp.out_fp32 = 0;
-            return "pair " + run_stream(ws, pl, sp, a.k_bits, a.codebook, a.stream);
+            if (a.norm) {
+                sp.norm_x = a.norm->x;
+                sp.norm_res = a.norm->res;
+                sp.norm_res_out = a.norm->res_out;
+                sp.norm_weight = (const uint16_t*)a.norm->weight;
+                sp.norm_eps = a.norm->epsilon;
+                sp.norm_bias = a.norm->constant_bias;
+                sp.norm_scale = a.norm->constant_scale;
+                sp.norm_weight_bf16 = a.norm->weight_bf16;
+            }
+            return std::string(a.norm ? "pair,norm " : "pair ") + run_stream(ws, pl, sp, a.k_bits, a.codebook, a.stream);
         }
     }
+    if (a.norm) throw std::runtime_error("exl3 gemv: the norm input needs the one-row streaming kernel");
     GemvParams p{};
     p.a = (const _Float16*)a.a;
     p.pair = 1;
@@ -302,7 +326,7 @@ std::string launch_mgemm(const MgemmArgs& m)
     const int mmax = m.size_m == 1 ? 1 : 8;
     if (m.host_lists) {
         // the lists are host memory: the problems travel by value in the kernel arguments
-        const StreamPlan pl = m.size_m == 1 && m.bszm_out <= kStreamMaxSlices
+        const StreamPlan pl = m.size_m == 1 && m.bszm_out <= kStreamMaxSlices && m.size_n / 128 <= 65535
                                   ? plan_stream(ws, m.bszm_out, m.size_k, m.size_n) : StreamPlan{};
         if (!pl.ok)
             throw std::runtime_error("exl3_mgemm (host lists): serves one row, at most " + std::to_string(kStreamMaxSlices) +
@@ -330,15 +354,15 @@ std::string launch_mgemm(const MgemmArgs& m)
                     throw std::runtime_error("exl3_mgemm (host lists): size_n_list entry must be a multiple of 128 within size_n");
                 sl.suh = (const _Float16*)su[src];
                 sl.c = (void*)((const uint64_t*)m.c_ptrs)[i];
-                sl.width = m.size_n_list[i];
+                sl.width128 = (uint16_t)(m.size_n_list[i] / 128);
                 sl.n_stride = m.n_stride_list[i];
-                sl.had_slab = src;
+                sl.had_slab = (uint16_t)src;
             } else {
                 sl.suh = (const _Float16*)su[i];
                 sl.c = (char*)m.c + (size_t)i * m.size_n * (m.c_fp32 ? 4 : 2);
-                sl.width = m.size_n;
+                sl.width128 = (uint16_t)(m.size_n / 128);
                 sl.n_stride = m.size_n;
-                sl.had_slab = i;
+                sl.had_slab = (uint16_t)i;
             }
         }
         return std::string(sliced ? "sliced x" : "uniform x") + std::to_string(m.bszm_out) + " by value " +

@@ -6,35 +6,35 @@
 
 namespace berth {
 
-template <int BITS, int CB, bool SILU, int LUTMASK>
+template <int BITS, int CB, int IN, int LUTMASK>
 static void launch_stream_one(const StreamParams& p, dim3 grid, hipStream_t stream)
 {
     constexpr int lds_bytes = stream_lds_bytes(LUTMASK);
     static bool raised[64] = {};
-    raise_dynamic_lds_limit((const void*)exl3_gemv_stream_kernel<BITS, CB, SILU, LUTMASK>, lds_bytes, raised,
+    raise_dynamic_lds_limit((const void*)exl3_gemv_stream_kernel<BITS, CB, IN, LUTMASK>, lds_bytes, raised,
                             "exl3_gemv_stream_kernel: dynamic LDS limit");
-    hipLaunchKernelGGL((exl3_gemv_stream_kernel<BITS, CB, SILU, LUTMASK>), grid, dim3(1024), lds_bytes, stream, p);
+    hipLaunchKernelGGL((exl3_gemv_stream_kernel<BITS, CB, IN, LUTMASK>), grid, dim3(1024), lds_bytes, stream, p);
 }
 
 template <int BITS, int CB>
 static void launch_stream_bits(const StreamParams& p, int lutmask, dim3 grid, hipStream_t stream)
 {
-    const bool silu = p.a_up != nullptr;
+    const int in = p.norm_x ? kInNorm : (p.a_up ? kInSilu : kInPlain);
+    auto by_input = [&](auto mask) {
+        constexpr int M = decltype(mask)::value;
+        if (in == kInNorm) launch_stream_one<BITS, CB, kInNorm, M>(p, grid, stream);
+        else if (in == kInSilu) launch_stream_one<BITS, CB, kInSilu, M>(p, grid, stream);
+        else launch_stream_one<BITS, CB, kInPlain, M>(p, grid, stream);
+    };
     switch (lutmask) {
-    case 0x0:
-        if (silu) launch_stream_one<BITS, CB, true, 0x0>(p, grid, stream);
-        else launch_stream_one<BITS, CB, false, 0x0>(p, grid, stream);
-        break;
+    case 0x0: by_input(std::integral_constant<int, 0x0>{}); break;
 #ifdef BERTH_STREAM_EXTRA_MASKS
-    case 0x2: launch_stream_one<BITS, CB, false, 0x2>(p, grid, stream); break;
-    case 0x8: launch_stream_one<BITS, CB, false, 0x8>(p, grid, stream); break;
-    case 0xE: launch_stream_one<BITS, CB, false, 0xE>(p, grid, stream); break;
-    case 0xF: launch_stream_one<BITS, CB, false, 0xF>(p, grid, stream); break;
+    case 0x2: launch_stream_one<BITS, CB, kInPlain, 0x2>(p, grid, stream); break;
+    case 0x8: launch_stream_one<BITS, CB, kInPlain, 0x8>(p, grid, stream); break;
+    case 0xE: launch_stream_one<BITS, CB, kInPlain, 0xE>(p, grid, stream); break;
+    case 0xF: launch_stream_one<BITS, CB, kInPlain, 0xF>(p, grid, stream); break;
 #endif
-    default:
-        if (silu) launch_stream_one<BITS, CB, true, 0xA>(p, grid, stream);
-        else launch_stream_one<BITS, CB, false, 0xA>(p, grid, stream);
-        break;
+    default: by_input(std::integral_constant<int, 0xA>{}); break;
     }
 }
 

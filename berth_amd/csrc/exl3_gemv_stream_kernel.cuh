@@ -51,7 +51,7 @@ constexpr int kStreamPieces = kStreamWaves + kStreamMaxCb - 1;
 // dynamic LDS of a launch: [table 128 KiB, if any][rotated activation][partial pieces][piece bounds]
 __host__ __device__ constexpr int stream_lds_bytes(int lutmask)
 {
-    return (lutmask ? 131072 : 0) + kStreamXsBlocks * 256 + kStreamPieces * 512 + 128;
+    return (lutmask ? 131072 : 0) + kStreamXsBlocks * 256 + kStreamPieces * 512 + 128 + 128;
 }
 
 // one problem of a bundle whose lists the host knows (mode 3)
@@ -60,7 +60,9 @@ struct StreamSlice {
     const _Float16* suh;
     const _Float16* svh;
     void* c;
-    int width, n_stride, had_slab, pad;
+    int n_stride;
+    uint16_t width128;          // columns / 128
+    uint16_t had_slab;
 };
 constexpr int kStreamMaxSlices = 16;
 
@@ -89,6 +91,15 @@ struct StreamParams {
     unsigned long long* accum;  // [problem][column block][128] fixed-point sums, zero between launches
     unsigned* fault;            // host-visible word for a finisher that gives up its bounded wait
     unsigned spin_limit;
+    // IN == kInNorm: the input row is rms(norm_res + norm_x) * (weight + bias) * scale, rounded to
+    // fp16, with norm_x and norm_res fp32 [K]; their sum also goes to norm_res_out (not an alias)
+    const float* norm_x;
+    const float* norm_res;
+    float* norm_res_out;
+    const uint16_t* norm_weight;
+    float norm_eps, norm_bias, norm_scale;
+    int norm_weight_bf16;
+    const float* out_add;       // optional fp32 [N] (one problem, fp32 output): added to the output row
     StreamSlice slice[kStreamMaxSlices];    // mode 3: the problems, by value
 };
 
@@ -252,9 +263,15 @@ __device__ __forceinline__ global_ptr<T> uniform_ptr(global_ptr<T> q)
     return (global_ptr<T>)(((uint64_t)hi << 32) | lo);
 }
 
-template <int BITS, int CB, bool SILU, int LUTMASK>
+// What the input row is: the fp16 row as given; silu(a) * a_up (the gated activation of an MLP's
+// down projection, formed with the fp16 steps of berth_ops_silu_mul); or the RMS norm of a
+// fp32 row with the residual added first (the steps of berth_ops_rms_norm_res_in).
+constexpr int kInPlain = 0, kInSilu = 1, kInNorm = 2;
+
+template <int BITS, int CB, int IN, int LUTMASK>
 __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams p)
 {
+    constexpr bool SILU = IN == kInSilu, NORM = IN == kInNorm;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     constexpr int kLutBytes = LUTMASK ? 131072 : 0;       // the table sits at LDS offset 0
     constexpr int kXsOff = kLutBytes;
@@ -265,8 +282,9 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
     float* const red = (float*)(lds + kRedOff);
     unsigned* const piece_first = (unsigned*)(lds + kMetaOff);
     unsigned* const piece_last = piece_first + 16;
+    double* const norm_part = (double*)(lds + kMetaOff + 128);         // NORM: one sum of squares per wave
 
-    static_assert(sizeof(StreamParams) > 15 * 64 && sizeof(StreamParams) <= 16 * 64, "argument lines touched below");
+    static_assert(sizeof(StreamParams) > 10 * 64 && sizeof(StreamParams) <= 16 * 64, "argument lines touched below");
     touch_kernel_arguments<16>();
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -283,9 +301,9 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
         lin.suh = sl.suh;
         lin.svh = sl.svh;
         cout = sl.c;
-        width = sl.width;
+        width = (int)sl.width128 * 128;
         n_stride = sl.n_stride;
-        had_slab = sl.had_slab;
+        had_slab = (int)sl.had_slab;
     } else if (p.mode) {
         lin.trellis = (const uint32_t*)p.b_list[prob];
         lin.svh = (const _Float16*)p.svh_list[prob];
@@ -330,6 +348,8 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
     const global_ptr<const half2_t> uin = (global_ptr<const half2_t>)as_global(p.a_up + (size_t)prob * p.in_stride);
     const global_ptr<const half2_t> sin = (global_ptr<const half2_t>)as_global(lin.suh);
     half2_t rot_x[kRot], rot_s[kRot], rot_u[kRot];
+    float2_t nrm_v[NORM ? kRot : 1];
+    uint32_t nrm_w[NORM ? kRot : 1];
     unsigned rot_kb[kRot];
 #pragma unroll
     for (int t = 0; t < kRot; ++t) {
@@ -337,7 +357,14 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
         unsigned kb = a_lo + (i < nk ? i : 0u);                         // past the end: any valid k-block, unused
         kb = kb >= KB ? kb - KB : kb;
         rot_kb[t] = kb;
-        rot_x[t] = xin[kb * 64 + lane];
+        if constexpr (NORM) {
+            const float2_t xv = ((global_ptr<const float2_t>)as_global(p.norm_x))[kb * 64 + lane];
+            const float2_t rv = ((global_ptr<const float2_t>)as_global(p.norm_res))[kb * 64 + lane];
+            nrm_w[t] = ((global_ptr<const uint32_t>)as_global((const uint32_t*)p.norm_weight))[kb * 64 + lane];
+            nrm_v[t] = float2_t{rv.x + xv.x, rv.y + xv.y};
+        } else {
+            rot_x[t] = xin[kb * 64 + lane];
+        }
         rot_s[t] = sin[kb * 64 + lane];
         if (SILU) rot_u[t] = uin[kb * 64 + lane];
     }
@@ -380,8 +407,11 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
     const unsigned cb_last = div_magic(u1 - 1, p.mtr);
     const unsigned ncb = cb_last - cb_first + 1;
     half2_t sv_mine = {};
-    if ((unsigned)wave < ncb && (cb_first + (unsigned)wave) * 128u < (unsigned)width)
+    float2_t add_mine = {0.0f, 0.0f};
+    if ((unsigned)wave < ncb && (cb_first + (unsigned)wave) * 128u < (unsigned)width) {
         sv_mine = ((global_ptr<const half2_t>)as_global(lin.svh + (cb_first + (unsigned)wave) * 128))[lane];
+        if (p.out_add) add_mine = ((global_ptr<const float2_t>)as_global(p.out_add + (cb_first + (unsigned)wave) * 128))[lane];
+    }
     if (threadIdx.x < 16) {
         piece_first[threadIdx.x] = 0xffffffffu;
         piece_last[threadIdx.x] = 0u;
@@ -397,6 +427,44 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
         for (int j = 0; j < 32; ++j) {
             const uint32_t s2 = 2u * (threadIdx.x + 1024u * (unsigned)j);
             tab[threadIdx.x + 1024u * (unsigned)j] = decode_pair<CB>(s2, s2 + 1u);
+        }
+    }
+    // ---- NORM: every workgroup sums the squares of the whole row (its k-blocks may be only a
+    // part of it), in double: per thread over a strided share, per wave by butterflies, the
+    // sixteen waves' sums added in order; then y = ((v * rmf) * (w + bias)) * scale rounded to
+    // fp16, as rms_norm_kernel forms it
+    if constexpr (NORM) {
+        double ss = 0.0;
+        for (unsigned e = threadIdx.x; e < (unsigned)p.K / 2; e += kStreamWaves * 64) {
+            const float2_t xv = ((global_ptr<const float2_t>)as_global(p.norm_x))[e];
+            const float2_t rv = ((global_ptr<const float2_t>)as_global(p.norm_res))[e];
+            const float2_t v = {rv.x + xv.x, rv.y + xv.y};
+            ss += (double)v.x * (double)v.x;
+            ss += (double)v.y * (double)v.y;
+            // the first workgroup of the first problem writes the updated residual stream
+            if (prob == 0 && gl == 0) ((global_ptr<float2_t>)as_global(p.norm_res_out))[e] = v;
+        }
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) ss += __shfl_xor(ss, d, 64);
+        if (lane == 0) norm_part[wave] = ss;
+        __syncthreads();
+        double total = 0.0;
+#pragma unroll
+        for (int w = 0; w < kStreamWaves; ++w) total += norm_part[w];
+        const float rmf = (float)(1.0 / sqrt(total / (double)p.K + (double)p.norm_eps));
+#pragma unroll
+        for (int t = 0; t < kRot; ++t) {
+            const float w0 = p.norm_weight_bf16 ? __builtin_bit_cast(float, nrm_w[t] << 16)
+                                                : (float)__builtin_bit_cast(_Float16, (uint16_t)(nrm_w[t] & 0xffffu));
+            const float w1 = p.norm_weight_bf16 ? __builtin_bit_cast(float, nrm_w[t] & 0xffff0000u)
+                                                : (float)__builtin_bit_cast(_Float16, (uint16_t)(nrm_w[t] >> 16));
+            float t0 = nrm_v[t].x * rmf, t1 = nrm_v[t].y * rmf;
+            t0 = t0 * (w0 + p.norm_bias);
+            t1 = t1 * (w1 + p.norm_bias);
+            t0 = t0 * p.norm_scale;
+            t1 = t1 * p.norm_scale;
+            rot_x[t].x = (_Float16)t0;
+            rot_x[t].y = (_Float16)t1;
         }
     }
     // ---- rotate; a_had: the workgroup that owns tile row 8 * kb of column block 0 writes k-block kb
@@ -580,7 +648,7 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
         z1 = (z1 * kRsqrt128) * (float)sv.y;
         const size_t at = (size_t)cbx * 128 + 2 * lane;
         if (p.out_fp32) {
-            float2_t o = {z0, z1};
+            float2_t o = {z0 + add_mine.x, z1 + add_mine.y};
             *(float2_t*)((float*)cout + at) = o;
         } else {
             half2_t o = {(_Float16)z0, (_Float16)z1};

@@ -448,6 +448,29 @@ public:
                            intermediate_, gate_.k_bits(), (int)gate_.codebook(), gpu.raw_stream()) != 0)
             throw KernelError(berth_exl3_last_error());
     }
+    // The FFN block around the MLP through berth_exl3_mlp_block: residual_out = residual + x,
+    // y = mlp(rms_norm(residual_out)) + residual_out; x, residual, residual_out, y fp32
+    // [rows][hidden], norm_weight bf16 (or fp16) [hidden].  One row of large linears is two
+    // launches; residual_out must be a buffer of its own.
+    void forward_block(const Gpu& gpu, const DeviceBuffer<float>& x, const DeviceBuffer<float>& residual,
+                       DeviceBuffer<float>& residual_out, const DeviceBuffer<uint16_t>& norm_weight, DeviceBuffer<float>& y,
+                       float epsilon = 1e-6f, float constant_bias = 1.0f, float constant_scale = 1.0f,
+                       bool weight_bf16 = true, int rows = 1) const
+    {
+        if (!uniform_) throw InputError("mlp: the one-call path needs one bit rate and codebook");
+        if (has_bias_) throw InputError("mlp: the one-call path does not add a bias");
+        if (rows < 1 || rows > max_rows_) throw InputError("mlp: rows exceed the layer scratch");
+        const size_t n = (size_t)rows * hidden_;
+        if (x.len() < n || residual.len() < n || residual_out.len() < n || y.len() < n || norm_weight.len() < (size_t)hidden_)
+            throw InputError(gate_.prefix() + ": buffer too small");
+        if (h_norm_.len() < n) h_norm_ = DeviceBuffer<Half>::zeroed(gpu, (size_t)max_rows_ * hidden_);
+        const berth_exl3_lin lins[3] = {gate_.table_entry(), up_.table_entry(), down_.table_entry()};
+        const berth_rms_norm norm{norm_weight.raw(), epsilon, constant_bias, constant_scale, weight_bf16 ? 1 : 0};
+        if (berth_exl3_mlp_block(x.raw(), residual.raw(), residual_out.raw(), &norm, lins, h_norm_.raw(), g_.raw(), u_.raw(),
+                                 x_had_.raw(), act_had_.raw(), y.raw(), rows, hidden_, intermediate_, gate_.k_bits(),
+                                 (int)gate_.codebook(), gpu.raw_stream()) != 0)
+            throw KernelError(berth_exl3_last_error());
+    }
     // x fp16 [hidden] -> y fp32 [hidden], the reference's four calls (mlp.rs:118-150)
     void forward(const Gpu& gpu, const DeviceBuffer<Half>& x, DeviceBuffer<float>& y) const
     {
@@ -479,6 +502,7 @@ private:
     int hidden_ = 0, intermediate_ = 0, max_rows_;
     bool uniform_ = false, has_bias_ = false;
     DeviceBuffer<Half> g_, u_, x_had_, act_had_;
+    mutable DeviceBuffer<Half> h_norm_;     // scratch of forward_block, allocated on first use
 };
 
 // An EXL3 linear that stacks `blocks` equal linears along K: tile rows [b * K/16, (b+1) * K/16)

@@ -106,6 +106,18 @@ struct LinearArgs {
     int size_m, size_k, size_n, k_bits, codebook, out_fp32;
     hipStream_t stream;
     const void* a_up = nullptr;   // VALU kernel only: the input is silu(a) * a_up, element by element
+    const float* out_add = nullptr;   // streaming kernel only (one row, fp32 output): a row added to the output
+};
+
+// RMS norm with the residual added first, as the input of a launch of the streaming kernel
+// (the arithmetic of berth_ops_rms_norm_res_in; the sum goes to res_out, which aliases neither)
+struct NormInput {
+    const float* x;             // fp32 [K]
+    const float* res;           // fp32 [K]
+    float* res_out;             // fp32 [K]
+    const void* weight;         // fp16 or bf16 [K]
+    float epsilon, constant_bias, constant_scale;
+    int weight_bf16;
 };
 
 // two linears of one shape on the same input rows in one launch (gate and up of an MLP)
@@ -118,8 +130,12 @@ struct PairArgs {
     void* a_had;                // [size_m][size_k]
     int size_m, size_k, size_n, k_bits, codebook;
     hipStream_t stream;
+    const NormInput* norm = nullptr;    // one row, streaming kernel only: `a` is then unused
 };
 std::string launch_gemv_pair(const PairArgs& args);
+// whether a one-row launch of `problems` linears of this shape takes the streaming kernel (and,
+// with whole_rows, whether every workgroup of it then holds the whole input row)
+bool gemv_stream_applies(int problems, int size_k, int size_n, bool whole_rows);
 
 // grouped (MoE) launches: problems, experts and num_problems are device memory
 struct GroupedArgs {

@@ -374,6 +374,27 @@ class MlpLayer:
         K.ops.silu_mul(ptr(self.g), ptr(self.u), ptr(self.u), self.intermediate, 0.0, gpu.raw_stream())
         self.down.forward(gpu, self.u, y, OutDtype.F32)
 
+    def forward_block(self, gpu: Gpu, x: torch.Tensor, residual: torch.Tensor, residual_out: torch.Tensor,
+                      norm_weight: torch.Tensor, y: torch.Tensor, epsilon: float = 1e-6, constant_bias: float = 1.0,
+                      constant_scale: float = 1.0, weight_bf16: bool = True, rows: int = 1) -> None:
+        """The FFN block around the MLP in one call (`berth_exl3_mlp_block`): residual_out =
+        residual + x; y = mlp(rms_norm(residual_out)) + residual_out.  x, residual, residual_out
+        and y fp32 [rows][hidden]."""
+        if not self.uniform or self.has_bias:
+            raise InputError(f"{self.gate.prefix}: the block call takes one bit rate and codebook and no bias")
+        if rows * self.intermediate > self.g.numel():
+            raise InputError(f"{self.gate.prefix}: buffer too small")
+        if self.x_had is None or self.x_had.numel() < rows * self.hidden:
+            self.x_had = torch.zeros(rows * self.hidden, dtype=torch.float16, device=x.device)
+            self.act_had = torch.zeros(self.g.numel(), dtype=torch.float16, device=x.device)
+        if getattr(self, "h_norm", None) is None or self.h_norm.numel() < rows * self.hidden:
+            self.h_norm = torch.zeros(rows * self.hidden, dtype=torch.float16, device=x.device)
+        norm = K.RmsNorm(ptr(norm_weight), epsilon, constant_bias, constant_scale, int(weight_bf16))
+        lins = [(ptr(l.trellis), ptr(l.suh), ptr(l.svh)) for l in (self.gate, self.up, self.down)]
+        K.exl3_mlp_block(ptr(x), ptr(residual), ptr(residual_out), norm, lins, ptr(self.h_norm), ptr(self.g), ptr(self.u),
+                         ptr(self.x_had), ptr(self.act_had), ptr(y), rows, self.hidden, self.intermediate,
+                         self.gate.k_bits, self.gate.codebook, gpu.raw_stream())
+
     def prefill(self, gpu: Gpu, scratch: RowScratch, x: torch.Tensor, y: torch.Tensor, rows: int) -> None:
         """x fp16 [rows][hidden] -> y fp32 [rows][hidden]."""
         if rows * self.intermediate > self.g.numel():

@@ -92,6 +92,7 @@ def load() -> C.CDLL:
         L.berth_moe_last_error.restype = C.c_char_p
         L.berth_moe_last_launch.restype = C.c_char_p
         L.berth_kernels_workspace.argtypes = [C.POINTER(vp), C.POINTER(C.c_size_t), C.POINTER(vp), C.POINTER(ci)]
+        L.berth_exl3_mlp_block.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         L.berth_kernels_pending_fault.restype = C.c_longlong
         L.berth_kernels_pending_fault.argtypes = [ci]
         L.berth_kernels_reload_env.restype = None
@@ -140,6 +141,23 @@ def exl3_mlp(x, lins, gate_out, up_out, a_had, act_had, y, size_m, hidden, inter
                                int(codebook), stream)
     if rc != 0:
         raise LaunchError(last_error() or f"exl3 mlp launch failed ({rc})")
+
+
+class RmsNorm(C.Structure):
+    """`berth_rms_norm`: the norm ahead of an MLP (weight fp16 or bf16 [hidden])."""
+    _fields_ = [("weight", C.c_void_p), ("epsilon", C.c_float), ("constant_bias", C.c_float),
+                ("constant_scale", C.c_float), ("weight_bf16", C.c_int)]
+
+
+def exl3_mlp_block(x, residual, residual_out, norm: RmsNorm, lins, h_norm, gate_out, up_out, a_had, act_had, y,
+                   size_m, hidden, intermediate, k_bits, codebook: Codebook, stream=None) -> None:
+    """berth_exl3_mlp_block: residual add + RMS norm, the MLP, and the residual add behind it
+    (two launches for one row of streaming-kernel sizes)."""
+    arr = (Exl3Lin * 3)(*[Exl3Lin(*l) for l in lins])
+    rc = load().berth_exl3_mlp_block(x, residual, residual_out, C.byref(norm), arr, h_norm, gate_out, up_out, a_had,
+                                     act_had, y, size_m, hidden, intermediate, k_bits, int(codebook), stream)
+    if rc != 0:
+        raise LaunchError(last_error() or f"exl3 mlp block launch failed ({rc})")
 
 
 def unpack_signs(packed, out, packed_bytes: int, stream=None) -> None:

@@ -261,6 +261,31 @@ int berth_exl3_mlp(const void* x, const berth_exl3_lin* lins, void* gate_out, vo
                    void* a_had, void* act_had, void* y, int size_m, int hidden, int intermediate,
                    int k_bits, int codebook, void* stream);
 
+/* No counterpart in the reference as one call: the FFN block of a decoder layer as its engine
+ * issues it (crates/berth-engine/src/mlp.rs:118-150 between the two glue ops of
+ * crates/berth-kernels/src/ops.rs:430-500 and :522-552):
+ *     residual_out = residual + x                                  (fp32, exact)
+ *     h = rms(residual_out) * (weight + constant_bias) * constant_scale   (fp16; berth_ops_rms_norm_res_in)
+ *     y = berth_exl3_mlp(h) + residual_out                         (fp32; berth_ops_add_f32)
+ * x, residual, residual_out, y fp32 [m][hidden]; residual_out must alias neither x nor residual
+ * (the in-place update of the reference's op would race with the workgroups still reading
+ * it); y may alias x.  h_norm fp16 [m][hidden] is scratch (written when the launches are not
+ * fused).  The other buffers are berth_exl3_mlp's.  One row: where the gate / up pair takes the
+ * one-row streaming kernel the norm is formed while that launch rotates its input (same fp32
+ * steps as berth_ops_rms_norm_res_in; the sum of squares in double, whose order of summation
+ * differs), and where the down projection takes it the residual is added where it writes its
+ * output: two launches when both do.  Anything else runs the same arithmetic as separate
+ * launches. */
+typedef struct {
+    const void* weight;         /* fp16 or bf16 [hidden] */
+    float epsilon, constant_bias, constant_scale;
+    int weight_bf16;
+} berth_rms_norm;
+int berth_exl3_mlp_block(const void* x, const void* residual, void* residual_out, const berth_rms_norm* norm,
+                         const berth_exl3_lin* lins, void* h_norm, void* gate_out, void* up_out, void* a_had,
+                         void* act_had, void* y, int size_m, int hidden, int intermediate, int k_bits,
+                         int codebook, void* stream);
+
 /* x fp16 [T][H]; wr fp16 [H][E] (the unquantised router, mlp.gate.weight laid out
  * input-major); bias fp32 [E] or NULL; idx int32 [T][k]; w fp32 [T][k]; logits fp32
  * [T][E] or NULL; parts_scratch fp32 [T][ceil(H/64)][E]. */

@@ -100,3 +100,50 @@ def test_cpp_mlp_forward_fused(tmp_path, rows):
     u, _ = O.linear(x, *trio["up"], H, I, bits, 2)
     want, _ = O.linear(O.silu_mul(g, u).reshape(rows, I), *trio["down"], I, H, bits, 2, out_fp32=True)
     assert np.abs(y - want.reshape(rows, H)).max() <= 2e-3 * np.abs(want).max()
+
+
+def _block_inputs(gpu, H, rows, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((rows, H)).astype(np.float32)
+    res = (3.0 * rng.standard_normal((rows, H))).astype(np.float32)
+    w = (0.1 * rng.standard_normal(H)).astype(np.float32)
+    w_bf16 = (w.view(np.uint32) >> 16).astype(np.uint16)          # truncated: any bf16 pattern will do
+    up = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu.device)
+    return up(x), up(res), torch.from_numpy(w_bf16.view(np.int16)).to(gpu.device)
+
+
+@pytest.mark.parametrize("rows,H,I,bits,fused", [(1, 2048, 12288, 3, "both"), (1, 1024, 2816, 4, "none"),
+                                                  (3, 256, 384, 4, "none"), (20, 256, 384, 4, "none")])
+def test_mlp_block_call_equals_norm_mlp_add_as_separate_calls(rows, H, I, bits, fused):
+    """berth_exl3_mlp_block against berth_ops_rms_norm_res_in -> berth_exl3_mlp -> berth_ops_add_f32
+    on the same inputs: the residual stream, the rotated input of gate / up (hence the norm's
+    fp16 output) and the gate / up outputs bit for bit; the block's output bit for bit where
+    the launches are the same, and within the summation-order bound otherwise."""
+    from berth_amd.device import ptr
+    gpu = Gpu(0)
+    _, mlp = _layer(gpu, H, I, bits, 9700 + rows, rows)
+    x, res, w = _block_inputs(gpu, H, rows, 9800 + rows)
+    eps = 1e-6
+    # the separate calls
+    res_ref = res.clone()
+    h = torch.zeros((rows, H), dtype=torch.float16, device=gpu.device)
+    K.ops.rms_norm_res_in(ptr(x), ptr(w), ptr(h), ptr(res_ref), rows, H, eps, 1.0, 1.0, True, gpu.raw_stream())
+    y_ref = torch.zeros((rows, H), dtype=torch.float32, device=gpu.device)
+    mlp.forward(gpu, h, y_ref, rows=rows)
+    K.ops.add_f32(ptr(y_ref), ptr(res_ref), ptr(y_ref), rows * H, gpu.raw_stream())
+    gpu.synchronize()
+    xh_ref, g_ref, u_ref = host_u16(mlp.x_had)[:rows * H].copy(), host_u16(mlp.g)[:rows * I].copy(), host_u16(mlp.u)[:rows * I].copy()
+    mlp.x_had.zero_(); mlp.g.zero_(); mlp.u.zero_()
+    # the block call
+    res_out = torch.zeros_like(res)
+    y = torch.zeros((rows, H), dtype=torch.float32, device=gpu.device)
+    mlp.forward_block(gpu, x, res, res_out, w, y, epsilon=eps, rows=rows)
+    gpu.synchronize()
+    launch = K.last_launch()
+    assert ("pair,norm" in launch) == (fused == "both") and ("+residual" in launch) == (fused == "both"), launch
+    assert np.array_equal(res_out.cpu().numpy().view(np.uint32), res_ref.cpu().numpy().view(np.uint32))
+    if rows <= 8:
+        assert np.array_equal(host_u16(mlp.x_had)[:rows * H], xh_ref)
+        assert np.array_equal(host_u16(mlp.g)[:rows * I], g_ref) and np.array_equal(host_u16(mlp.u)[:rows * I], u_ref)
+    a, b = y.cpu().numpy(), y_ref.cpu().numpy()
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), float(np.abs(a - b).max())
