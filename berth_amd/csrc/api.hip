@@ -62,8 +62,9 @@ Workspace& workspace_for_current_device()
 std::string describe_device_fault(unsigned code)
 {
     if (code >= 0x40000000u)
-        return "an earlier streaming GEMV launch on this device gave up waiting for the other contributors of column block " +
-               std::to_string(code - 0x40000001u) + " and wrote NaN there";
+        return "an earlier streaming GEMV launch on this device found the accumulator of column block " +
+               std::to_string(code - 0x40000001u) + " inconsistent (contributions missing or left over) and wrote NaN "
+               "there; the accumulators have been cleared";
     return "an earlier launch on this device gave up waiting for the split-K partial sums of tile " +
            std::to_string(code - 1u) + " and left it unwritten";
 }
@@ -74,6 +75,11 @@ void throw_pending_device_fault(const Workspace& ws)
     const unsigned code = *ws.fault_host;
     if (code == 0u) return;
     *ws.fault_host = 0u;
+    if (code >= 0x40000000u && ws.accum) {
+        // a streaming launch found its accumulators in a state no launch leaves behind: start over
+        (void)hipDeviceSynchronize();
+        (void)hipMemset(ws.accum, 0, (size_t)ws.accum_slots * 1024);
+    }
     throw std::runtime_error(describe_device_fault(code) +
                              " (the library's workspace serves one launch at a time per device: launches "
                              "that overlap on two streams mix their counters); this call launched nothing");
@@ -320,6 +326,22 @@ extern "C" long long berth_kernels_pending_fault(int device)
     const unsigned code = *ws.fault_host;
     if (code) *ws.fault_host = 0u;
     return (long long)code;
+}
+
+// Diagnostics: the streaming GEMV's column-block accumulators of the current device
+// (`slots` blocks of 128 64-bit words, zero between launches).
+extern "C" int berth_kernels_accumulators(void** accum, int* slots)
+{
+    try {
+        const Workspace& ws = workspace_for_current_device();
+        if (accum) *accum = ws.accum;
+        if (slots) *slots = ws.accum_slots;
+        return 0;
+    } catch (const std::exception& err) {
+        g_exl3_err = err.what();
+        (void)hipGetLastError();
+        return -1;
+    }
 }
 
 // Diagnostics: the per-device internals (allocated on first use), for tools that inspect or

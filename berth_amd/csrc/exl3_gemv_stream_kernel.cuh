@@ -617,11 +617,20 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
             unsigned long long t0 = __hip_atomic_fetch_add(word, f0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + f0;
             unsigned long long t1 = __hip_atomic_fetch_add(word + 1, f1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + f1;
             // the sharer whose add completed column 0 finishes the column block
-            if ((unsigned)__builtin_amdgcn_readfirstlane((int)((unsigned)t0 & 0xffu)) != count) continue;
+            const unsigned arrived = (unsigned)__builtin_amdgcn_readfirstlane((int)((unsigned)t0 & 0xffu));
+            if (arrived < count) continue;
             // usually every column is complete by then; one that another sharer's add had not
             // reached yet is read again (that sharer's add is in flight: the wait is short)
             unsigned spins = 0;
             while (true) {
+                if (arrived > count) {
+                    // more contributions than sharers: the accumulator was not zero when the launch
+                    // began (an earlier launch died, or two launches overlapped on this device)
+                    if (p.fault && lane == 0)
+                        __hip_atomic_store(p.fault, 0x40000001u + (unsigned)cbx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    t0 = t1 = 0x100ull;
+                    break;
+                }
                 const bool done = ((unsigned)t0 & 0xffu) == count && ((unsigned)t1 & 0xffu) == count;
                 if (__builtin_amdgcn_ballot_w64(!done) == 0ull) break;
                 if (++spins > p.spin_limit) {
@@ -637,8 +646,10 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
                     t1 = __hip_atomic_load(word + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
-            __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(word + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (arrived == count) {
+                __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(word + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
             z0 = from_fixed_tagged(t0);
             z1 = from_fixed_tagged(t1);
         }

@@ -92,6 +92,7 @@ def load() -> C.CDLL:
         L.berth_moe_last_error.restype = C.c_char_p
         L.berth_moe_last_launch.restype = C.c_char_p
         L.berth_kernels_workspace.argtypes = [C.POINTER(vp), C.POINTER(C.c_size_t), C.POINTER(vp), C.POINTER(ci)]
+        L.berth_kernels_accumulators.argtypes = [C.POINTER(vp), C.POINTER(ci)]
         L.berth_exl3_mlp_block.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
         L.berth_kernels_pending_fault.restype = C.c_longlong
         L.berth_kernels_pending_fault.argtypes = [ci]

@@ -88,6 +88,12 @@ int berth_kernels_init(int device);
  * kernel on the device returns -1 with that report instead of launching. */
 int berth_kernels_workspace(void** partials, size_t* partial_bytes, void** counters, int* counter_slots);
 
+/* Diagnostics, no counterpart in the reference: the one-row streaming GEMV's column-block
+ * accumulators of the current device, `slots` blocks of 128 64-bit words that every launch
+ * leaves at zero (value in units of 2^-18 in bits 16..63, contributions that did not fit in
+ * bits 8..15, contributions in bits 0..7). */
+int berth_kernels_accumulators(void** accum, int* slots);
+
 /* No counterpart in the reference.  Host-only query for the caller's synchronisation points:
  * 0 when no kernel on `device` has reported a fault since the last report, else the fault
  * code, and the report is cleared (-1: no such device).  A bounded wait inside a kernel that

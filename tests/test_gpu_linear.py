@@ -483,6 +483,7 @@ def test_very_wide_output_uses_closer_counters(rows):
 @pytest.mark.parametrize("name,kernel", [("gate_proj", "exl3_gemm_wide_kernel<4,2,256x256>"),
                                          ("down_proj", "exl3_gemm_balanced_kernel<4,2,128x256>"),
                                          ("q_proj", "exl3_gemm_balanced_kernel<4,2,128x256>"),
+                                         ("o_proj", "exl3_gemm_balanced_kernel<4,2,128x256>"),
                                          ("k_proj", "exl3_gemm_kernel<4,2,32x256>")])
 def test_prefill_27b_shapes_at_512_rows_slices_match_oracle(name, kernel):
     """BASELINE configs[2] at full size (512 rows, 4 bpw, the 27B shapes): each of the four
@@ -630,8 +631,8 @@ def test_27b_shapes_batch1_4bpw_windows_match_oracle(name):
 
 
 @pytest.mark.parametrize("bits", [2, 3, 5])
-@pytest.mark.parametrize("name", ["gate_proj", "down_proj"])
+@pytest.mark.parametrize("name", ["gate_proj", "down_proj", "q_proj", "o_proj", "k_proj"])
 def test_27b_shapes_batch1_other_rates_windows_match_oracle(name, bits):
-    """BASELINE configs[1] at 2, 3 and 5 bpw on the two large shapes."""
+    """BASELINE configs[1] at 2, 3 and 5 bpw on every shape of the set (v_proj has k_proj's)."""
     Kk, N = synth.SHAPES_27B[name]
-    _window_check(name, Kk, N, bits, name == "down_proj", 7200 + 10 * bits + Kk % 97)
+    _window_check(name, Kk, N, bits, name in ("down_proj", "o_proj"), 7200 + 10 * bits + Kk % 97 + len(name))

@@ -127,11 +127,21 @@ def _check_stages(layer, x, experts_np, shared_np, idx, w, out, T, H, E, k, I, b
     base = np.zeros((T, H), dtype=np.float32)
     if shared_np is not None:
         base = view("shared_out", np.float32, (T, H)).copy()
-        sg, _ = O.linear(x, *shared_np[0], H, shared_I, bits, 2)
-        su, _ = O.linear(x, *shared_np[1], H, shared_I, bits, 2)
-        # the shared expert's own down output is checked end to end below; its
-        # gate/up feed a SiLU whose fp16 rounding is shared by both sides
-        del sg, su
+        # the always-on expert, stage by stage like the routed ones: its gate / up rows
+        # (where the layer keeps them) against the oracle, its down row from the GPU's own
+        # gate / up outputs
+        sg_want, _ = O.linear(x, *shared_np[0], H, shared_I, bits, 2)
+        su_want, _ = O.linear(x, *shared_np[1], H, shared_I, bits, 2)
+        if shared_I == I:           # one more expert of the grouped launches: rows P .. P + T - 1
+            sg = ws[offs["gate_out"] + P * I * 2:offs["gate_out"] + (P + T) * I * 2].view(np.float16).reshape(T, I)
+            su = ws[offs["up_out"] + P * I * 2:offs["up_out"] + (P + T) * I * 2].view(np.float16).reshape(T, I)
+            assert close(sg, sg_want)[0] == 0 and close(su, su_want)[0] == 0, "shared gate / up"
+            act = O.silu_mul(sg, su).reshape(T, I)
+        else:
+            act = O.silu_mul(sg_want.astype(np.float16), su_want.astype(np.float16)).reshape(T, shared_I)
+        sd_want, _ = O.linear(act, *shared_np[2], shared_I, H, bits, 2, out_fp32=True)
+        tol = dict() if shared_I == I else dict(rtol=4e-3, atol=2e-3)      # oracle gate / up: their fp16 roundings differ in a few last bits
+        assert close(base, sd_want, **tol)[0] == 0, "shared down"
     acc = base.astype(np.float32)
     for j in range(k):
         acc = (np.float32(1) * acc + w[:, j:j + 1].astype(np.float32) * slot[inv.reshape(T, k)[:, j]]).astype(np.float32)

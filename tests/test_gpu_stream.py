@@ -210,3 +210,127 @@ def test_state_tables_hold_every_decoded_state():
     for cb in (0, 1, 2):
         with forced(wgs=2, lut="0xA"):
             check(Kk, N, 8, cb, True, 6000 + cb)
+
+
+def test_mgemm_host_lists_give_the_bits_of_device_lists():
+    """berth_ops_mgemm_hostlists (the problems by value in the kernel arguments) against
+    berth_ops_mgemm (device lists) on one sliced bundle with a narrow slice and on a uniform
+    bundle with one shared and with per-problem inputs: outputs and rotated inputs bit for bit."""
+    Kk = 1024
+    widths = (384, 128, 256)
+    lins = [synth.linear(930 + i, Kk, n, 4) for i, n in enumerate(widths)]
+    d = [[dev(t.view(np.uint16)) for t in lin] for lin in lins]
+    x = synth.activations(940, 3, Kk)
+    d_x = dev(x.view(np.uint16))
+    host = dict(b=np.array([dd[0].data_ptr() for dd in d], dtype=np.uint64),
+                suh=np.array([dd[1].data_ptr() for dd in d], dtype=np.uint64),
+                svh=np.array([dd[2].data_ptr() for dd in d], dtype=np.uint64),
+                size_n=np.array(widths, dtype=np.int32), stride=np.array(widths, dtype=np.int32),
+                src=np.array([0, 1, 2], dtype=np.int32))
+    devl = {k: torch.from_numpy(v.view(np.int64) if v.dtype == np.uint64 else v).to(DEV) for k, v in host.items()}
+
+    def sliced(fn, lists, addr):
+        outs = [torch.zeros((1, n), dtype=torch.float32, device=DEV) for n in widths]
+        a_had = torch.zeros((3, Kk), dtype=torch.float16, device=DEV)
+        c_host = np.array([o.data_ptr() for o in outs], dtype=np.uint64)
+        c_list = c_host if lists is host else torch.from_numpy(c_host.view(np.int64)).to(DEV)
+        with forced(wgs=2, lut="0"):
+            fn(d_x.data_ptr(), addr(lists["b"]), outs[0].data_ptr(), addr(lists["suh"]), a_had.data_ptr(),
+               addr(lists["svh"]), 1, Kk, 384, 4, Codebook.MUL1, OutDtype.F32, 1, 3, addr(lists["size_n"]), addr(c_list),
+               addr(lists["stride"]), addr(lists["src"]), 3)
+            launch = K.ops.last_launch()
+        torch.cuda.synchronize()
+        return [o.cpu().numpy().view(np.uint32) for o in outs], host_u16(a_had), launch
+
+    ref, ref_had, ref_launch = sliced(K.ops.exl3_mgemm, devl, lambda t: t.data_ptr())
+    got, got_had, got_launch = sliced(K.ops.exl3_mgemm_hostlists, host, lambda a: a.ctypes.data)
+    assert "by value" in got_launch and "by value" not in ref_launch and "exl3_gemv_stream_kernel" in ref_launch
+    assert all(np.array_equal(a, b) for a, b in zip(got, ref)) and np.array_equal(got_had, ref_had)
+
+    # uniform: three linears of one shape
+    N = 256
+    ulins = [synth.linear(950 + i, Kk, N, 4) for i in range(3)]
+    ud = [[dev(t.view(np.uint16)) for t in lin] for lin in ulins]
+    uh = [np.array([dd[j].data_ptr() for dd in ud], dtype=np.uint64) for j in range(3)]
+    udv = [torch.from_numpy(a.view(np.int64)).to(DEV) for a in uh]
+    for bszm_in in (3, 1):
+        res = []
+        for fn, lists, addr in ((K.ops.exl3_mgemm, udv, lambda t: t.data_ptr()),
+                                (K.ops.exl3_mgemm_hostlists, uh, lambda a: a.ctypes.data)):
+            c = torch.zeros((3, 1, N), dtype=torch.float16, device=DEV)
+            a_had = torch.zeros((3, Kk), dtype=torch.float16, device=DEV)
+            with forced(wgs=2, lut="0"):
+                fn(d_x.data_ptr(), addr(lists[0]), c.data_ptr(), addr(lists[1]), a_had.data_ptr(), addr(lists[2]), 1, Kk, N,
+                   4, Codebook.MUL1, OutDtype.F16, bszm_in, 3)
+            torch.cuda.synchronize()
+            res.append((host_u16(c), host_u16(a_had)))
+        assert np.array_equal(res[0][0], res[1][0]) and np.array_equal(res[0][1], res[1][1]), bszm_in
+
+
+def test_mgemm_host_lists_refuse_what_the_streaming_kernel_does_not_serve():
+    bad = 0xdead000
+    one = np.array([bad], dtype=np.uint64)
+    with pytest.raises(K.LaunchError, match="host lists"):      # three rows
+        K.ops.exl3_mgemm_hostlists(bad, one.ctypes.data, bad, one.ctypes.data, bad, one.ctypes.data, 3, 1024, 256, 4,
+                                   Codebook.MUL1, OutDtype.F16, 1, 1)
+    with pytest.raises(K.LaunchError, match="host lists"):      # a weight too small for the streaming kernel
+        K.ops.exl3_mgemm_hostlists(bad, one.ctypes.data, bad, one.ctypes.data, bad, one.ctypes.data, 1, 128, 128, 4,
+                                   Codebook.MUL1, OutDtype.F16, 1, 1)
+    many = np.full(17, bad, dtype=np.uint64)
+    with pytest.raises(K.LaunchError, match="host lists"):      # seventeen problems
+        K.ops.exl3_mgemm_hostlists(bad, many.ctypes.data, bad, many.ctypes.data, bad, many.ctypes.data, 1, 5120, 17408, 4,
+                                   Codebook.MUL1, OutDtype.F16, 1, 17)
+    assert K.ops.last_launch() == ""
+
+
+def test_stale_accumulator_is_reported_and_cleared():
+    """Forced from the host: an accumulator word of the streaming kernel is given a contribution
+    count no launch leaves behind.  The launch that meets it writes NaN into that column block
+    and raises the device's fault word; the next launch reports it (and launches nothing), the
+    query reads clean afterwards, and the launch after that is back to normal.  Every kernel
+    exits by itself."""
+    import ctypes as C
+    from tests.test_gpu_runtime import Runtime
+    Kk, N, bits = 4096, 8192, 4
+    tr, suh, svh = synth.linear(960, Kk, N, bits)
+    x = synth.activations(961, 1, Kk)
+    d = {k: dev(v.view(np.uint16)) for k, v in dict(tr=tr, suh=suh, svh=svh, x=x).items()}
+    a_had = torch.zeros(Kk, dtype=torch.float16, device=DEV)
+
+    def launch(c):
+        K.exl3_linear(d["x"].data_ptr(), d["tr"].data_ptr(), c.data_ptr(), d["suh"].data_ptr(), a_had.data_ptr(),
+                      d["svh"].data_ptr(), 1, Kk, N, bits, Codebook.MUL1, OutDtype.F32)
+        text = K.last_launch()
+        torch.cuda.synchronize()
+        return text
+
+    good = torch.zeros(N, dtype=torch.float32, device=DEV)
+    assert "exl3_gemv_stream_kernel" in launch(good)
+    accum, slots = C.c_void_p(), C.c_int()
+    assert K.load().berth_kernels_accumulators(C.byref(accum), C.byref(slots)) == 0 and slots.value >= N // 128
+    rt = Runtime()
+    block = 5
+    stale = np.array([200], dtype=np.uint64)                       # 200 contributions already "there"
+    rt.ok(rt.copy_from_host(None, accum.value + block * 1024, stale.ctypes.data, 8))
+    assert K.pending_fault(0) == 0
+    c = torch.zeros(N, dtype=torch.float32, device=DEV)
+    launch(c)                                                       # accepted; every kernel exits
+    got = c.cpu().numpy()
+    assert np.isnan(got[block * 128:(block + 1) * 128]).all()
+    keep = np.ones(N, dtype=bool)
+    keep[block * 128:(block + 1) * 128] = False
+    assert np.array_equal(got[keep].view(np.uint32), good.cpu().numpy()[keep].view(np.uint32))
+    with pytest.raises(K.LaunchError, match=f"accumulator of column block {block} inconsistent"):
+        launch(c)
+    assert K.last_launch() == "" and K.pending_fault(0) == 0       # reported once, accumulators cleared
+    launch(c)
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), good.cpu().numpy().view(np.uint32))
+    # the query alone also reads and clears a report
+    rt.ok(rt.copy_from_host(None, accum.value + block * 1024, stale.ctypes.data, 8))
+    launch(c)
+    assert K.pending_fault(0) == 0x40000001 + block and K.pending_fault(0) == 0
+    zero = np.zeros(128, dtype=np.uint64)
+    rt.ok(rt.copy_from_host(None, accum.value + block * 1024, zero.ctypes.data, 1024))
+    launch(c)
+    assert np.array_equal(c.cpu().numpy().view(np.uint32), good.cpu().numpy().view(np.uint32))
+    rt.context_free(rt.ctx)

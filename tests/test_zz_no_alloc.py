@@ -69,3 +69,83 @@ def test_no_alloc_refuses_what_does_not_fit():
         with pytest.raises(K.LaunchError, match="bytes of split-K scratch"):
             K.exl3_linear_noalloc(bad, bad, bad, bad, bad, bad, 8, 16384, 16384, 2, Codebook.MUL1, OutDtype.F32)
     assert K.last_launch() == ""
+
+
+_CAPTURE_SCRIPT = r"""
+import sys
+import numpy as np
+import torch
+sys.path.insert(0, sys.argv[1])
+from berth_amd import kernels as K
+from berth_amd import synth
+from berth_amd.kernels import Codebook, OutDtype
+
+DEV = "cuda:0"
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).to(DEV)
+
+cases = []
+for m, Kk, N, bits, seed in ((1, 4096, 8192, 4, 8300), (1, 512, 256, 4, 8301), (3, 1024, 384, 3, 8302)):
+    tr, suh, svh = synth.linear(seed, Kk, N, bits)
+    x = synth.activations(seed + 1, m, Kk)
+    d = {k: dev(v.view(np.uint16)) for k, v in dict(tr=tr, suh=suh, svh=svh, x=x).items()}
+    c = torch.zeros((m, N), dtype=torch.float32, device=DEV)
+    a_had = torch.zeros((m, Kk), dtype=torch.float16, device=DEV)
+    cases.append((m, Kk, N, bits, d, c, a_had))
+
+def run(fn):
+    texts = []
+    for m, Kk, N, bits, d, c, a_had in cases:
+        fn(d["x"].data_ptr(), d["tr"].data_ptr(), c.data_ptr(), d["suh"].data_ptr(), a_had.data_ptr(),
+           d["svh"].data_ptr(), m, Kk, N, bits, Codebook.MUL1, OutDtype.F32, torch.cuda.current_stream().cuda_stream)
+        texts.append(K.last_launch())
+    return texts
+
+def outputs():
+    torch.cuda.synchronize()
+    return [c.cpu().numpy().view(np.uint32).copy() for *_, c, _ in cases]
+
+def clear():
+    for *_, c, _ in cases:
+        c.fill_(-3.0)
+
+# the very first calls of the entry point in this process are the recorded ones
+graph = torch.cuda.CUDAGraph()
+side = torch.cuda.Stream(device=DEV)
+with torch.cuda.stream(side):
+    with torch.cuda.graph(graph, stream=side):
+        texts = run(K.exl3_linear_noalloc)
+torch.cuda.synchronize()
+assert "exl3_gemv_stream_kernel" in texts[0] and "exl3_gemv_kernel" in texts[1], texts
+clear()
+run(K.exl3_linear)                      # eager, the allocating entry point: the reference bits
+want = outputs()
+for replay in range(3):
+    clear()
+    graph.replay()
+    got = outputs()
+    for g, w, t in zip(got, want, texts):
+        assert np.array_equal(g, w), (replay, t)
+    run(K.exl3_linear)                  # eager work of the same library between the replays
+    torch.cuda.synchronize()
+clear()
+run(K.exl3_linear_noalloc)              # and eagerly after the replays
+for g, w in zip(outputs(), want):
+    assert np.array_equal(g, w)
+print("capture ok")
+"""
+
+
+def test_no_alloc_first_call_inside_a_stream_capture_replays_bit_exact(tmp_path):
+    """The entry point's stated use: its first calls in a process are recorded into a HIP graph
+    (nothing may allocate, synchronise or clear memory there), the graph is replayed three
+    times with eager launches of the library in between, and every replay gives the bits of
+    berth_exl3_linear.  A process of its own, so that the calls really are the first."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    script = tmp_path / "capture.py"
+    script.write_text(_CAPTURE_SCRIPT)
+    r = subprocess.run([sys.executable, str(script), root], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "capture ok" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
