@@ -50,6 +50,7 @@ Workspace& workspace_for_current_device()
         hip_ok(hipHostGetDevicePointer(&fault_dev, fault_host, 0), "fault word device address");
         ws.fault_host = (volatile unsigned*)fault_host;
         ws.fault_dev = (unsigned*)fault_dev;
+        hip_ok(hipEventCreateWithFlags(&ws.order_event, hipEventDisableTiming), "ordering event");
         ws.cu_count = cus;
         ws.partial_bytes = kPartialBytes;
         ws.counter_slots = kCounters;
@@ -63,10 +64,58 @@ std::string describe_device_fault(unsigned code)
 {
     if (code >= 0x40000000u)
         return "an earlier streaming GEMV launch on this device found the accumulator of column block " +
-               std::to_string(code - 0x40000001u) + " inconsistent (contributions missing or left over) and wrote NaN "
-               "there; the accumulators have been cleared";
+               std::to_string(code - 0x40000001u) + " inconsistent (contributions left over: the block was left "
+               "unwritten; or missing: it holds NaN); the accumulators have been cleared";
     return "an earlier launch on this device gave up waiting for the split-K partial sums of tile " +
            std::to_string(code - 1u) + " and left it unwritten";
+}
+
+namespace {
+bool stream_is_capturing(hipStream_t stream)
+{
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;            // the legacy stream while another stream captures: leave it alone
+    }
+    return status != hipStreamCaptureStatusNone;
+}
+}  // namespace
+
+LaunchScope::LaunchScope(hipStream_t stream_) : ws(workspace_for_current_device()), stream(stream_)
+{
+    if (!knobs().stream_order) return;
+    std::lock_guard<std::mutex> lock(g_ws_mu);
+    if (ws.have_last && ws.last_stream == stream) {
+        // the usual case costs a comparison: no runtime call on the launch path
+        if (ws.multi_stream && ++ws.same_stream_run > 4096) {
+            ws.multi_stream = false;
+            ws.event_recorded = false;
+        }
+        record = ws.multi_stream && ws.order_event && !stream_is_capturing(stream);
+        return;
+    }
+    if (stream_is_capturing(stream)) return;
+    if (ws.have_last) {
+        if (ws.multi_stream && ws.event_recorded) {
+            hip_ok(hipStreamWaitEvent(stream, ws.order_event, 0), "hipStreamWaitEvent");
+        } else if (hipDeviceSynchronize() != hipSuccess) {
+            (void)hipGetLastError();        // another stream is capturing: nothing can be waited for here
+        }
+        ws.multi_stream = true;
+        ws.same_stream_run = 0;
+    }
+    ws.last_stream = stream;
+    ws.have_last = true;
+    record = ws.multi_stream && ws.order_event;
+}
+
+LaunchScope::~LaunchScope()
+{
+    if (!record) return;
+    std::lock_guard<std::mutex> lock(g_ws_mu);
+    if (hipEventRecord(ws.order_event, stream) == hipSuccess) ws.event_recorded = true;
+    else (void)hipGetLastError();
 }
 
 void throw_pending_device_fault(const Workspace& ws)
@@ -112,6 +161,7 @@ Knobs read_knobs()
     k.moe_fold_combine = env_int("BERTH_MOE_FOLD_COMBINE", 2);
     k.moe_inline_route = env_int("BERTH_MOE_INLINE_ROUTE", 1);
     k.moe_resolved = env_int("BERTH_MOE_RESOLVED", 1);
+    k.stream_order = env_int("BERTH_STREAM_ORDER", 1);
     const int spins = env_int("BERTH_SPIN_LIMIT", 0);
     k.spin_limit = spins > 0 ? (unsigned)spins : (1u << 20);
     return k;

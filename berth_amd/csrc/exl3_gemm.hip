@@ -53,7 +53,8 @@ static int gemm_counter_stride(long tiles)
 std::string launch_gemm(const LinearArgs& a)
 {
     if (a.size_k % 128 != 0) throw std::runtime_error("exl3 linear: size_k must be a multiple of 128");
-    Workspace& ws = workspace_for_current_device();
+    LaunchScope scope(a.stream);
+    Workspace& ws = scope.ws;
     throw_pending_device_fault(ws);
     std::string d0 = launch_had_r_128(a.a, a.a_had, a.suh, 1, a.size_m, a.size_k, 0, a.stream);
     GemmParams p{};
@@ -137,7 +138,8 @@ std::string launch_gemm_grouped(const GroupedArgs& g)
     const int mb = g.mb == 4 ? 4 : 1;
     if (g.size_k % 128 != 0 || g.size_n % 128 != 0)
         throw std::runtime_error("moe grouped linear: sizes must be multiples of 128");
-    Workspace& ws = workspace_for_current_device();
+    LaunchScope scope(g.stream);
+    Workspace& ws = scope.ws;
     throw_pending_device_fault(ws);
     GemmParams p{};
     p.fault = ws.fault_dev;

@@ -19,6 +19,7 @@
 #include "launch.h"
 
 #include <algorithm>
+#include <optional>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -203,7 +204,10 @@ std::string launch_gemv(const LinearArgs& a, const Workspace* scratch)
 {
     if (a.size_m < 1 || a.size_m > 8) throw std::runtime_error("exl3 gemv: rows must be in 1..=8");
     if (a.size_k % 128 != 0) throw std::runtime_error("exl3 linear: size_k must be a multiple of 128");
-    const Workspace& ws = scratch ? *scratch : workspace_for_current_device();
+    std::optional<LaunchScope> scope;
+    if (!scratch) scope.emplace(a.stream);
+    const Workspace& ws = scratch ? *scratch : scope->ws;
+    throw_pending_device_fault(ws);
     const int mmax = a.size_m == 1 ? 1 : 8;
     if (a.size_m == 1) {
         const StreamPlan pl = plan_stream(ws, 1, a.size_k, a.size_n);
@@ -257,7 +261,9 @@ std::string launch_gemv_pair(const PairArgs& a)
 {
     if (a.size_m < 1 || a.size_m > 8) throw std::runtime_error("exl3 gemv: rows must be in 1..=8");
     if (a.size_k % 128 != 0) throw std::runtime_error("exl3 linear: size_k must be a multiple of 128");
-    Workspace& ws = workspace_for_current_device();
+    LaunchScope scope(a.stream);
+    Workspace& ws = scope.ws;
+    throw_pending_device_fault(ws);
     const int mmax = a.size_m == 1 ? 1 : 8;
     if (a.size_m == 1) {
         const StreamPlan pl = plan_stream(ws, 2, a.size_k, a.size_n);
@@ -321,7 +327,9 @@ std::string launch_mgemm(const MgemmArgs& m)
 {
     if (m.size_k % 128 != 0) throw std::runtime_error("exl3_mgemm: size_k must be a multiple of 128");
     if (m.size_m > 8) throw std::runtime_error("exl3_mgemm: more than 8 rows is not built (use one linear per call)");
-    Workspace& ws = workspace_for_current_device();
+    LaunchScope scope(m.stream);
+    Workspace& ws = scope.ws;
+    throw_pending_device_fault(ws);
     const bool sliced = m.had_src_list != nullptr;
     const int mmax = m.size_m == 1 ? 1 : 8;
     if (m.host_lists) {
@@ -429,7 +437,9 @@ std::string launch_gemv_grouped(const GroupedArgs& g)
 {
     if (g.size_k % 128 != 0 || g.size_n % 128 != 0)
         throw std::runtime_error("moe grouped linear: sizes must be multiples of 128");
-    Workspace& ws = workspace_for_current_device();
+    LaunchScope scope(g.stream);
+    Workspace& ws = scope.ws;
+    throw_pending_device_fault(ws);
     GemvParams p{};
     p.a = (const _Float16*)g.a;
     p.a_up = (const _Float16*)g.a_up;

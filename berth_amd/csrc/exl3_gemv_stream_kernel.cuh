@@ -284,8 +284,11 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
     unsigned* const piece_last = piece_first + 16;
     double* const norm_part = (double*)(lds + kMetaOff + 128);         // NORM: one sum of squares per wave
 
-    static_assert(sizeof(StreamParams) > 10 * 64 && sizeof(StreamParams) <= 16 * 64, "argument lines touched below");
-    touch_kernel_arguments<16>();
+    // The scalar fields sit in the first six lines of the argument block; the by-value problems
+    // behind them are read by the launches that use them (touching all sixteen lines at the
+    // head cost every launch: 1.4 us per four-launch layer set, measured).
+    static_assert(offsetof(StreamParams, slice) <= 6 * 64 && sizeof(StreamParams) <= 16 * 64, "argument lines touched below");
+    touch_kernel_arguments<6>();
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const unsigned prob = div_magic(blockIdx.x, p.mgp);
@@ -618,24 +621,22 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
             unsigned long long t1 = __hip_atomic_fetch_add(word + 1, f1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + f1;
             // the sharer whose add completed column 0 finishes the column block
             const unsigned arrived = (unsigned)__builtin_amdgcn_readfirstlane((int)((unsigned)t0 & 0xffu));
-            if (arrived < count) continue;
+            if (arrived != count) {
+                // more contributions than sharers: the accumulator was not zero when the launch
+                // began (an earlier launch died, or two launches overlapped on this device).
+                // Nobody can finish the block then: it stays unwritten, and the host is told.
+                if (arrived > count && p.fault && lane == 0)
+                    __hip_atomic_store(p.fault, 0x40000001u + (unsigned)cbx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                continue;
+            }
             // usually every column is complete by then; one that another sharer's add had not
             // reached yet is read again (that sharer's add is in flight: the wait is short)
             unsigned spins = 0;
             while (true) {
-                if (arrived > count) {
-                    // more contributions than sharers: the accumulator was not zero when the launch
-                    // began (an earlier launch died, or two launches overlapped on this device)
-                    if (p.fault && lane == 0)
-                        __hip_atomic_store(p.fault, 0x40000001u + (unsigned)cbx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                    t0 = t1 = 0x100ull;
-                    break;
-                }
                 const bool done = ((unsigned)t0 & 0xffu) == count && ((unsigned)t1 & 0xffu) == count;
                 if (__builtin_amdgcn_ballot_w64(!done) == 0ull) break;
                 if (++spins > p.spin_limit) {
-                    // a contributor is missing (a stale accumulator, two launches mixed on one
-                    // device): say so, and leave no plausible numbers behind
+                    // a contributor is missing: say so, and leave no plausible numbers behind
                     if (p.fault && lane == 0)
                         __hip_atomic_store(p.fault, 0x40000001u + (unsigned)cbx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                     t0 = t1 = 0x100ull;
@@ -646,10 +647,8 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
                     t1 = __hip_atomic_load(word + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
-            if (arrived == count) {
-                __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(word + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
+            __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(word + 1, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             z0 = from_fixed_tagged(t0);
             z1 = from_fixed_tagged(t1);
         }

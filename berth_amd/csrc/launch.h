@@ -47,6 +47,13 @@ struct Workspace {
     int counter_slots = 0;          // most counters a launch may use
     size_t counter_words = 0;       // words behind `counters` (counters can be spread over them)
     bool strict = false;            // true: a launch that would not fit is refused instead of split less
+    // the stream of the device's previous launch, and the event later launches on other streams wait for
+    hipStream_t last_stream = nullptr;
+    bool have_last = false;
+    bool multi_stream = false;      // events are being recorded behind every launch
+    bool event_recorded = false;
+    int same_stream_run = 0;
+    hipEvent_t order_event = nullptr;
 };
 constexpr size_t kPartialBytes = (size_t)256 << 20;
 constexpr int kCounters = 65536;
@@ -72,6 +79,7 @@ struct Knobs {
     int moe_inline_route;       // BERTH_MOE_INLINE_ROUTE
     int moe_resolved;           // BERTH_MOE_RESOLVED
     unsigned spin_limit;        // BERTH_SPIN_LIMIT             polls of a bounded wait before it gives up
+    int stream_order;           // BERTH_STREAM_ORDER           0: launches of different streams are not ordered
 };
 const Knobs& knobs();
 void reload_knobs();
@@ -91,6 +99,24 @@ inline int counter_stride(const Workspace& ws, long units)
     return stride;
 }
 Workspace& workspace_for_current_device();
+// The workspace serves one launch at a time per device.  Launches of one stream are ordered
+// by the stream; a launch that arrives on another stream than the device's previous one must
+// not start while that one may still be running, or the two mix their partial sums and
+// counters.  LaunchScope, held by a launcher around its launches, sees to that without ever
+// touching the previous stream's handle (its owner may have destroyed it): the first time the
+// stream changes the device is drained once; from then on every scope records an event behind
+// its launches and a launch on another stream waits for that event.  After 4096 launches in
+// a row on one stream the events stop again, so a single-stream caller pays nothing.  Streams
+// that are being captured into a graph are left alone.
+struct LaunchScope {
+    explicit LaunchScope(hipStream_t stream);
+    ~LaunchScope();
+    LaunchScope(const LaunchScope&) = delete;
+    LaunchScope& operator=(const LaunchScope&) = delete;
+    Workspace& ws;
+    hipStream_t stream;
+    bool record = false;
+};
 // throws if a kernel of an earlier launch on this device reported a fault (and clears the report)
 void throw_pending_device_fault(const Workspace& ws);
 // polls a split-K finisher spends on its wait before it gives up (BERTH_SPIN_LIMIT, default 2^20)

@@ -676,7 +676,8 @@ std::string run_route(const void* x, const void* wr, const float* bias, int32_t*
                       float* logits, float* parts, int T, int H, int E, int k, int renorm,
                       hipStream_t stream, const PermuteParams* sort = nullptr)
 {
-    Workspace& ws = workspace_for_current_device();
+    LaunchScope scope(stream);
+    Workspace& ws = scope.ws;
     RouteParams p{};
     p.x = (const _Float16*)x;
     p.wr = (const _Float16*)wr;

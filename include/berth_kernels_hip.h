@@ -101,7 +101,8 @@ int berth_kernels_accumulators(void** accum, int* slots);
  * and fail with the report, but a caller that synchronises and launches nothing of this library
  * afterwards learns of it only here.  Codes below 0x40000000: 1 + the tile an MFMA split-K
  * finisher left unwritten; from 0x40000001: 0x40000001 + the column block a streaming GEMV
- * finisher filled with NaN. */
+ * launch left unwritten (contributions left over in its accumulator) or filled with NaN (a
+ * contribution missing). */
 long long berth_kernels_pending_fault(int device);
 
 /* No counterpart in the reference.  The BERTH_* environment knobs are read once per process;

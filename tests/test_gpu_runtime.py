@@ -246,3 +246,52 @@ def test_loading_what_is_not_a_code_object_fails_with_a_text(rt):
     rc = rt.module_load_file(rt.ctx, b"/nonexistent/berth.hsaco", C.byref(m))
     assert rc != 0 and rt.error_string(rc) and b"hipModuleLoad" in rt.last_error()
     assert rt.module_load_bytes(rt.ctx, None, 16, C.byref(m)) != 0          # refused before the driver sees it
+
+
+def test_launches_on_two_streams_are_ordered_on_the_shared_workspace():
+    """The library's split-K workspace serves one launch at a time per device.  Launches of
+    different streams used to mix their partial sums silently; now a launch on another stream
+    than the device's previous one waits for that stream's work so far.  Many alternating
+    launches of two different split-K linears on two non-blocking streams, with no
+    synchronisation by the caller in between, must each give the bits of a launch alone."""
+    import torch
+    from berth_amd import kernels as K
+    from berth_amd import synth
+    from berth_amd.kernels import Codebook, OutDtype
+    from tests.gpu_util import DEV, dev
+    rt = Runtime()
+    streams = [rt.stream() for _ in range(2)]
+    raw = [C.c_void_p(rt.stream_handle(s)) for s in streams]     # the hipStream_t behind each handle
+    shapes = [(1, 4096, 8192, 4), (1, 2048, 768, 4)]            # streaming kernel; 1..8-row kernel with split-K
+    work = []
+    for i, (m, Kk, N, bits) in enumerate(shapes):
+        tr, suh, svh = synth.linear(9900 + i, Kk, N, bits)
+        x = synth.activations(9910 + i, m, Kk)
+        d = {k: dev(v.view(np.uint16)) for k, v in dict(tr=tr, suh=suh, svh=svh, x=x).items()}
+        c = torch.zeros((m, N), dtype=torch.float32, device=DEV)
+        a_had = torch.zeros((m, Kk), dtype=torch.float16, device=DEV)
+        work.append((m, Kk, N, bits, d, c, a_had))
+
+    def launch(i, stream):
+        m, Kk, N, bits, d, c, a_had = work[i]
+        K.exl3_linear(d["x"].data_ptr(), d["tr"].data_ptr(), c.data_ptr(), d["suh"].data_ptr(), a_had.data_ptr(),
+                      d["svh"].data_ptr(), m, Kk, N, bits, Codebook.MUL1, OutDtype.F32, stream)
+
+    want = []
+    for i in range(2):
+        launch(i, None)
+        torch.cuda.synchronize()
+        want.append(work[i][5].cpu().numpy().view(np.uint32).copy())
+    for rep in range(40):
+        for i in range(2):
+            work[i][5].fill_(-1.0)
+        torch.cuda.synchronize()
+        for burst in range(4):
+            launch(0, raw[0])
+            launch(1, raw[1])
+        torch.cuda.synchronize()
+        for i in range(2):
+            assert np.array_equal(work[i][5].cpu().numpy().view(np.uint32), want[i]), (rep, i)
+    for s in streams:
+        rt.stream_free(s)
+    rt.context_free(rt.ctx)

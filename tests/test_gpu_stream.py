@@ -285,7 +285,7 @@ def test_mgemm_host_lists_refuse_what_the_streaming_kernel_does_not_serve():
 
 def test_stale_accumulator_is_reported_and_cleared():
     """Forced from the host: an accumulator word of the streaming kernel is given a contribution
-    count no launch leaves behind.  The launch that meets it writes NaN into that column block
+    count no launch leaves behind.  The launch that meets it leaves that column block unwritten
     and raises the device's fault word; the next launch reports it (and launches nothing), the
     query reads clean afterwards, and the launch after that is back to normal.  Every kernel
     exits by itself."""
@@ -313,10 +313,10 @@ def test_stale_accumulator_is_reported_and_cleared():
     stale = np.array([200], dtype=np.uint64)                       # 200 contributions already "there"
     rt.ok(rt.copy_from_host(None, accum.value + block * 1024, stale.ctypes.data, 8))
     assert K.pending_fault(0) == 0
-    c = torch.zeros(N, dtype=torch.float32, device=DEV)
+    c = torch.full((N,), 555.0, dtype=torch.float32, device=DEV)
     launch(c)                                                       # accepted; every kernel exits
     got = c.cpu().numpy()
-    assert np.isnan(got[block * 128:(block + 1) * 128]).all()
+    assert (got[block * 128:(block + 1) * 128] == 555.0).all()      # nobody could finish the block: left unwritten
     keep = np.ones(N, dtype=bool)
     keep[block * 128:(block + 1) * 128] = False
     assert np.array_equal(got[keep].view(np.uint32), good.cpu().numpy()[keep].view(np.uint32))
