@@ -324,7 +324,7 @@ def moe_plan_bytes(H: int, E: int, k: int, I: int, bits: int, shared_I: int = 0)
     listed = P.TensorBytes(tensors)
     placed = P.place(P.build_plan(shape), listed)
     pool = sum(b for n, b in listed.tensors if P.is_routed_expert(n))
-    return listed.total() - pool, pool, placed.bytes_moved.vram
+    return listed.total() - pool, pool, placed.bytes_moved
 
 
 def moe_bench(gpu, steps: int, warmup: int):

@@ -198,14 +198,14 @@ static int run_ckpt_plan(const std::string& ckpt_dir)
     const berth::exl3::Checkpoint ckpt = berth::exl3::Checkpoint::open(ckpt_dir);
     const plan::ModelPlan model = plan::build_plan(plan::model_shape(ckpt.config));
     const plan::TensorBytes bytes = plan::tensor_bytes(ckpt);
-    const plan::Placement placed = plan::place(model, bytes, plan::MachineBudget::mi355x());
+    const plan::Placement placed = plan::place(model, bytes, plan::HbmBudget{});
     size_t moe_layers = 0, expert_tensors = 0;
     for (const plan::LayerPlan& l : model.layers) moe_layers += l.ffn.is_moe ? 1 : 0;
-    for (const plan::PlacedTensor& t : placed.tensors) expert_tensors += plan::is_routed_expert(t.name) ? 1 : 0;
-    std::printf("plan arch=%s layers=%zu moe_layers=%zu tensors=%zu expert_tensors=%zu resident_vram=%llu "
-                "bytes_moved_vram=%llu\n",
-                model.arch_string.c_str(), model.layers.size(), moe_layers, placed.tensors.size(), expert_tensors,
-                (unsigned long long)placed.resident.vram, (unsigned long long)placed.bytes_moved.vram);
+    for (const auto& t : bytes.tensors) expert_tensors += plan::is_routed_expert(t.first) ? 1 : 0;
+    std::printf("plan arch=%s layers=%zu moe_layers=%zu tensors=%zu expert_tensors=%zu resident=%llu "
+                "bytes_moved=%llu\n",
+                model.arch_string.c_str(), model.layers.size(), moe_layers, bytes.tensors.size(), expert_tensors,
+                (unsigned long long)placed.resident, (unsigned long long)placed.bytes_moved);
     if (moe_layers) {
         const plan::Ffn& f = model.layers[0].ffn;
         std::printf("ffn router=%u/%u shared=%u experts=%u/%u/%u\n", f.router.num_experts, f.router.experts_per_tok,

@@ -5,10 +5,11 @@
 //                                         crates/berth-plan/src/plan.rs:10-267
 //   is_routed_expert / place / bytes_moved crates/berth-plan/src/place.rs:175-376
 //   model_shape / tensor_bytes            crates/berth-plan/src/from_exl3/{shape,bytes}.rs
-// Same rules, same error texts.  The default budget is one MI355X (288 GiB of HBM,
-// no pinned-RAM tier): every tensor lands in VRAM, and what remains of `place` is the
-// accounting - above all bytes_moved, the bytes one decoded token reads, which is the
-// algorithmic-bytes figure the MoE measurements are priced with.
+// Same rules, same error texts for the shape and the plan.  The reference's placement over
+// VRAM, pinned RAM and SSD is collapsed: one MI355X holds the whole weight set in its 288 GiB
+// of HBM, so `place` only checks that it fits beside the reservation and does the accounting,
+// above all bytes_moved, the bytes one decoded token reads, which is the algorithmic-bytes
+// figure the MoE measurements are priced with.
 // Header-only, host only.
 #pragma once
 
@@ -34,8 +35,8 @@ public:
         // plan.rs:115-125
         NotYet = 20, Unknown,
         // place.rs:126-173
-        EmptyName = 40, DuplicateTensor, Overflow, ReservationExceedsVram, DenseExceedsVram, BackboneExceedsVram,
-        ExpertsExceedPinnedRam, InconsistentMoe, InvalidMoe,
+        EmptyName = 40, DuplicateTensor, Overflow, ReservationExceedsHbm, WeightsExceedHbm,
+        InconsistentMoe = 47, InvalidMoe,
         // from_exl3/shape.rs:12-24
         UnknownLayerType = 60, IncompleteMoe,
     };
@@ -209,40 +210,23 @@ inline ModelPlan build_plan(const ModelShape& shape)
 // ------------------------------------------------------------------------------------------
 // placement
 
-enum class Berth : int { Vram = 0, PinnedRam = 1, Ssd = 2 };                // place.rs:19-35
-
 constexpr uint64_t kMi355xHbmBytes = 288ull << 30;
 
-struct MachineBudget {                                                      // place.rs:39-61
-    uint64_t vram_bytes = kMi355xHbmBytes;
-    uint64_t pinned_ram_bytes = 0;       // no host tier: what does not fit in HBM is an error
-    uint64_t vram_reserved_bytes = 0;    // KV cache, activations, workspaces
-    static MachineBudget mi355x(uint64_t reserved = 0) { return MachineBudget{kMi355xHbmBytes, 0, reserved}; }
+// what the weights may take of the device: its HBM less what the caller keeps for the KV
+// cache, activations and workspaces (the role of MachineBudget, place.rs:39-61, with its
+// pinned-RAM tier gone)
+struct HbmBudget {
+    uint64_t hbm_bytes = kMi355xHbmBytes;
+    uint64_t reserved_bytes = 0;
 };
 
 struct TensorBytes {                                                        // place.rs:71-79
     std::vector<std::pair<std::string, uint64_t>> tensors;
 };
 
-struct PlacedTensor {                                                       // place.rs:83-87
-    std::string name;
-    uint64_t bytes = 0;
-    Berth berth = Berth::Vram;
-};
-
-struct BerthBytes {                                                         // place.rs:91-107
-    uint64_t vram = 0, pinned_ram = 0, ssd = 0;
-    void add(Berth b, uint64_t bytes)
-    {
-        uint64_t& slot = b == Berth::Vram ? vram : b == Berth::PinnedRam ? pinned_ram : ssd;
-        if (__builtin_add_overflow(slot, bytes, &slot)) throw Error(Error::Kind::Overflow, "tensor byte sizes overflow u64");
-    }
-};
-
-struct Placement {                                                          // place.rs:111-122
-    std::vector<PlacedTensor> tensors;   // input order
-    BerthBytes resident;                 // bytes held per berth
-    BerthBytes bytes_moved;              // bytes one decoded token reads per berth
+struct Placement {                                                          // place.rs:111-122, one berth
+    uint64_t resident = 0;               // bytes held in HBM: every listed tensor
+    uint64_t bytes_moved = 0;            // bytes one decoded token reads
 };
 
 // a tensor belongs to the routed expert pool when one dot-separated segment of its name is
@@ -315,15 +299,6 @@ uint64_t sum_bytes(const std::vector<Classed>& classed, Keep keep)          // p
     return total;
 }
 
-template <typename BerthOf, typename Keep>
-BerthBytes tally(const std::vector<Classed>& classed, BerthOf berth_of, Keep keep)    // place.rs:331-343
-{
-    BerthBytes out;
-    for (const Classed& t : classed)
-        if (keep(t)) out.add(berth_of(t), t.bytes);
-    return out;
-}
-
 // bytes * per_tok / num_experts in 128 bits, truncated once (place.rs:367-376)
 inline uint64_t portion(uint64_t bytes, uint32_t per_tok, uint32_t num_experts)
 {
@@ -333,64 +308,37 @@ inline uint64_t portion(uint64_t bytes, uint32_t per_tok, uint32_t num_experts)
     return (uint64_t)moved;
 }
 
-// dense: every listed tensor is read once per token.  MoE: the backbone plus a top-k slice of
-// the expert pool, summed per berth and scaled once (place.rs:345-365)
-template <typename BerthOf>
-BerthBytes moved_bytes(const std::vector<Classed>& classed, BerthOf berth_of,
-                       const std::optional<std::pair<uint32_t, uint32_t>>& ratio)
-{
-    if (!ratio) return tally(classed, berth_of, [](const Classed&) { return true; });
-    BerthBytes backbone = tally(classed, berth_of, [](const Classed& t) { return !t.expert; });
-    const BerthBytes experts = tally(classed, berth_of, [](const Classed& t) { return t.expert; });
-    backbone.add(Berth::Vram, portion(experts.vram, ratio->first, ratio->second));
-    backbone.add(Berth::PinnedRam, portion(experts.pinned_ram, ratio->first, ratio->second));
-    backbone.add(Berth::Ssd, portion(experts.ssd, ratio->first, ratio->second));
-    return backbone;
-}
-
-template <typename BerthOf>
-Placement pack(const std::vector<Classed>& classed, BerthOf berth_of,
-               const std::optional<std::pair<uint32_t, uint32_t>>& ratio)   // place.rs:306-329
-{
-    Placement p;
-    p.resident = tally(classed, berth_of, [](const Classed&) { return true; });
-    p.bytes_moved = moved_bytes(classed, berth_of, ratio);
-    p.tensors.reserve(classed.size());
-    for (const Classed& t : classed) p.tensors.push_back(PlacedTensor{t.name, t.bytes, berth_of(t)});
-    return p;
-}
-
 }  // namespace detail
 
-// place.rs:189-232.  Everything in VRAM when it fits beside the reservation; otherwise a MoE
-// plan moves its whole expert pool to pinned RAM (when the budget has any), a dense plan fails.
-inline Placement place(const ModelPlan& plan, const TensorBytes& bytes, const MachineBudget& budget = MachineBudget{})
+// place.rs:189-232 with one berth: everything is resident in HBM or the call fails.
+// bytes_moved (place.rs:345-365): a dense plan reads every listed tensor once per token; a MoE
+// plan reads the backbone plus experts_per_tok / num_experts of the routed-expert pool.
+inline Placement place(const ModelPlan& plan, const TensorBytes& bytes, const HbmBudget& budget = HbmBudget{})
 {
     using K = Error::Kind;
     auto n = [](uint64_t v) { return std::to_string(v); };
-    if (budget.vram_reserved_bytes > budget.vram_bytes)
-        throw Error(K::ReservationExceedsVram, "VRAM reservation of " + n(budget.vram_reserved_bytes) +
-                                                   " bytes exceeds the VRAM budget of " + n(budget.vram_bytes) + " bytes");
-    const uint64_t available = budget.vram_bytes - budget.vram_reserved_bytes;
+    if (budget.reserved_bytes > budget.hbm_bytes)
+        throw Error(K::ReservationExceedsHbm, "HBM reservation of " + n(budget.reserved_bytes) +
+                                                  " bytes exceeds the HBM budget of " + n(budget.hbm_bytes) + " bytes");
     const std::vector<detail::Classed> classed = detail::classify(bytes);
     const auto ratio = detail::moe_ratio(plan);
-    const uint64_t total = detail::sum_bytes(classed, [](const detail::Classed&) { return true; });
-    if (total <= available) return detail::pack(classed, [](const detail::Classed&) { return Berth::Vram; }, ratio);
-    if (!ratio)
-        throw Error(K::DenseExceedsVram, "dense weights (" + n(total) + " bytes) plus the VRAM reservation (" +
-                                             n(budget.vram_reserved_bytes) + " bytes) exceed VRAM (" +
-                                             n(budget.vram_bytes) + " bytes)");
     const uint64_t backbone = detail::sum_bytes(classed, [](const detail::Classed& t) { return !t.expert; });
     const uint64_t experts = detail::sum_bytes(classed, [](const detail::Classed& t) { return t.expert; });
-    if (backbone > available)
-        throw Error(K::BackboneExceedsVram, "backbone (" + n(backbone) + " bytes) plus the VRAM reservation (" +
-                                                n(budget.vram_reserved_bytes) + " bytes) exceed VRAM (" +
-                                                n(budget.vram_bytes) + " bytes)");
-    if (experts > budget.pinned_ram_bytes)
-        throw Error(K::ExpertsExceedPinnedRam, "routed experts (" + n(experts) + " bytes) exceed pinned RAM (" +
-                                                   n(budget.pinned_ram_bytes) +
-                                                   " bytes); SSD placement is not implemented");
-    return detail::pack(classed, [](const detail::Classed& t) { return t.expert ? Berth::PinnedRam : Berth::Vram; }, ratio);
+    uint64_t total = 0;
+    if (__builtin_add_overflow(backbone, experts, &total)) throw Error(K::Overflow, "tensor byte sizes overflow u64");
+    if (total > budget.hbm_bytes - budget.reserved_bytes)
+        throw Error(K::WeightsExceedHbm, "weights (" + n(total) + " bytes) plus the HBM reservation (" +
+                                             n(budget.reserved_bytes) + " bytes) exceed HBM (" + n(budget.hbm_bytes) +
+                                             " bytes); this build keeps every tensor resident");
+    Placement p;
+    p.resident = total;
+    p.bytes_moved = total;
+    if (ratio) {
+        p.bytes_moved = backbone;
+        if (__builtin_add_overflow(p.bytes_moved, detail::portion(experts, ratio->first, ratio->second), &p.bytes_moved))
+            throw Error(K::Overflow, "tensor byte sizes overflow u64");
+    }
+    return p;
 }
 
 // ------------------------------------------------------------------------------------------

@@ -70,22 +70,15 @@ ModelShape shape_of(const berth_plan_shape& in)
     return s;
 }
 
-void copy_out(const BerthBytes& b, berth_plan_berth_bytes* out)
-{
-    if (out) *out = berth_plan_berth_bytes{b.vram, b.pinned_ram, b.ssd};
-}
-
-int place_list(const berth_plan* plan, const TensorBytes& list, const berth_plan_budget* budget, int* berths,
-               berth_plan_berth_bytes* resident, berth_plan_berth_bytes* bytes_moved)
+int place_list(const berth_plan* plan, const TensorBytes& list, const berth_plan_budget* budget, uint64_t* resident,
+               uint64_t* bytes_moved)
 {
     return guarded([&] {
-        MachineBudget b;
-        if (budget) b = MachineBudget{budget->vram_bytes, budget->pinned_ram_bytes, budget->vram_reserved_bytes};
+        HbmBudget b;
+        if (budget) b = HbmBudget{budget->hbm_bytes, budget->reserved_bytes};
         const Placement placed = place(plan->plan, list, b);
-        if (berths)
-            for (size_t i = 0; i < placed.tensors.size(); ++i) berths[i] = (int)placed.tensors[i].berth;
-        copy_out(placed.resident, resident);
-        copy_out(placed.bytes_moved, bytes_moved);
+        if (resident) *resident = placed.resident;
+        if (bytes_moved) *bytes_moved = placed.bytes_moved;
     });
 }
 
@@ -191,16 +184,13 @@ int berth_plan_layer_at(const berth_plan* plan, size_t i, berth_plan_layer* out)
 
 int berth_plan_is_routed_expert(const char* name) { return name && is_routed_expert(name) ? 1 : 0; }
 
-void berth_plan_budget_mi355x(uint64_t vram_reserved_bytes, berth_plan_budget* out)
+void berth_plan_budget_mi355x(uint64_t reserved_bytes, berth_plan_budget* out)
 {
-    if (!out) return;
-    const MachineBudget b = MachineBudget::mi355x(vram_reserved_bytes);
-    *out = berth_plan_budget{b.vram_bytes, b.pinned_ram_bytes, b.vram_reserved_bytes};
+    if (out) *out = berth_plan_budget{kMi355xHbmBytes, reserved_bytes};
 }
 
 int berth_plan_place(const berth_plan* plan, const char* const* names, const uint64_t* bytes, size_t n,
-                     const berth_plan_budget* budget, int* berths, berth_plan_berth_bytes* resident,
-                     berth_plan_berth_bytes* bytes_moved)
+                     const berth_plan_budget* budget, uint64_t* resident, uint64_t* bytes_moved)
 {
     if (!plan || (n && (!names || !bytes))) return fail(BERTH_PLAN_ARGUMENT, "berth_plan_place: null argument");
     TensorBytes list;
@@ -208,7 +198,7 @@ int berth_plan_place(const berth_plan* plan, const char* const* names, const uin
         if (!names[i]) return fail(BERTH_PLAN_ARGUMENT, "berth_plan_place: null tensor name");
         list.tensors.emplace_back(names[i], bytes[i]);
     }
-    return place_list(plan, list, budget, berths, resident, bytes_moved);
+    return place_list(plan, list, budget, resident, bytes_moved);
 }
 
 int berth_plan_tensor_bytes(const berth_ckpt* ckpt, berth_plan_bytes** out)
@@ -234,10 +224,10 @@ int berth_plan_bytes_at(const berth_plan_bytes* list, size_t i, const char** nam
 }
 
 int berth_plan_place_bytes(const berth_plan* plan, const berth_plan_bytes* list, const berth_plan_budget* budget,
-                           int* berths, berth_plan_berth_bytes* resident, berth_plan_berth_bytes* bytes_moved)
+                           uint64_t* resident, uint64_t* bytes_moved)
 {
     if (!plan || !list) return fail(BERTH_PLAN_ARGUMENT, "berth_plan_place_bytes: null argument");
-    return place_list(plan, list->list, budget, berths, resident, bytes_moved);
+    return place_list(plan, list->list, budget, resident, bytes_moved);
 }
 
 }  // extern "C"

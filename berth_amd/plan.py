@@ -1,7 +1,8 @@
 """ctypes binding of the model planner in libberth_exl3_reader.so, shaped like the
 reference's `berth_plan` crate (crates/berth-plan/src/lib.rs): `ModelShape`,
 `MoeDims`, `build_plan` -> `ModelPlan` with an `Ffn` per layer, `TensorBytes`,
-`MachineBudget`, `place` -> `Placement` with `resident` and `bytes_moved`,
+`HbmBudget`, `place` -> `Placement` with `resident` and `bytes_moved` (one berth: the
+reference's VRAM / pinned RAM / SSD tiers are collapsed into "resident in HBM"),
 `is_routed_expert`, and the checkpoint adapters `model_shape` / `tensor_bytes`.
 Every rule and check runs in the C++ library; this file copies records in and out.
 """
@@ -37,10 +38,8 @@ class ErrorKind(enum.IntEnum):
     EMPTY_NAME = 40
     DUPLICATE_TENSOR = 41
     OVERFLOW = 42
-    RESERVATION_EXCEEDS_VRAM = 43
-    DENSE_EXCEEDS_VRAM = 44
-    BACKBONE_EXCEEDS_VRAM = 45
-    EXPERTS_EXCEED_PINNED_RAM = 46
+    RESERVATION_EXCEEDS_HBM = 43
+    WEIGHTS_EXCEED_HBM = 44
     INCONSISTENT_MOE = 47
     INVALID_MOE = 48
     UNKNOWN_LAYER_TYPE = 60
@@ -76,13 +75,6 @@ class Mixer(enum.IntEnum):
     GDN = 0
     FULL_ATTN = 1
     QSA = 2
-
-
-class Berth(enum.IntEnum):
-    """place.rs:19-35."""
-    VRAM = 0
-    PINNED_RAM = 1
-    SSD = 2
 
 
 @dataclasses.dataclass(frozen=True)
@@ -164,41 +156,26 @@ class LayerPlan:
 
 
 @dataclasses.dataclass(frozen=True)
-class MachineBudget:
-    """place.rs:39-61; the default is one MI355X: 288 GiB of HBM and no pinned-RAM tier."""
-    vram_bytes: int = MI355X_HBM_BYTES
-    pinned_ram_bytes: int = 0
-    vram_reserved_bytes: int = 0
+class HbmBudget:
+    """What the weights may take of the device: its HBM less the caller's reservation (the
+    role of MachineBudget, place.rs:39-61, with the pinned-RAM tier gone).  The default is one
+    MI355X: 288 GiB."""
+    hbm_bytes: int = MI355X_HBM_BYTES
+    reserved_bytes: int = 0
 
     @classmethod
-    def mi355x(cls, vram_reserved_bytes: int = 0) -> "MachineBudget":
+    def mi355x(cls, reserved_bytes: int = 0) -> "HbmBudget":
         b = _Budget()
-        _load().berth_plan_budget_mi355x(vram_reserved_bytes, C.byref(b))
-        return cls(int(b.vram_bytes), int(b.pinned_ram_bytes), int(b.vram_reserved_bytes))
-
-
-@dataclasses.dataclass(frozen=True)
-class BerthBytes:
-    """place.rs:91-107."""
-    vram: int = 0
-    pinned_ram: int = 0
-    ssd: int = 0
-
-
-@dataclasses.dataclass(frozen=True)
-class PlacedTensor:
-    """place.rs:83-87."""
-    name: str
-    bytes: int
-    berth: Berth
+        _load().berth_plan_budget_mi355x(reserved_bytes, C.byref(b))
+        return cls(int(b.hbm_bytes), int(b.reserved_bytes))
 
 
 @dataclasses.dataclass(frozen=True)
 class Placement:
-    """place.rs:111-122."""
-    tensors: list
-    resident: BerthBytes
-    bytes_moved: BerthBytes
+    """place.rs:111-122 with one berth: `resident` bytes held in HBM (every listed tensor),
+    `bytes_moved` bytes one decoded token reads."""
+    resident: int
+    bytes_moved: int
 
 
 class TensorBytes:
@@ -240,11 +217,7 @@ class _Summary(C.Structure):
 
 
 class _Budget(C.Structure):
-    _fields_ = [(n, C.c_uint64) for n in ("vram_bytes", "pinned_ram_bytes", "vram_reserved_bytes")]
-
-
-class _BerthBytes(C.Structure):
-    _fields_ = [(n, C.c_uint64) for n in ("vram", "pinned_ram", "ssd")]
+    _fields_ = [(n, C.c_uint64) for n in ("hbm_bytes", "reserved_bytes")]
 
 
 _bound = False
@@ -268,15 +241,14 @@ def _load() -> C.CDLL:
         L.berth_plan_budget_mi355x.argtypes = [u64, C.POINTER(_Budget)]
         L.berth_plan_budget_mi355x.restype = None
         L.berth_plan_place.argtypes = [vp, C.POINTER(C.c_char_p), C.POINTER(u64), sz, C.POINTER(_Budget),
-                                       C.POINTER(C.c_int), C.POINTER(_BerthBytes), C.POINTER(_BerthBytes)]
+                                       C.POINTER(u64), C.POINTER(u64)]
         L.berth_plan_tensor_bytes.argtypes = [vp, C.POINTER(vp)]
         L.berth_plan_bytes_free.argtypes = [vp]
         L.berth_plan_bytes_free.restype = None
         L.berth_plan_bytes_count.argtypes = [vp]
         L.berth_plan_bytes_count.restype = sz
         L.berth_plan_bytes_at.argtypes = [vp, sz, C.POINTER(C.c_char_p), C.POINTER(u64)]
-        L.berth_plan_place_bytes.argtypes = [vp, vp, C.POINTER(_Budget), C.POINTER(C.c_int), C.POINTER(_BerthBytes),
-                                             C.POINTER(_BerthBytes)]
+        L.berth_plan_place_bytes.argtypes = [vp, vp, C.POINTER(_Budget), C.POINTER(u64), C.POINTER(u64)]
         _bound = True
     return L
 
@@ -404,16 +376,12 @@ def is_routed_expert(name: str) -> bool:
     return bool(_load().berth_plan_is_routed_expert(name.encode()))
 
 
-def place(plan: ModelPlan, weights: TensorBytes, budget: MachineBudget = MachineBudget()) -> Placement:
-    """place.rs:189-232; `bytes_moved` follows place.rs:345-376."""
+def place(plan: ModelPlan, weights: TensorBytes, budget: HbmBudget = HbmBudget()) -> Placement:
+    """place.rs:189-232 with one berth; `bytes_moved` follows place.rs:345-376."""
     n = len(weights.tensors)
     names = (C.c_char_p * max(1, n))(*[name.encode() for name, _ in weights.tensors])
     sizes = (C.c_uint64 * max(1, n))(*[size for _, size in weights.tensors])
-    berths = (C.c_int * max(1, n))()
-    b = _Budget(budget.vram_bytes, budget.pinned_ram_bytes, budget.vram_reserved_bytes)
-    resident, moved = _BerthBytes(), _BerthBytes()
-    _check(_load().berth_plan_place(plan._handle, names, sizes, n, C.byref(b), berths, C.byref(resident),
-                                    C.byref(moved)))
-    tensors = [PlacedTensor(name, size, Berth(berths[i])) for i, (name, size) in enumerate(weights.tensors)]
-    return Placement(tensors, BerthBytes(int(resident.vram), int(resident.pinned_ram), int(resident.ssd)),
-                     BerthBytes(int(moved.vram), int(moved.pinned_ram), int(moved.ssd)))
+    b = _Budget(budget.hbm_bytes, budget.reserved_bytes)
+    resident, moved = C.c_uint64(), C.c_uint64()
+    _check(_load().berth_plan_place(plan._handle, names, sizes, n, C.byref(b), C.byref(resident), C.byref(moved)))
+    return Placement(int(resident.value), int(moved.value))

@@ -1,8 +1,10 @@
 /*
  * berth_plan.h — C ABI of the model planner in libberth_exl3_reader.so: model
  * shape -> per-layer plan (which layers carry a dense MLP, which a MoE block of
- * router + shared expert + routed experts) -> placement and the bytes one
- * decoded token reads.  Host only; no device call is made.
+ * router + shared expert + routed experts) -> the bytes resident in HBM and the
+ * bytes one decoded token reads.  The reference's three-tier placement (VRAM,
+ * pinned RAM, SSD) is collapsed: one MI355X keeps the whole weight set in HBM.
+ * Host only; no device call is made.
  *
  * The reference plans with a Rust crate (crates/berth-plan) that has no foreign
  * interface; this header is the surface a non-Rust host uses for the same
@@ -32,8 +34,7 @@ enum {
     BERTH_PLAN_UNEXPECTED_MOE = 4, BERTH_PLAN_MISSING_MOE = 5, BERTH_PLAN_ZERO = 6, BERTH_PLAN_EXPERTS_PER_TOK = 7,
     BERTH_PLAN_NOT_YET = 20, BERTH_PLAN_UNKNOWN_ARCH = 21,
     BERTH_PLAN_EMPTY_NAME = 40, BERTH_PLAN_DUPLICATE_TENSOR = 41, BERTH_PLAN_OVERFLOW = 42,
-    BERTH_PLAN_RESERVATION_EXCEEDS_VRAM = 43, BERTH_PLAN_DENSE_EXCEEDS_VRAM = 44,
-    BERTH_PLAN_BACKBONE_EXCEEDS_VRAM = 45, BERTH_PLAN_EXPERTS_EXCEED_PINNED_RAM = 46,
+    BERTH_PLAN_RESERVATION_EXCEEDS_HBM = 43, BERTH_PLAN_WEIGHTS_EXCEED_HBM = 44,
     BERTH_PLAN_INCONSISTENT_MOE = 47, BERTH_PLAN_INVALID_MOE = 48,
     BERTH_PLAN_UNKNOWN_LAYER_TYPE = 60, BERTH_PLAN_INCOMPLETE_MOE = 61,
     BERTH_PLAN_ARGUMENT = 90
@@ -102,25 +103,20 @@ int berth_plan_layer_at(const berth_plan* plan, size_t i, berth_plan_layer* out)
 /* is_routed_expert (place.rs:175-187): 1 when a dot-separated segment of the name is "experts" */
 int berth_plan_is_routed_expert(const char* name);
 
-/* MachineBudget (place.rs:39-61).  berth_plan_budget_mi355x: 288 GiB of HBM, no pinned-RAM tier. */
+/* What the weights may take of the device (the role of MachineBudget, place.rs:39-61, with
+ * its pinned-RAM tier gone).  berth_plan_budget_mi355x: 288 GiB of HBM. */
 typedef struct {
-    uint64_t vram_bytes, pinned_ram_bytes, vram_reserved_bytes;
+    uint64_t hbm_bytes, reserved_bytes;
 } berth_plan_budget;
-void berth_plan_budget_mi355x(uint64_t vram_reserved_bytes, berth_plan_budget* out);
+void berth_plan_budget_mi355x(uint64_t reserved_bytes, berth_plan_budget* out);
 
-/* BerthBytes (place.rs:91-107) */
-typedef struct {
-    uint64_t vram, pinned_ram, ssd;
-} berth_plan_berth_bytes;
-
-/* place (place.rs:189-232) over n (name, bytes) pairs.  berths[n] (optional) receives 0 VRAM,
- * 1 pinned RAM, 2 SSD per tensor in input order; `resident` the bytes held per berth;
- * `bytes_moved` the bytes one decoded token reads per berth (place.rs:345-376: every tensor for
- * a dense plan; for a MoE plan the backbone plus experts_per_tok / num_experts of the expert
- * pool, scaled once per berth in 128-bit arithmetic). */
+/* place (place.rs:189-232, one berth) over n (name, bytes) pairs: every tensor is resident in
+ * HBM, or the call fails with BERTH_PLAN_WEIGHTS_EXCEED_HBM.  `resident`: the bytes held;
+ * `bytes_moved`: the bytes one decoded token reads (place.rs:345-376: every tensor for a dense
+ * plan; for a MoE plan the backbone plus experts_per_tok / num_experts of the expert pool,
+ * scaled once in 128-bit arithmetic).  budget NULL: one MI355X, nothing reserved. */
 int berth_plan_place(const berth_plan* plan, const char* const* names, const uint64_t* bytes, size_t n,
-                     const berth_plan_budget* budget, int* berths, berth_plan_berth_bytes* resident,
-                     berth_plan_berth_bytes* bytes_moved);
+                     const berth_plan_budget* budget, uint64_t* resident, uint64_t* bytes_moved);
 
 /* tensor_bytes (from_exl3/bytes.rs:57-93): one entry per EXL3 linear (all its parts) and one per
  * other tensor, sorted by name, without the vision tower and the MTP head. */
@@ -131,7 +127,7 @@ size_t berth_plan_bytes_count(const berth_plan_bytes* list);
 int berth_plan_bytes_at(const berth_plan_bytes* list, size_t i, const char** name, uint64_t* bytes);
 /* place() on a list from berth_plan_tensor_bytes */
 int berth_plan_place_bytes(const berth_plan* plan, const berth_plan_bytes* list, const berth_plan_budget* budget,
-                           int* berths, berth_plan_berth_bytes* resident, berth_plan_berth_bytes* bytes_moved);
+                           uint64_t* resident, uint64_t* bytes_moved);
 
 #ifdef __cplusplus
 }

@@ -250,7 +250,7 @@ def test_python_moe_loader_follows_the_plan(request, which, T):
     listed = P.tensor_bytes(ckpt)
     pool = sum(b for n, b in listed.tensors if P.is_routed_expert(n))
     placed = P.place(plan, listed)
-    assert pool > 0 and placed.bytes_moved.vram == listed.total() - pool + pool * MOE_K // MOE_E
+    assert pool > 0 and placed.bytes_moved == listed.total() - pool + pool * MOE_K // MOE_E
     assert not any(n.startswith("model.visual.") for n, _ in listed.tensors)
 
 

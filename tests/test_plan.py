@@ -1,6 +1,6 @@
 """The model planner (berth_amd/csrc/host/plan.hpp through include/berth_plan.h and
 berth_amd/plan.py) against the cases and known answers of the reference's own tests:
-crates/berth-plan/tests/plan.rs (27B dense, 35B MoE, spill, errors, the expert name
+crates/berth-plan/tests/plan.rs (27B dense, 35B MoE, one berth, errors, the expert name
 rule), tests/from_exl3_shape.rs (config -> shape) and tests/from_exl3_bytes.rs
 (checkpoint -> byte list).  Host only."""
 import json
@@ -44,8 +44,8 @@ def bytes_35b():          # tests/plan.rs:96-120: 16.1 + 1.2 + 0.25 GB
     ])
 
 
-def this_machine(reserved):   # the reference's development box (place.rs:12-15): the known answers are quoted on it
-    return P.MachineBudget(24 * GIB, 18 * GIB, reserved)
+def this_machine(reserved):   # the VRAM of the reference's development box (place.rs:12-15): the known answers are quoted on it
+    return P.HbmBudget(24 * GIB, reserved)
 
 
 def mixers(plan):
@@ -72,10 +72,7 @@ def test_27b_dense_plan_and_placement():
     ])
     assert weights.total() == 13_200_000_000
     placed = P.place(plan, weights, this_machine(4_600_000_000))
-    assert all(t.berth == P.Berth.VRAM for t in placed.tensors)
-    assert placed.resident == P.BerthBytes(13_200_000_000, 0, 0)
-    assert placed.bytes_moved == P.BerthBytes(13_200_000_000, 0, 0)
-    assert [t.name for t in placed.tensors] == [n for n, _ in weights.tensors]
+    assert placed == P.Placement(resident=13_200_000_000, bytes_moved=13_200_000_000)
 
 
 def test_35b_moe_plan_and_bytes_moved():
@@ -90,25 +87,26 @@ def test_35b_moe_plan_and_bytes_moved():
         assert layer.ffn.experts == P.RoutedExperts(256, 8, 512)
     weights = bytes_35b()
     assert weights.total() == 17_550_000_000
-    for budget in (this_machine(2_500_000_000), P.MachineBudget.mi355x(2_500_000_000), P.MachineBudget()):
+    for budget in (this_machine(2_500_000_000), P.HbmBudget.mi355x(2_500_000_000), P.HbmBudget()):
         placed = P.place(plan, weights, budget)
-        assert all(t.berth == P.Berth.VRAM for t in placed.tensors)
-        assert placed.resident == P.BerthBytes(17_550_000_000, 0, 0)
         assert 16_100_000_000 * 8 // 256 == 503_125_000
-        assert placed.bytes_moved == P.BerthBytes(1_450_000_000 + 503_125_000, 0, 0)
+        assert placed == P.Placement(resident=17_550_000_000, bytes_moved=1_450_000_000 + 503_125_000)
 
 
-def test_moe_spills_the_expert_pool_to_pinned_ram_when_the_budget_has_one():
-    """tests/plan.rs:248-282."""
+def test_a_pool_that_does_not_fit_hbm_is_an_error_not_a_spill():
+    """The budget of tests/plan.rs:248-282 (8 GB of device memory, where the reference moves the
+    expert pool to pinned RAM): with one berth the same call fails and names the sizes."""
     plan = P.build_plan(shape_35b())
-    placed = P.place(plan, bytes_35b(), P.MachineBudget(8_000_000_000, 18 * GIB, 2_500_000_000))
-    for t in placed.tensors:
-        assert t.berth == (P.Berth.PINNED_RAM if P.is_routed_expert(t.name) else P.Berth.VRAM), t.name
-    assert placed.resident == P.BerthBytes(1_450_000_000, 16_100_000_000, 0)
-    assert placed.bytes_moved == P.BerthBytes(1_450_000_000, 503_125_000, 0)
-    by_name = {t.name: t.berth for t in placed.tensors}
-    assert by_name["model.language_model.layers.0.mlp.shared_expert.down_proj.trellis"] == P.Berth.VRAM
-    assert by_name["model.language_model.layers.0.mlp.gate.weight"] == P.Berth.VRAM
+    with pytest.raises(P.PlanError) as e:
+        P.place(plan, bytes_35b(), P.HbmBudget(8_000_000_000, 2_500_000_000))
+    assert e.value.kind == P.ErrorKind.WEIGHTS_EXCEED_HBM
+    assert str(e.value) == ("weights (17550000000 bytes) plus the HBM reservation (2500000000 bytes) exceed HBM "
+                            "(8000000000 bytes); this build keeps every tensor resident")
+    # the shared expert and the router are backbone: only `experts` names are scaled by k / E
+    names = [n for n, _ in bytes_35b().tensors]
+    assert not P.is_routed_expert("model.language_model.layers.0.mlp.shared_expert.down_proj.trellis")
+    assert not P.is_routed_expert("model.language_model.layers.0.mlp.gate.weight")
+    assert sum(P.is_routed_expert(n) for n in names) == 2
 
 
 def test_later_and_unknown_architectures():
@@ -182,30 +180,24 @@ def test_bad_shapes():
 
 
 def test_overflowing_budgets():
-    """tests/plan.rs:365-406."""
+    """tests/plan.rs:365-406 with one berth: what does not fit beside the reservation is refused."""
     dense = P.build_plan(shape_27b())
     with pytest.raises(P.PlanError) as e:
-        P.place(dense, P.TensorBytes([("lm_head.weight", 13_200_000_000)]),
-                P.MachineBudget(16_000_000_000, 18 * GIB, 4_600_000_000))
-    assert e.value.kind == P.ErrorKind.DENSE_EXCEEDS_VRAM
-    assert str(e.value) == ("dense weights (13200000000 bytes) plus the VRAM reservation (4600000000 bytes) "
-                            "exceed VRAM (16000000000 bytes)")
+        P.place(dense, P.TensorBytes([("lm_head.weight", 13_200_000_000)]), P.HbmBudget(16_000_000_000, 4_600_000_000))
+    assert e.value.kind == P.ErrorKind.WEIGHTS_EXCEED_HBM
+    assert str(e.value) == ("weights (13200000000 bytes) plus the HBM reservation (4600000000 bytes) exceed HBM "
+                            "(16000000000 bytes); this build keeps every tensor resident")
     moe, weights = P.build_plan(shape_35b()), bytes_35b()
     with pytest.raises(P.PlanError) as e:
         P.place(moe, weights, this_machine(24 * GIB + 1))
-    assert e.value.kind == P.ErrorKind.RESERVATION_EXCEEDS_VRAM
+    assert e.value.kind == P.ErrorKind.RESERVATION_EXCEEDS_HBM
+    assert str(e.value) == f"HBM reservation of {24 * GIB + 1} bytes exceeds the HBM budget of {24 * GIB} bytes"
     with pytest.raises(P.PlanError) as e:
-        P.place(moe, weights, P.MachineBudget(3_000_000_000, 18 * GIB, 2_500_000_000))
-    assert e.value.kind == P.ErrorKind.BACKBONE_EXCEEDS_VRAM
-    assert str(e.value) == ("backbone (1450000000 bytes) plus the VRAM reservation (2500000000 bytes) "
-                            "exceed VRAM (3000000000 bytes)")
-    with pytest.raises(P.PlanError) as e:
-        P.place(moe, weights, P.MachineBudget(8_000_000_000, 1_000_000_000, 2_500_000_000))
-    assert e.value.kind == P.ErrorKind.EXPERTS_EXCEED_PINNED_RAM
-    # one MI355X has no pinned tier: a pool that does not fit beside the reservation is an error, not a spill
-    with pytest.raises(P.PlanError) as e:
-        P.place(moe, weights, P.MachineBudget.mi355x(288 * GIB - 10_000_000_000))
-    assert e.value.kind == P.ErrorKind.EXPERTS_EXCEED_PINNED_RAM
+        P.place(moe, weights, P.HbmBudget.mi355x(288 * GIB - 10_000_000_000))
+    assert e.value.kind == P.ErrorKind.WEIGHTS_EXCEED_HBM
+    # exactly full is placed
+    placed = P.place(moe, weights, P.HbmBudget(17_550_000_000 + 7, 7))
+    assert placed.resident == 17_550_000_000
 
 
 def test_placement_input_checks_and_arithmetic():
@@ -219,16 +211,16 @@ def test_placement_input_checks_and_arithmetic():
     assert e.value.kind == P.ErrorKind.DUPLICATE_TENSOR
     big = (1 << 64) - 1
     with pytest.raises(P.PlanError, match="tensor byte sizes overflow u64") as e:
-        P.place(moe, P.TensorBytes([("a", big), ("b", 1)]), P.MachineBudget(big, 0, 0))
+        P.place(moe, P.TensorBytes([("a", big), ("b", 1)]), P.HbmBudget(big, 0))
     assert e.value.kind == P.ErrorKind.OVERFLOW
     # bytes * 8 would not fit 64 bits; the quotient does
-    placed = P.place(moe, P.TensorBytes([("x.experts.w", big - 5), ("y", 5)]), P.MachineBudget(big, 0, 0))
-    assert placed.bytes_moved.vram == 5 + (big - 5) * 8 // 256
+    placed = P.place(moe, P.TensorBytes([("x.experts.w", big - 5), ("y", 5)]), P.HbmBudget(big, 0))
+    assert placed.bytes_moved == 5 + (big - 5) * 8 // 256
     # per-tensor truncation would lose a byte here: 3 tensors of 100 bytes -> 300 * 8 // 256 = 9, not 3 * 3
     placed = P.place(moe, P.TensorBytes([(f"l.{i}.experts.w", 100) for i in range(3)]))
-    assert placed.bytes_moved.vram == 9
+    assert placed.bytes_moved == 9
     # an empty list is a valid placement
-    assert P.place(moe, P.TensorBytes([])).resident == P.BerthBytes()
+    assert P.place(moe, P.TensorBytes([])) == P.Placement(0, 0)
 
 
 def test_routed_expert_name_rule():
@@ -244,9 +236,9 @@ def test_routed_expert_name_rule():
 
 def test_mi355x_budget():
     """The counterpart of tests/plan.rs:432-443 for this build's default machine."""
-    b = P.MachineBudget.mi355x(4)
-    assert (b.vram_bytes, b.pinned_ram_bytes, b.vram_reserved_bytes) == (288 << 30, 0, 4)
-    assert P.MachineBudget() == P.MachineBudget.mi355x(0)
+    b = P.HbmBudget.mi355x(4)
+    assert (b.hbm_bytes, b.reserved_bytes) == (288 << 30, 4)
+    assert P.HbmBudget() == P.HbmBudget.mi355x(0)
 
 
 # ---------------------------------------------------------------------------------------------
@@ -383,7 +375,7 @@ def test_tensor_bytes_sums_owned_parts_keeps_expert_names_and_drops_vision_and_m
     shape = P.model_shape(ckpt)
     shape.arch_string = P.ARCH_QWEN3_5
     placed = P.place(P.build_plan(shape), listed)
-    assert placed.resident.vram == placed.bytes_moved.vram == listed.total()
+    assert placed.resident == placed.bytes_moved == listed.total()
 
 
 # ---------------------------------------------------------------------------------------------
@@ -415,12 +407,12 @@ def test_cpp_plan_of_a_moe_checkpoint(tmp_path):
     assert r.returncode == 0, r.stdout + r.stderr
     backbone, pool = 2048 + 16384 + 512 + 512, 4 * (8192 + 256 + 512)
     assert (f"plan arch={P.ARCH_QWEN3_5_MOE} layers=2 moe_layers=2 tensors=6 expert_tensors=4 "
-            f"resident_vram={backbone + pool} bytes_moved_vram={backbone + pool * 2 // 4}") in r.stdout
+            f"resident={backbone + pool} bytes_moved={backbone + pool * 2 // 4}") in r.stdout
     assert "ffn router=4/2 shared=256 experts=4/2/128" in r.stdout
     # the same through the C interface
     ckpt = exl3.Checkpoint.open(tmp_path)
     placed = P.place(P.build_plan(P.model_shape(ckpt)), P.tensor_bytes(ckpt))
-    assert (placed.resident.vram, placed.bytes_moved.vram) == (backbone + pool, backbone + pool // 2)
+    assert (placed.resident, placed.bytes_moved) == (backbone + pool, backbone + pool // 2)
     # a dense architecture string with MoE keys is refused by the plan, as in the reference
     cfg["architectures"] = [P.ARCH_QWEN3_5]
     U.write_checkpoint(tmp_path, tensors, cfg)
