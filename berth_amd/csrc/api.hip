@@ -82,13 +82,18 @@ bool stream_is_capturing(hipStream_t stream)
 }
 }  // namespace
 
+constexpr int kSameStreamDecay = 32;
+
 LaunchScope::LaunchScope(hipStream_t stream_) : ws(workspace_for_current_device()), stream(stream_)
 {
     if (!knobs().stream_order) return;
     std::lock_guard<std::mutex> lock(g_ws_mu);
     if (ws.have_last && ws.last_stream == stream) {
         // the usual case costs a comparison: no runtime call on the launch path
-        if (ws.multi_stream && ++ws.same_stream_run > 4096) {
+        // An event behind every launch costs the device about 2.7 us per launch, so the mode is
+        // left again after a short run on one stream; the next change of stream then pays one
+        // device-wide wait instead.
+        if (ws.multi_stream && ++ws.same_stream_run > kSameStreamDecay) {
             ws.multi_stream = false;
             ws.event_recorded = false;
         }
@@ -157,7 +162,7 @@ Knobs read_knobs()
     k.gemm_balanced = env_int("BERTH_GEMM_BALANCED", 1);
     k.gemm_rows256 = env_int("BERTH_GEMM_ROWS256", 1);
     k.counter_stride = clamp(env_int("BERTH_COUNTER_STRIDE", 32), 1, 32);
-    k.moe_big_min = env_int("BERTH_MOE_BIG_MIN", 0);
+    k.moe_big_min = env_int("BERTH_MOE_BIG_MIN", 33);
     k.moe_fold_combine = env_int("BERTH_MOE_FOLD_COMBINE", 2);
     k.moe_inline_route = env_int("BERTH_MOE_INLINE_ROUTE", 1);
     k.moe_resolved = env_int("BERTH_MOE_RESOLVED", 1);

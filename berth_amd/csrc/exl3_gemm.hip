@@ -165,9 +165,19 @@ std::string launch_gemm_grouped(const GroupedArgs& g)
     const long tiles = (long)g.max_problems * g.num_lins * nblocks;
     p.cstride = gemm_counter_stride(tiles);
     p.S = gemm_split(ws, tiles, g.size_k / 128, mb);
-    if (g.max_problems > 65535) throw std::runtime_error("moe grouped linear: too many problems");
+    if (g.max_problems + g.max_big > 65535) throw std::runtime_error("moe grouped linear: too many problems");
     std::string desc;
     p.tiles_y = g.max_problems;
+    if (g.max_big > 0) {
+        // both lists in one launch, whole K per workgroup
+        p.big_problems = (const GroupProblem*)g.big_problems;
+        p.num_big = g.num_big;
+        p.max_big = g.max_big;
+        p.S = 1;
+        gemm_bits(p, g.k_bits, g.codebook, mb, g.stream, desc, dim3(nblocks, g.num_lins, g.max_problems + g.max_big));
+        hip_ok(hipGetLastError(), "exl3_gemm_mixed_kernel launch");
+        return desc + " grouped";
+    }
     gemm_bits(p, g.k_bits, g.codebook, mb, g.stream, desc, dim3(nblocks * p.S, g.num_lins, g.max_problems));
     hip_ok(hipGetLastError(), "exl3_gemm_kernel grouped launch");
     return desc + " grouped";

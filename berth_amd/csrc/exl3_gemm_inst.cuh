@@ -53,10 +53,25 @@ static void gemm_launch_wide(const GemmParams& p, hipStream_t stream, std::strin
            " smem=" + std::to_string(kWideSmem);
 }
 
+// two problem lists in one grouped launch: 128-row problems first, 32-row problems behind them
+template <int BITS, int CB>
+static void gemm_launch_mixed(const GemmParams& p, hipStream_t stream, std::string& desc, dim3 grid)
+{
+    const size_t smem = (size_t)2 * 128 * kAStride * sizeof(_Float16);
+    static bool raised[64] = {};
+    raise_dynamic_lds_limit((const void*)exl3_gemm_mixed_kernel<BITS, CB>, (int)smem, raised,
+                            "exl3_gemm_mixed_kernel shared-memory attribute");
+    hipLaunchKernelGGL((exl3_gemm_mixed_kernel<BITS, CB>), grid, dim3(256), smem, stream, p);
+    desc = "exl3_gemm_mixed_kernel<" + std::to_string(BITS) + "," + std::to_string(CB) + ",128x256+32x256> grid=" +
+           std::to_string(grid.x) + "x" + std::to_string(grid.y) + "x(" + std::to_string(p.max_big) + "+" +
+           std::to_string(grid.z - p.max_big) + ") smem=" + std::to_string(smem);
+}
+
 template <int BITS, int CB>
 static void gemm_launch(const GemmParams& p, int mb, hipStream_t stream, std::string& desc, dim3 grid)
 {
-    if (mb == 1) gemm_launch_mb<BITS, CB, 1>(p, stream, desc, grid);
+    if (p.max_big > 0) gemm_launch_mixed<BITS, CB>(p, stream, desc, grid);
+    else if (mb == 1) gemm_launch_mb<BITS, CB, 1>(p, stream, desc, grid);
     else if (mb == 8) gemm_launch_wide<BITS, CB>(p, stream, desc, grid);
     else gemm_launch_mb<BITS, CB, 4>(p, stream, desc, grid);
 }

@@ -43,6 +43,11 @@ struct GemmParams {
     int lins_per_expert, lin_base;
     ExpertLin shared[3];        // an always-on expert passed by value (problem.expert == shared_expert)
     int shared_expert;
+    // mixed grouped launches (exl3_gemm_mixed_kernel): problems of up to 128 rows, whose units
+    // of work come first; those of `problems` follow
+    const GroupProblem* big_problems;
+    const int* num_big;
+    int max_big;
     int tiles_y;                // dense: row blocks; grouped: capacity of the problem list
     int tile0;                  // dense: first (row block, column block) tile of this launch, row-major
     // split-K
@@ -91,7 +96,7 @@ constexpr int kAStride = 128 + 8;   // halves per LDS row of the A tile (272 B: 
 // one output tile: rows of problem / row block `tile_y`, 256 columns
 template <int BITS, int CB, int MB, bool DENSE>  // MB = 32-row blocks per workgroup; DENSE: never a problem list
 __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y, const int nblk, const KRange kr,
-                                          const int which, unsigned char* smem)
+                                          const int which, unsigned char* smem, const GroupProblem* problems = nullptr)
 {
     constexpr int BM = MB * 32;
     _Float16* a_tile = (_Float16*)smem;                 // [2][BM][kAStride]
@@ -112,7 +117,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
     if constexpr (!DENSE) {
         // (dynamic indexing of the parameter block: kept out of the dense instantiations, where
         // it would force the whole block into private memory)
-        const GroupProblem gp = p.problems[tile_y];
+        const GroupProblem gp = problems[tile_y];
         lin = gp.expert == p.shared_expert ? p.shared[p.lin_base + which]
                                            : p.experts[gp.expert * p.lins_per_expert + p.lin_base + which];
         m0 = gp.row0;
@@ -463,7 +468,38 @@ __global__ __launch_bounds__(256, 2) void exl3_gemm_kernel(GemmParams p)
     // grouped: (linear, problem, column block)
     kr.counter = ((size_t)blockIdx.y * p.tiles_y + blockIdx.z) * nblocks + unit;
     kr.slot0 = kr.counter * p.S;
-    gemm_tile<BITS, CB, MB, false>(p, blockIdx.z, unit, kr, blockIdx.y, smem);
+    gemm_tile<BITS, CB, MB, false>(p, blockIdx.z, unit, kr, blockIdx.y, smem, p.problems);
+}
+
+// Grouped launch over two problem lists at once: blockIdx.z < max_big takes a problem of up
+// to 128 rows (weights decoded once for all of them, so an expert with many rows costs one
+// decode per 128 rows instead of one per 32), the values after that the problems of up to 32
+// rows.  Both kinds sit in one launch, the long tiles first, so the short ones fill in around
+// them (as two launches the 128-row tiles would run alone on a fraction of the compute units).
+// blockIdx.x = column block (whole K per workgroup: no hand-over), blockIdx.y the linear.
+// Measured and dropped: cutting K in two with the split-K hand-over (the shorter units pack
+// better, the hand-over costs more than that gains), and resident workgroups that take units
+// from a counter (the same schedule as the hardware's, with slower code).
+template <int BITS, int CB>
+__global__ __launch_bounds__(256, 2) void exl3_gemm_mixed_kernel(GemmParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    KRange kr;
+    kr.kb0 = 0;
+    kr.kb1 = p.K >> 7;
+    kr.step = 1;
+    kr.part = 0;
+    kr.parts = 1;
+    kr.counter = 0;
+    kr.slot0 = 0;
+    const int z = blockIdx.z;
+    if (z < p.max_big) {
+        if (z >= *p.num_big) return;
+        gemm_tile<BITS, CB, 4, false>(p, z, blockIdx.x, kr, blockIdx.y, smem, p.big_problems);
+        return;
+    }
+    if (z - p.max_big >= *p.num_problems) return;
+    gemm_tile<BITS, CB, 1, false>(p, z - p.max_big, blockIdx.x, kr, blockIdx.y, smem, p.problems);
 }
 
 // Dense launches whose tile count does not divide over the compute units: the

@@ -105,8 +105,9 @@ Workspace& workspace_for_current_device();
 // counters.  LaunchScope, held by a launcher around its launches, sees to that without ever
 // touching the previous stream's handle (its owner may have destroyed it): the first time the
 // stream changes the device is drained once; from then on every scope records an event behind
-// its launches and a launch on another stream waits for that event.  After 4096 launches in
-// a row on one stream the events stop again, so a single-stream caller pays nothing.  Streams
+// its launches and a launch on another stream waits for that event.  After 32 launches in
+// a row on one stream the events stop again (each costs the device about 2.7 us), so a
+// single-stream caller pays nothing and a rare change of stream pays one drain.  Streams
 // that are being captured into a graph are left alone.
 struct LaunchScope {
     explicit LaunchScope(hipStream_t stream);
@@ -177,6 +178,11 @@ struct GroupedArgs {
     const void* problems;       // GroupProblem[max_problems]
     const int* num_problems;
     int max_problems;
+    // MFMA path, optional: problems of up to 128 rows that run in the same launch, ahead of
+    // `problems` (which then hold at most 32 rows each)
+    const void* big_problems = nullptr;
+    const int* num_big = nullptr;
+    int max_big = 0;
     int lins_per_expert, lin_base, num_lins;   // num_lins 1 or 2 consecutive linears per launch
     void* c0;
     void* c1;

@@ -493,66 +493,145 @@ struct HadRowsParams {
     ExpertLin shared[3];        // the always-on expert (row_expert == shared_expert)
     int shared_expert;
     int lins_per_expert, lin_base;
-    _Float16* out[2];           // per blockIdx.z
+    int num_lins;               // 1 or 2: the same input rotated under the scales of linear lin_base (+ 1)
+    _Float16* out[2];           // per linear
     int P, K;
 };
 
+// An item is one 128 block of one row; sixteen lanes (one DPP row) rotate it, eight consecutive
+// elements per lane (16-byte accesses).  A lane group takes kHadItems consecutive items and
+// issues each step's loads for all of them before the first is used (row -> expert and source
+// row -> scale pointer -> values: three dependent reads, paid once per group instead of once
+// per workgroup), and the input is read once for both linears.
+constexpr int kHadItems = 4;
+
 __global__ __launch_bounds__(256) void moe_had_rows_kernel(HadRowsParams p)
 {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int r = blockIdx.x;
-    const int which = blockIdx.y;
-    const int ex = p.row_expert[r];
-    const ExpertLin lin = ex == p.shared_expert ? p.shared[p.lin_base + which]
-                                                : p.experts[ex * p.lins_per_expert + p.lin_base + which];
-    const int src = p.gather ? p.gather[r] / p.gather_div : r;
-    const _Float16* xrow = p.a + (size_t)src * p.K;
-    const _Float16* urow = p.a_up ? p.a_up + (size_t)src * p.K : nullptr;
-    const _Float16* srow = lin.suh;
-    _Float16* orow = p.out[which] + (size_t)r * p.K;
-    // sixteen lanes per 128 block, eight consecutive elements per lane (16-byte accesses): the
-    // workgroup rotates sixteen blocks at a time
+    const int lane = threadIdx.x & 63;
     const int l16 = lane & 15;
     const int nkb = p.K >> 7;
-    for (int kb0 = 0; kb0 < nkb; kb0 += 16) {
-        const int kb = kb0 + wave * 4 + (lane >> 4);
-        const bool live = kb < nkb;
-        const int at = (live ? kb : nkb - 1) * 128 + 8 * l16;   // lanes past the end redo the last block, store nothing
-        half8_t x = *(const half8_t*)(xrow + at);
-        if (urow) {
-            const half8_t u = *(const half8_t*)(urow + at);
+    const int total = p.P * nkb;
+    const int first = (blockIdx.x * 16 + (threadIdx.x >> 4)) * kHadItems;
+    int row[kHadItems], at[kHadItems], ex[kHadItems], src[kHadItems];
+    bool live[kHadItems];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) x[i] = silu_mul_h(x[i], u[i]);
-        }
-        const half8_t sc = *(const half8_t*)(srow + at);
-        float v[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = (float)x[i] * (float)sc[i];
-        had128_row16(v, lane);
-        half8_t o;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) o[i] = (_Float16)(v[i] * kRsqrt128);
-        if (live) *(half8_t*)(orow + at) = o;
+    for (int j = 0; j < kHadItems; ++j) {
+        live[j] = first + j < total;
+        const int item = live[j] ? first + j : total - 1;   // groups past the end redo the last item, store nothing
+        row[j] = item / nkb;
+        at[j] = (item - row[j] * nkb) * 128 + 8 * l16;
     }
+#pragma unroll
+    for (int j = 0; j < kHadItems; ++j) {
+        ex[j] = p.row_expert[row[j]];
+        src[j] = p.gather ? p.gather[row[j]] : row[j];
+    }
+    const _Float16* scale[2][kHadItems];
+#pragma unroll
+    for (int j = 0; j < kHadItems; ++j) {
+        if (p.gather) src[j] /= p.gather_div;
+#pragma unroll
+        for (int which = 0; which < 2; ++which) {
+            if (which >= p.num_lins) continue;
+            scale[which][j] = ex[j] == p.shared_expert
+                                  ? p.shared[p.lin_base + which].suh
+                                  : p.experts[(size_t)ex[j] * p.lins_per_expert + p.lin_base + which].suh;
+        }
+    }
+    half8_t x[kHadItems], sc[2][kHadItems];
+#pragma unroll
+    for (int j = 0; j < kHadItems; ++j) {
+        x[j] = *(const half8_t*)(p.a + (size_t)src[j] * p.K + at[j]);
+#pragma unroll
+        for (int which = 0; which < 2; ++which)
+            if (which < p.num_lins) sc[which][j] = *(const half8_t*)(scale[which][j] + at[j]);
+    }
+    if (p.a_up) {
+        half8_t u[kHadItems];
+#pragma unroll
+        for (int j = 0; j < kHadItems; ++j) u[j] = *(const half8_t*)(p.a_up + (size_t)src[j] * p.K + at[j]);
+#pragma unroll
+        for (int j = 0; j < kHadItems; ++j)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[j][i] = silu_mul_h(x[j][i], u[j][i]);
+    }
+#pragma unroll
+    for (int j = 0; j < kHadItems; ++j) {
+#pragma unroll
+        for (int which = 0; which < 2; ++which) {
+            if (which >= p.num_lins) continue;
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = (float)x[j][i] * (float)sc[which][j][i];
+            had128_row16(v, lane);
+            half8_t o;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] = (_Float16)(v[i] * kRsqrt128);
+            if (live[j]) *(half8_t*)(p.out[which] + (size_t)row[j] * p.K + at[j]) = o;
+        }
+    }
+}
+
+inline void launch_had_rows(const HadRowsParams& h, hipStream_t stream)
+{
+    const long items = (long)h.P * (h.K >> 7);
+    const unsigned wgs = (unsigned)((items + 16 * kHadItems - 1) / (16 * kHadItems));
+    hipLaunchKernelGGL(moe_had_rows_kernel, dim3(wgs), dim3(256), 0, stream, h);
+    hip_ok(hipGetLastError(), "moe_had_rows_kernel launch");
 }
 
 // ---------------------------------------------------------------- combine
 
+// out[t][h] = shared_out[t][h] + sum_j w[t][j] * slot_out[inv[t * k + j]][h], fma in slot order.
+// VEC consecutive columns per thread; the positions, weights and rows of eight slots are
+// requested together, the chain of fmas stays in slot order.
+template <int VEC>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ slot_out,
                                                           const float* __restrict__ shared_out,
                                                           const float* __restrict__ w,
                                                           const int32_t* __restrict__ inv,
                                                           float* __restrict__ out, int T, int H, int k)
 {
+    typedef float vec_t __attribute__((ext_vector_type(VEC)));
+    const int per_row = H / VEC;
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= (size_t)T * H) return;
-    const int t = (int)(i / H), h = (int)(i % H);
-    float acc = shared_out ? shared_out[i] : 0.0f;
-    for (int j = 0; j < k; ++j) {
-        const int pos = inv[t * k + j];
-        acc = __builtin_fmaf(w[t * k + j], slot_out[(size_t)pos * H + h], acc);
+    if (i >= (size_t)T * per_row) return;
+    const int t = (int)(i / per_row), h = (int)(i % per_row) * VEC;
+    vec_t acc;
+    if (shared_out) acc = *(const vec_t*)(shared_out + (size_t)t * H + h);
+    else acc = vec_t(0.0f);
+    for (int j0 = 0; j0 < k; j0 += 8) {
+        int pos[8];
+        float wj[8];
+        vec_t v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int jj = j0 + j < k ? j0 + j : k - 1;
+            pos[j] = inv[t * k + jj];
+            wj[j] = w[t * k + jj];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = *(const vec_t*)(slot_out + (size_t)pos[j] * H + h);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (j0 + j < k) {
+#pragma unroll
+                for (int c = 0; c < VEC; ++c) acc[c] = __builtin_fmaf(wj[j], v[j][c], acc[c]);
+            }
+        }
     }
-    out[i] = acc;
+    *(vec_t*)(out + (size_t)t * H + h) = acc;
+}
+
+inline void launch_combine(const float* slot_out, const float* shared_out, const float* w, const int32_t* inv,
+                           float* out, int T, int H, int k, hipStream_t stream)
+{
+    const bool vec4 = H % 4 == 0 && ((uintptr_t)slot_out | (uintptr_t)shared_out | (uintptr_t)out) % 16 == 0;
+    const size_t threads = (size_t)T * (vec4 ? H / 4 : H);
+    const dim3 grid((unsigned)((threads + 255) / 256));
+    if (vec4) hipLaunchKernelGGL(moe_combine_kernel<4>, grid, dim3(256), 0, stream, slot_out, shared_out, w, inv, out, T, H, k);
+    else hipLaunchKernelGGL(moe_combine_kernel<1>, grid, dim3(256), 0, stream, slot_out, shared_out, w, inv, out, T, H, k);
+    hip_ok(hipGetLastError(), "moe_combine_kernel launch");
 }
 
 // ------------------------------------------------------------ host side
@@ -566,9 +645,33 @@ size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 // byte offsets inside the scratch of berth_moe_permute: the sorted rows' experts, the three
 // problem counts, one-row (VALU) problems and 32-row (MFMA) problems
 struct PermuteScratch {
-    size_t row_expert, counts, vprob, mprob, total;
-    int max_m;
+    size_t row_expert, counts, vprob, mprob, bprob, total;
+    int max_m, max_b, big_min;
 };
+
+// An expert's rows beyond 32 go to MFMA problems of up to 128 rows (the weights are decoded
+// once per problem, so once per 128 rows instead of once per 32); a remainder of fewer than
+// `big_min` rows stays a 32-row problem.  BERTH_MOE_BIG_MIN: 0 keeps 32-row problems only.
+// Calls with few rows keep them too: there the launch splits K over several workgroups,
+// which the mixed launch does not.
+constexpr int kBigMinRows = 256;
+int moe_big_min(size_t rows)
+{
+    const int v = knobs().moe_big_min;
+    return v > 0 && v <= kGemmBigRows && rows >= (size_t)kBigMinRows ? v : 0;
+}
+// capacities of the two problem lists of `rows` rows over `experts` experts
+void problem_capacity(size_t rows, size_t experts, int big_min, int& max_m, int& max_b)
+{
+    if (big_min > 0) {
+        max_m = (int)std::min<size_t>(((size_t)(big_min + kGemmRows - 2) / kGemmRows) * experts, rows);
+        max_b = (int)(rows / big_min);
+    } else {
+        max_m = (int)(std::min<size_t>(experts, rows) + rows / kGemmRows + 1);
+        max_b = 0;
+    }
+}
+
 PermuteScratch permute_scratch_layout(int T, int k, int E)
 {
     const size_t P = (size_t)T * k, small = std::min<size_t>((size_t)E, P);
@@ -578,23 +681,19 @@ PermuteScratch permute_scratch_layout(int T, int k, int E)
     s.counts = at; at = align_up(at + 16);
     s.vprob = at; at = align_up(at + small * sizeof(GroupProblem));
     s.mprob = at;
-    s.max_m = (int)(small + P / kGemmRows + 2);
-    s.total = align_up(at + (size_t)s.max_m * sizeof(GroupProblem));
+    s.big_min = moe_big_min(P);
+    problem_capacity(P, (size_t)E, s.big_min, s.max_m, s.max_b);
+    at = align_up(at + (size_t)std::max(s.max_m, 1) * sizeof(GroupProblem));
+    s.bprob = at;
+    s.total = align_up(at + (size_t)std::max(s.max_b, 1) * sizeof(GroupProblem));
     return s;
 }
 
 struct MoeLayout {
     size_t idx, w, parts, offsets, perm, inv, row_expert, counts, vprob, mprob, bprob;
     size_t ah0, ah1, g, u, ahd, slot_out, sg, su, s_ahad, shared_out, vlin, total;
-    int max_v, max_m, max_b, nseg;
+    int max_v, max_m, max_b, big_min, nseg;
 };
-
-// Experts with many rows can be cut into 128-row MFMA problems (a remainder of at
-// least BERTH_MOE_BIG_MIN rows, 65 is the natural value, becomes one more).  Off by
-// default: at the measured shapes 32-row problems alone are faster, because the
-// 128-row tile spends more time per k-block than four 32-row tiles running side by
-// side.
-int moe_big_min() { return knobs().moe_big_min; }
 
 // One token: the down projection's last arrival per column block also combines the block.
 // BERTH_MOE_FOLD_COMBINE: 0 keeps the separate combine launch, 1 the two-stage form (split-K
@@ -624,13 +723,9 @@ MoeLayout moe_layout(int T, int H, int E, int k, int I, int shared_I)
     L.nseg = (H + kRouteSeg - 1) / kRouteSeg;
     const bool use_valu = T == 1 || R <= (size_t)kValuPairs;      // one row per problem, or very few rows
     L.max_v = use_valu ? (int)(std::min<size_t>((size_t)E, P) + (fold ? 1 : 0)) : 0;
-    // an expert leaves at most two small problems (fewer than 65 rows) next to its big ones
     const size_t E1 = (size_t)E + (fold ? 1 : 0);
-    const int big_min = moe_big_min();
-    const bool big = big_min > 0 && big_min <= kGemmBigRows;
-    L.max_m = use_valu ? 0 : (int)(big ? std::min<size_t>(((size_t)big_min / kGemmRows + 1) * E1, R)
-                                       : std::min<size_t>(E1, R) + R / kGemmRows + 1);
-    L.max_b = (use_valu || !big) ? 0 : (int)(R / big_min);
+    L.big_min = use_valu ? 0 : moe_big_min(R);
+    if (!use_valu) problem_capacity(R, E1, L.big_min, L.max_m, L.max_b);
     size_t at = 0;
     auto take = [&](size_t bytes) { size_t r = at; at = align_up(at + bytes); return r; };
     L.idx = take(P * 4);
@@ -732,7 +827,7 @@ PermuteParams permute_params(const int32_t* idx, unsigned char* wsb, const MoeLa
     p.E = E;
     p.use_valu = L.max_v > 0 ? 1 : 0;
     p.shared_rows = fold ? 1 : 0;
-    p.big_min = L.max_b > 0 ? moe_big_min() : (1 << 30);
+    p.big_min = L.big_min > 0 ? L.big_min : (1 << 30);
     return p;
 }
 
@@ -804,13 +899,13 @@ extern "C" int berth_moe_permute(const int32_t* idx, int32_t* offsets, int32_t* 
     p.counts = (int32_t*)(sb + at.counts);
     p.vprob = (GroupProblem*)(sb + at.vprob);
     p.mprob = (GroupProblem*)(sb + at.mprob);
-    p.bprob = p.mprob;
+    p.bprob = (GroupProblem*)(sb + at.bprob);
     p.T = T;
     p.k = k;
     p.E = E;
     p.use_valu = (T == 1 || P <= (size_t)kValuPairs) ? 1 : 0;
     p.shared_rows = 0;
-    p.big_min = 1 << 30;
+    p.big_min = !p.use_valu && at.big_min > 0 ? at.big_min : (1 << 30);
     hipLaunchKernelGGL(moe_permute_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, p);
     hip_ok(hipGetLastError(), "moe_permute_kernel launch");
     g_moe_launch = "moe_permute_kernel";
@@ -894,14 +989,19 @@ extern "C" int berth_moe_grouped_exl3(const void* a, const void* a_up, const int
         h.out[1] = (_Float16*)a_had + (size_t)P * size_k;
         h.P = P;
         h.K = size_k;
-        hipLaunchKernelGGL(moe_had_rows_kernel, dim3(P, num_lins), dim3(256), 0, stream, h);
-        hip_ok(hipGetLastError(), "moe_had_rows_kernel launch");
+        h.num_lins = num_lins;
+        launch_had_rows(h, stream);
         g.a_had = h.out[0];
         g.a_had2 = num_lins == 2 ? h.out[1] : nullptr;
         g.problems = sb + at.mprob;
         g.num_problems = (const int*)(sb + at.counts) + 1;
         g.max_problems = at.max_m;
         g.mb = 1;
+        if (at.max_b > 0) {
+            g.big_problems = sb + at.bprob;
+            g.num_big = (const int*)(sb + at.counts) + 2;
+            g.max_big = at.max_b;
+        }
         g_moe_launch = "moe_had_rows_kernel + " + launch_gemm_grouped(g);
     }
     MOE_TRY_END
@@ -914,10 +1014,7 @@ extern "C" int berth_moe_combine(const void* slot_out, const void* shared_out, c
     MOE_TRY_BEGIN
     if (!slot_out || !w || !inv || !out) throw std::runtime_error("moe combine: null device pointer");
     if (T < 1 || H < 1 || k < 1) throw std::runtime_error("moe: sizes must be positive");
-    const size_t total = (size_t)T * H;
-    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                       (const float*)slot_out, (const float*)shared_out, w, inv, (float*)out, T, H, k);
-    hip_ok(hipGetLastError(), "moe_combine_kernel launch");
+    launch_combine((const float*)slot_out, (const float*)shared_out, w, inv, (float*)out, T, H, k, (hipStream_t)stream);
     g_moe_launch = "moe_combine_kernel";
     MOE_TRY_END
 }
@@ -1030,17 +1127,15 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
         h.out[1] = (_Float16*)(wsb + L.ah1);
         h.P = R;
         h.K = H;
-        hipLaunchKernelGGL(moe_had_rows_kernel, dim3(R, 2), dim3(256), 0, stream, h);
-        hip_ok(hipGetLastError(), "moe_had_rows_kernel launch");
+        h.num_lins = 2;
+        launch_had_rows(h, stream);
         g.a_had = wsb + L.ah0;
         g.a_had2 = wsb + L.ah1;
         desc += " + moe_had_rows_kernel";
         if (L.max_b > 0) {
-            g.problems = wsb + L.bprob;
-            g.num_problems = (const int*)(wsb + L.counts) + 2;
-            g.max_problems = L.max_b;
-            g.mb = kGemmBigRows / 32;
-            desc += " + " + launch_gemm_grouped(g);
+            g.big_problems = wsb + L.bprob;
+            g.num_big = (const int*)(wsb + L.counts) + 2;
+            g.max_big = L.max_b;
         }
         g.problems = wsb + L.mprob;
         g.num_problems = (const int*)(wsb + L.counts) + 1;
@@ -1127,17 +1222,15 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
         h.out[0] = (_Float16*)(wsb + L.ahd);
         h.P = R;
         h.K = I;
-        hipLaunchKernelGGL(moe_had_rows_kernel, dim3(R, 1), dim3(256), 0, stream, h);
-        hip_ok(hipGetLastError(), "moe_had_rows_kernel launch");
+        h.num_lins = 1;
+        launch_had_rows(h, stream);
         g.a_had = wsb + L.ahd;
         g.a_had2 = nullptr;
         desc += " + moe_had_rows_kernel";
         if (L.max_b > 0) {
-            g.problems = wsb + L.bprob;
-            g.num_problems = (const int*)(wsb + L.counts) + 2;
-            g.max_problems = L.max_b;
-            g.mb = kGemmBigRows / 32;
-            desc += " + " + launch_gemm_grouped(g);
+            g.big_problems = wsb + L.bprob;
+            g.num_big = (const int*)(wsb + L.counts) + 2;
+            g.max_big = L.max_b;
         }
         g.problems = wsb + L.mprob;
         g.num_problems = (const int*)(wsb + L.counts) + 1;
@@ -1147,11 +1240,8 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
     }
 
     if (!fold_combine) {
-        const size_t total = (size_t)T * H;
-        hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
-                           (const float*)(wsb + L.slot_out), shared_out, (const float*)w,
-                           (const int32_t*)(wsb + L.inv), (float*)out, T, H, k);
-        hip_ok(hipGetLastError(), "moe_combine_kernel launch");
+        launch_combine((const float*)(wsb + L.slot_out), shared_out, (const float*)w, (const int32_t*)(wsb + L.inv),
+                       (float*)out, T, H, k, stream);
         desc += " + moe_combine_kernel";
     }
     if (idx_out) hip_ok(hipMemcpyAsync(idx_out, idx, (size_t)P * 4, hipMemcpyDeviceToDevice, stream), "idx copy");

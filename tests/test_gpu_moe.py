@@ -182,11 +182,9 @@ def test_moe_layer_matches_oracle(T, H, E, k, I, bits, shared_I, scale):
     err = np.abs(out.cpu().numpy() - want)
     assert err.max() <= 2e-3 * np.abs(want).max(), (err.max(), np.abs(want).max(), launch)
     if T > 1 and T * k + (T if shared_I == I else 0) > 8:
-        assert "exl3_gemm_kernel" in launch and "exl3_gemv_kernel" not in launch
-        import os
-        assert ("128x256" in launch) == (os.environ.get("BERTH_MOE_BIG_MIN", "0") not in ("", "0") and T * k >= 65)
+        assert ("exl3_gemm_kernel" in launch or "exl3_gemm_mixed_kernel" in launch) and "exl3_gemv_kernel" not in launch
     else:
-        assert "exl3_gemv_kernel" in launch and "exl3_gemm_kernel" not in launch
+        assert "exl3_gemv_kernel" in launch and "exl3_gemm_" not in launch
     # a second call reuses the workspace and the self-resetting counters
     out2 = torch.zeros_like(out)
     layer.forward(gpu, d_x, out2, T)
@@ -232,7 +230,7 @@ def test_moe_config3_shape_batch64():
     assert np.allclose(w.cpu().numpy(), ow, rtol=1e-5, atol=1e-7)
     _check_stages(layer, x, experts_np, None, oi, w.cpu().numpy(), out.cpu().numpy(), T, H, E, k, I, bits, 0)
     assert np.abs(out.cpu().numpy() - want).max() <= 2e-3 * np.abs(want).max(), launch
-    assert "exl3_gemm_kernel" in launch
+    assert "exl3_gemm_kernel" in launch or "exl3_gemm_mixed_kernel" in launch
 
 
 def test_moe_config4_shape_zipf_shared():
@@ -324,20 +322,28 @@ def test_moe_one_token_combine_inside_down_projection(tmp_path):
             assert np.array_equal(here[name + "_rows"], there[name + "_rows"]), (mode, name)
 
 
-def test_moe_layer_with_128_row_problems():
-    """The optional 128-row MFMA problems (BERTH_MOE_BIG_MIN, read once per process)
-    in a process of their own: the skewed case and the long-list case again."""
-    import os
-    import subprocess
-    import sys
-
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    env = dict(os.environ, BERTH_MOE_BIG_MIN="65")
-    r = subprocess.run([sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", os.path.abspath(__file__), "-k",
-                        "test_moe_layer_matches_oracle and (70-256 or 300-128)"],
-                       cwd=root, env=env, capture_output=True, text=True, timeout=600)
-    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-2000:]
-    assert "2 passed" in r.stdout, r.stdout[-2000:]
+def test_moe_128_row_problems_give_the_bits_of_32_row_problems():
+    """From 256 rows on, an expert's rows beyond 32 run as problems of up to 128 rows in the same
+    launch as the 32-row ones (BERTH_MOE_BIG_MIN: the smallest remainder that still becomes one;
+    0 switches them off).  Every output element sums the same products in the same order either
+    way, so the layer's bits do not depend on the setting."""
+    gpu = Gpu(0)
+    for T, H, E, k, I, bits, shared_I, scale in ((300, 128, 3, 1, 128, 4, 0, 50.0), (160, 256, 6, 2, 128, 3, 128, 30.0)):
+        wr, _, experts, _, shared = _make_layer(gpu, 7300 + T, H, E, I, bits, shared_I, scale)
+        x = (synth.activations(7400 + T, T, H).astype(np.float32) / np.sqrt(H)).astype(np.float16)
+        d_x = dev(x.view(np.uint16))
+        res = {}
+        for big_min in (0, 33, 65, 128):
+            with knobs(BERTH_MOE_BIG_MIN=big_min):
+                layer = MoeLayer(gpu, wr, experts, k, shared=shared, bias=synth.zipf_bias(7, E))
+                out = torch.zeros((T, H), dtype=torch.float32, device=DEV)
+                layer.forward(gpu, d_x, out, T)
+                torch.cuda.synchronize()
+                launch = K.moe.last_launch()
+                assert ("exl3_gemm_mixed_kernel" in launch) == (big_min > 0), launch
+                res[big_min] = out.cpu().numpy().view(np.uint32).copy()
+        for big_min in (33, 65, 128):
+            assert np.array_equal(res[big_min], res[0]), big_min
 
 
 def test_moe_validation_errors():
@@ -426,7 +432,7 @@ def test_stage_entry_points_compose_to_the_layer(T, H, E, k, I, bits):
     out = torch.zeros((T, H), dtype=torch.float32, device=DEV)
     K.moe.combine(slot.data_ptr(), None, w.data_ptr(), inv.data_ptr(), out.data_ptr(), T, H, k)
     torch.cuda.synchronize()
-    assert ("exl3_gemm_kernel" in first) == (P > 8), first
+    assert ("exl3_gemm_" in first) == (P > 8), first
     assert np.array_equal(idx.cpu().numpy(), inside("idx", np.int32, (T, k)))
     assert np.array_equal(perm.cpu().numpy(), inside("perm", np.int32, (P,)))
     assert np.array_equal(inv.cpu().numpy(), inside("inv", np.int32, (P,)))
