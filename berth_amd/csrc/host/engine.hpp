@@ -17,7 +17,10 @@
 #include "exl3_checkpoint.hpp"
 #include "plan.hpp"
 
+#include <atomic>
 #include <cstdint>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <stdexcept>
 #include <string>
@@ -35,6 +38,27 @@ struct DeviceError : std::runtime_error {
     int code;
     DeviceError(int c, const std::string& what) : std::runtime_error(what), code(c) {}
 };
+
+// Loader conventions that no file of the reference fixes (it refuses a bias and never opens a
+// stacked expert tensor): each is announced once per process on stderr, with the first tensor
+// that used it, so that a wrong guess shows up in a log instead of only in the outputs.
+// BERTH_QUIET_UNPINNED=1 silences the notes.
+enum class Unpinned { Bias = 0, StackedExperts = 1, SharedExpertGate = 2 };
+inline void note_unpinned(Unpinned what, const std::string& tensor)
+{
+    static std::atomic<unsigned> said{0};
+    const unsigned bit = 1u << (unsigned)what;
+    if (said.fetch_or(bit) & bit) return;
+    const char* quiet = std::getenv("BERTH_QUIET_UNPINNED");
+    if (quiet && *quiet && *quiet != '0') return;
+    static const char* const text[] = {
+        "a linear's .bias is added in fp32 after the output scales (y = W x + b)",
+        "stacked expert tensors are read K-major, expert after expert, gate columns before up columns",
+        "shared_expert_gate scales the shared expert's row by sigmoid(x . w)",
+    };
+    std::fprintf(stderr, "berth: convention not fixed by the reference, applied as assumed: %s (first: %s)\n",
+                 text[(unsigned)what], tensor.c_str());
+}
 
 inline void device_ok(int rc, const char* what)
 {
@@ -284,7 +308,10 @@ public:
         const std::vector<uint8_t> body = exl3::read_tensor(linear.trellis);
         out.trellis_ = DeviceBuffer<uint16_t>::from_host(gpu, (const uint16_t*)body.data(), body.size() / 2);
         out.a_had_ = DeviceBuffer<Half>::zeroed(gpu, (size_t)out.size_k_);
-        if (linear.bias) out.set_bias(gpu, read_float_tensor(*linear.bias));
+        if (linear.bias) {
+            note_unpinned(Unpinned::Bias, prefix + ".bias");
+            out.set_bias(gpu, read_float_tensor(*linear.bias));
+        }
         return out;
     }
 
@@ -516,6 +543,7 @@ public:
     StackedLinear(const exl3::Checkpoint& ckpt, const std::string& prefix, int blocks) : prefix_(prefix), blocks_(blocks)
     {
         const exl3::LinearExl3& linear = find_linear(ckpt, prefix);
+        note_unpinned(Unpinned::StackedExperts, prefix);
         if (linear.k.is_half()) throw WeightsError(prefix + ": half-integer rate");
         if (linear.input_scale.packed || linear.output_scale.packed)
             throw WeightsError(prefix + ": packed signs in a stacked expert tensor");

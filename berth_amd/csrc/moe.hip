@@ -498,85 +498,49 @@ struct HadRowsParams {
     int P, K;
 };
 
-// An item is one 128 block of one row; sixteen lanes (one DPP row) rotate it, eight consecutive
-// elements per lane (16-byte accesses).  A lane group takes kHadItems consecutive items and
-// issues each step's loads for all of them before the first is used (row -> expert and source
-// row -> scale pointer -> values: three dependent reads, paid once per group instead of once
-// per workgroup), and the input is read once for both linears.
-constexpr int kHadItems = 4;
-
+// An item is one 128 block of one row under one linear's scales; sixteen lanes (one DPP row)
+// rotate it, eight consecutive elements per lane (16-byte accesses).  blockIdx.x walks the
+// (row, block) items, sixteen per workgroup, so that a narrow K does not leave waves idle;
+// blockIdx.y is the linear.  Measured on 2816 rows (K 2048 under two linears / K 512 under one):
+// 14.4 / 5.0 us; with both linears in one thread 14.4 / 5.9 us, with two or four items per lane
+// group on top of that 13.7 / 6.4 and 15.9 / 7.9 us.  The K 2048 pair writes 23 MB.
 __global__ __launch_bounds__(256) void moe_had_rows_kernel(HadRowsParams p)
 {
     const int lane = threadIdx.x & 63;
     const int l16 = lane & 15;
+    const int which = blockIdx.y;
     const int nkb = p.K >> 7;
     const int total = p.P * nkb;
-    const int first = (blockIdx.x * 16 + (threadIdx.x >> 4)) * kHadItems;
-    int row[kHadItems], at[kHadItems], ex[kHadItems], src[kHadItems];
-    bool live[kHadItems];
-#pragma unroll
-    for (int j = 0; j < kHadItems; ++j) {
-        live[j] = first + j < total;
-        const int item = live[j] ? first + j : total - 1;   // groups past the end redo the last item, store nothing
-        row[j] = item / nkb;
-        at[j] = (item - row[j] * nkb) * 128 + 8 * l16;
-    }
-#pragma unroll
-    for (int j = 0; j < kHadItems; ++j) {
-        ex[j] = p.row_expert[row[j]];
-        src[j] = p.gather ? p.gather[row[j]] : row[j];
-    }
-    const _Float16* scale[2][kHadItems];
-#pragma unroll
-    for (int j = 0; j < kHadItems; ++j) {
-        if (p.gather) src[j] /= p.gather_div;
-#pragma unroll
-        for (int which = 0; which < 2; ++which) {
-            if (which >= p.num_lins) continue;
-            scale[which][j] = ex[j] == p.shared_expert
-                                  ? p.shared[p.lin_base + which].suh
-                                  : p.experts[(size_t)ex[j] * p.lins_per_expert + p.lin_base + which].suh;
-        }
-    }
-    half8_t x[kHadItems], sc[2][kHadItems];
-#pragma unroll
-    for (int j = 0; j < kHadItems; ++j) {
-        x[j] = *(const half8_t*)(p.a + (size_t)src[j] * p.K + at[j]);
-#pragma unroll
-        for (int which = 0; which < 2; ++which)
-            if (which < p.num_lins) sc[which][j] = *(const half8_t*)(scale[which][j] + at[j]);
-    }
+    const int first = blockIdx.x * 16 + (threadIdx.x >> 4);
+    const bool live = first < total;
+    const int item = live ? first : total - 1;              // groups past the end redo the last item, store nothing
+    const int row = item / nkb;
+    const int at = (item - row * nkb) * 128 + 8 * l16;
+    const int ex = p.row_expert[row];
+    const int src = p.gather ? p.gather[row] / p.gather_div : row;
+    const _Float16* scale = ex == p.shared_expert ? p.shared[p.lin_base + which].suh
+                                                  : p.experts[(size_t)ex * p.lins_per_expert + p.lin_base + which].suh;
+    half8_t x = *(const half8_t*)(p.a + (size_t)src * p.K + at);
+    const half8_t sc = *(const half8_t*)(scale + at);
     if (p.a_up) {
-        half8_t u[kHadItems];
+        const half8_t u = *(const half8_t*)(p.a_up + (size_t)src * p.K + at);
 #pragma unroll
-        for (int j = 0; j < kHadItems; ++j) u[j] = *(const half8_t*)(p.a_up + (size_t)src[j] * p.K + at[j]);
-#pragma unroll
-        for (int j = 0; j < kHadItems; ++j)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) x[j][i] = silu_mul_h(x[j][i], u[j][i]);
+        for (int i = 0; i < 8; ++i) x[i] = silu_mul_h(x[i], u[i]);
     }
+    float v[8];
 #pragma unroll
-    for (int j = 0; j < kHadItems; ++j) {
+    for (int i = 0; i < 8; ++i) v[i] = (float)x[i] * (float)sc[i];
+    had128_row16(v, lane);
+    half8_t o;
 #pragma unroll
-        for (int which = 0; which < 2; ++which) {
-            if (which >= p.num_lins) continue;
-            float v[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = (float)x[j][i] * (float)sc[which][j][i];
-            had128_row16(v, lane);
-            half8_t o;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) o[i] = (_Float16)(v[i] * kRsqrt128);
-            if (live[j]) *(half8_t*)(p.out[which] + (size_t)row[j] * p.K + at[j]) = o;
-        }
-    }
+    for (int i = 0; i < 8; ++i) o[i] = (_Float16)(v[i] * kRsqrt128);
+    if (live) *(half8_t*)(p.out[which] + (size_t)row * p.K + at) = o;
 }
 
 inline void launch_had_rows(const HadRowsParams& h, hipStream_t stream)
 {
     const long items = (long)h.P * (h.K >> 7);
-    const unsigned wgs = (unsigned)((items + 16 * kHadItems - 1) / (16 * kHadItems));
-    hipLaunchKernelGGL(moe_had_rows_kernel, dim3(wgs), dim3(256), 0, stream, h);
+    hipLaunchKernelGGL(moe_had_rows_kernel, dim3((unsigned)((items + 15) / 16), h.num_lins), dim3(256), 0, stream, h);
     hip_ok(hipGetLastError(), "moe_had_rows_kernel launch");
 }
 

@@ -287,6 +287,9 @@ def test_cpp_moe_loader_follows_the_plan(request, tmp_path, which):
     assert r.returncode == 0, r.stdout + r.stderr
     assert (f"ckpt-moe ok layer=1 tokens={T} hidden={MOE_H} experts={MOE_E} top_k={MOE_K} intermediate={MOE_I} "
             f"shared={case[4]}") in r.stdout
+    # the stacking order of a pooled expert tensor is this loader's assumption: said once, on stderr
+    assert ("convention not fixed by the reference" in r.stderr and "stacked expert tensors" in r.stderr) == \
+        (which == "stacked"), r.stderr
     want, oi, _ = _moe_want(case, x)
     assert np.array_equal(np.fromfile(tmp_path / "idx.bin", dtype=np.int32).reshape(T, MOE_K), oi)
     y = np.fromfile(tmp_path / "y.bin", dtype=np.float32).reshape(T, MOE_H)
