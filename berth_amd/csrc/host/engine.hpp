@@ -628,10 +628,13 @@ public:
     //   {mlp}.experts.<e>.{gate,up,down}_proj  one EXL3 linear per routed expert and projection, or
     //   {mlp}.experts.{gate_up,down}_proj      the stacked pair (StackedLinear; gate columns, then up)
     //   {mlp}.shared_expert.{gate,up,down}_proj the always-on expert
+    //   {mlp}.shared_expert_gate.weight        optional, [1][hidden] or [hidden] in F16 / BF16 / F32: the
+    //                                          always-on expert's row of token t is scaled by
+    //                                          sigmoid(x[t] . weight) (the reference never opens this
+    //                                          tensor: the formula is this loader's assumption)
     // with {mlp} = model.language_model.layers.<layer>.mlp.  Refused: a plan layer that is not MoE,
-    // sizes that differ from the plan's, a quantized router, a bias on an expert linear (the grouped
-    // launches have no place for it) and {mlp}.shared_expert_gate.weight (a per-token scale of the
-    // shared expert that no launch here applies).
+    // sizes that differ from the plan's, a quantized router and a bias on an expert linear (the
+    // grouped launches have no place for it).
     static MoeLayer load(const Gpu& gpu, const exl3::Checkpoint& ckpt, uint32_t layer, const plan::Ffn& ffn,
                          bool renorm = true)
     {
@@ -649,8 +652,15 @@ public:
         std::vector<Half> router((size_t)H * E);
         for (int e = 0; e < E; ++e)
             for (int h = 0; h < H; ++h) router[(size_t)h * E + e] = f32_to_f16_bits(w[(size_t)e * H + h]);
-        if (ckpt.tensors.get(mlp + ".shared_expert_gate.weight"))
-            throw WeightsError(mlp + ".shared_expert_gate.weight is present and is not applied");
+        std::vector<float> shared_gate;
+        if (const exl3::TensorInfo* sg = ckpt.tensors.get(mlp + ".shared_expert_gate.weight")) {
+            uint64_t n = 1;
+            for (uint64_t d : sg->shape) n *= d;
+            if (n != (uint64_t)H || sg->shape.size() > 2)
+                throw WeightsError(sg->name + ": expected [1][" + std::to_string(H) + "]");
+            shared_gate = read_float_tensor(*sg);
+            note_unpinned(Unpinned::SharedExpertGate, sg->name);
+        }
 
         auto checked = [&](Exl3Linear lin, int k, int n) {
             if (lin.size_k() != k || lin.size_n() != n)
@@ -689,6 +699,7 @@ public:
         out.set_shared(Expert{checked(Exl3Linear::load(gpu, ckpt, sh + ".gate_proj"), H, SI),
                               checked(Exl3Linear::load(gpu, ckpt, sh + ".up_proj"), H, SI),
                               checked(Exl3Linear::load(gpu, ckpt, sh + ".down_proj"), SI, H)});
+        if (!shared_gate.empty()) out.set_shared_gate(gpu, shared_gate);
         return out;
     }
     int hidden() const { return hidden_; }
@@ -706,6 +717,17 @@ public:
         shared_.push_back(std::move(shared));
     }
 
+    // weights [hidden] of the per-token scale sigmoid(x . w) on the always-on expert's row
+    void set_shared_gate(const Gpu& gpu, const std::vector<float>& w)
+    {
+        if (shared_.empty()) throw InputError("moe: a shared-expert gate without a shared expert");
+        if ((int)w.size() != hidden_)
+            throw InputError("moe: shared-expert gate has " + std::to_string(w.size()) + " weights for hidden size " +
+                             std::to_string(hidden_));
+        shared_gate_ = DeviceBuffer<float>::from_host(gpu, w);
+    }
+    bool has_shared_gate() const { return shared_gate_.len() != 0; }
+
     // x fp16 [tokens][hidden] -> out fp32 [tokens][hidden]; idx_out / w_out optional [tokens][top_k]
     void forward(const Gpu& gpu, const DeviceBuffer<Half>& x, DeviceBuffer<float>& out, int tokens,
                  DeviceBuffer<int32_t>* idx_out = nullptr, DeviceBuffer<float>* w_out = nullptr)
@@ -721,11 +743,12 @@ public:
             sh[1] = shared_[0].up.table_entry();
             sh[2] = shared_[0].down.table_entry();
         }
-        if (berth_moe_layer(x.raw(), router_.raw(), bias_.len() ? (const float*)bias_.raw() : nullptr, table_.raw(),
-                            shared_.empty() ? nullptr : sh, out.raw(), idx_out ? (int32_t*)idx_out->raw() : nullptr,
-                            w_out ? (float*)w_out->raw() : nullptr, ws_.raw(), ws_.len(), tokens, hidden_, num_experts_,
-                            top_k_, intermediate_, shared_i, k_bits_, (int)codebook_, renorm_ ? 1 : 0,
-                            gpu.raw_stream()) != 0)
+        if (berth_moe_layer_gated(x.raw(), router_.raw(), bias_.len() ? (const float*)bias_.raw() : nullptr,
+                                  table_.raw(), shared_.empty() ? nullptr : sh,
+                                  shared_gate_.len() ? (const float*)shared_gate_.raw() : nullptr, out.raw(),
+                                  idx_out ? (int32_t*)idx_out->raw() : nullptr, w_out ? (float*)w_out->raw() : nullptr,
+                                  ws_.raw(), ws_.len(), tokens, hidden_, num_experts_, top_k_, intermediate_, shared_i,
+                                  k_bits_, (int)codebook_, renorm_ ? 1 : 0, gpu.raw_stream()) != 0)
             throw KernelError(berth_moe_last_error());
     }
 
@@ -738,6 +761,7 @@ private:
     DeviceBuffer<berth_exl3_lin> table_;
     DeviceBuffer<Half> router_;
     DeviceBuffer<float> bias_;
+    DeviceBuffer<float> shared_gate_;
     DeviceBuffer<uint8_t> ws_;
 };
 

@@ -544,14 +544,40 @@ inline void launch_had_rows(const HadRowsParams& h, hipStream_t stream)
     hip_ok(hipGetLastError(), "moe_had_rows_kernel launch");
 }
 
+// ------------------------------------------------- shared expert's gate
+
+// scale[t] = sigmoid(z), z = x[t] . wg with the routing's arithmetic: an fp32 fma chain in row
+// order over every 64-row segment, the segment sums added in segment order (the per-token scale
+// on the always-on expert's row that Qwen-MoE checkpoints carry as shared_expert_gate.weight;
+// the reference has no MoE arithmetic).  One wave per token, lane l takes segments l, l + 64, ...
+__global__ __launch_bounds__(64) void moe_shared_gate_kernel(const _Float16* __restrict__ x, const float* __restrict__ wg,
+                                                             float* __restrict__ scale, int H)
+{
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const int nseg = (H + kRouteSeg - 1) / kRouteSeg;
+    float z = 0.0f;
+    for (int s0 = 0; s0 < nseg; s0 += 64) {
+        const int seg = s0 + lane;
+        float part = 0.0f;
+        if (seg < nseg) {
+            const int h0 = seg * kRouteSeg, hn = min(kRouteSeg, H - h0);
+            for (int i = 0; i < hn; ++i) part = __builtin_fmaf((float)x[(size_t)t * H + h0 + i], wg[h0 + i], part);
+        }
+        const int n = min(64, nseg - s0);
+        for (int j = 0; j < n; ++j) z += lane_value(part, j);       // segment order; the same sum in every lane
+    }
+    if (lane == 0) scale[t] = 1.0f / (1.0f + expf(-z));
+}
+
 // ---------------------------------------------------------------- combine
 
-// out[t][h] = shared_out[t][h] + sum_j w[t][j] * slot_out[inv[t * k + j]][h], fma in slot order.
-// VEC consecutive columns per thread; the positions, weights and rows of eight slots are
+// out[t][h] = shared_out[t][h] (times shared_scale[t] when given) + sum_j w[t][j] *
+// slot_out[inv[t * k + j]][h], fma in slot order.  VEC consecutive columns per thread; the positions, weights and rows of eight slots are
 // requested together, the chain of fmas stays in slot order.
 template <int VEC>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ slot_out,
                                                           const float* __restrict__ shared_out,
+                                                          const float* __restrict__ shared_scale,
                                                           const float* __restrict__ w,
                                                           const int32_t* __restrict__ inv,
                                                           float* __restrict__ out, int T, int H, int k)
@@ -562,8 +588,16 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     if (i >= (size_t)T * per_row) return;
     const int t = (int)(i / per_row), h = (int)(i % per_row) * VEC;
     vec_t acc;
-    if (shared_out) acc = *(const vec_t*)(shared_out + (size_t)t * H + h);
-    else acc = vec_t(0.0f);
+    if (shared_out) {
+        acc = *(const vec_t*)(shared_out + (size_t)t * H + h);
+        if (shared_scale) {
+            const float sc = shared_scale[t];
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) acc[c] *= sc;
+        }
+    } else {
+        acc = vec_t(0.0f);
+    }
     for (int j0 = 0; j0 < k; j0 += 8) {
         int pos[8];
         float wj[8];
@@ -587,14 +621,18 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     *(vec_t*)(out + (size_t)t * H + h) = acc;
 }
 
-inline void launch_combine(const float* slot_out, const float* shared_out, const float* w, const int32_t* inv,
-                           float* out, int T, int H, int k, hipStream_t stream)
+inline void launch_combine(const float* slot_out, const float* shared_out, const float* shared_scale, const float* w,
+                           const int32_t* inv, float* out, int T, int H, int k, hipStream_t stream)
 {
     const bool vec4 = H % 4 == 0 && ((uintptr_t)slot_out | (uintptr_t)shared_out | (uintptr_t)out) % 16 == 0;
     const size_t threads = (size_t)T * (vec4 ? H / 4 : H);
     const dim3 grid((unsigned)((threads + 255) / 256));
-    if (vec4) hipLaunchKernelGGL(moe_combine_kernel<4>, grid, dim3(256), 0, stream, slot_out, shared_out, w, inv, out, T, H, k);
-    else hipLaunchKernelGGL(moe_combine_kernel<1>, grid, dim3(256), 0, stream, slot_out, shared_out, w, inv, out, T, H, k);
+    if (vec4)
+        hipLaunchKernelGGL(moe_combine_kernel<4>, grid, dim3(256), 0, stream, slot_out, shared_out, shared_scale, w, inv, out,
+                           T, H, k);
+    else
+        hipLaunchKernelGGL(moe_combine_kernel<1>, grid, dim3(256), 0, stream, slot_out, shared_out, shared_scale, w, inv, out,
+                           T, H, k);
     hip_ok(hipGetLastError(), "moe_combine_kernel launch");
 }
 
@@ -655,7 +693,7 @@ PermuteScratch permute_scratch_layout(int T, int k, int E)
 
 struct MoeLayout {
     size_t idx, w, parts, offsets, perm, inv, row_expert, counts, vprob, mprob, bprob;
-    size_t ah0, ah1, g, u, ahd, slot_out, sg, su, s_ahad, shared_out, vlin, total;
+    size_t ah0, ah1, g, u, ahd, slot_out, sg, su, s_ahad, shared_out, vlin, gate_scale, total;
     int max_v, max_m, max_b, big_min, nseg;
 };
 
@@ -719,6 +757,7 @@ MoeLayout moe_layout(int T, int H, int E, int k, int I, int shared_I)
         L.shared_out = take(shared_I ? (size_t)T * H * 4 : 0);
     }
     L.vlin = take((size_t)std::max(L.max_v, 1) * sizeof(ExpertLin));
+    L.gate_scale = take((size_t)T * 4);
     L.total = at;
     return L;
 }
@@ -978,7 +1017,8 @@ extern "C" int berth_moe_combine(const void* slot_out, const void* shared_out, c
     MOE_TRY_BEGIN
     if (!slot_out || !w || !inv || !out) throw std::runtime_error("moe combine: null device pointer");
     if (T < 1 || H < 1 || k < 1) throw std::runtime_error("moe: sizes must be positive");
-    launch_combine((const float*)slot_out, (const float*)shared_out, w, inv, (float*)out, T, H, k, (hipStream_t)stream);
+    launch_combine((const float*)slot_out, (const float*)shared_out, nullptr, w, inv, (float*)out, T, H, k,
+                   (hipStream_t)stream);
     g_moe_launch = "moe_combine_kernel";
     MOE_TRY_END
 }
@@ -987,6 +1027,16 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
                                const berth_exl3_lin* shared, void* out, int32_t* idx_out, float* w_out,
                                void* workspace, size_t workspace_bytes, int T, int H, int E, int k,
                                int I, int shared_I, int k_bits, int codebook, int renorm, void* stream_)
+{
+    return berth_moe_layer_gated(x, wr, bias, experts, shared, nullptr, out, idx_out, w_out, workspace, workspace_bytes, T,
+                                 H, E, k, I, shared_I, k_bits, codebook, renorm, stream_);
+}
+
+extern "C" int berth_moe_layer_gated(const void* x, const void* wr, const float* bias, const void* experts,
+                                     const berth_exl3_lin* shared, const float* shared_gate, void* out,
+                                     int32_t* idx_out, float* w_out, void* workspace, size_t workspace_bytes, int T,
+                                     int H, int E, int k, int I, int shared_I, int k_bits, int codebook, int renorm,
+                                     void* stream_)
 {
     MOE_TRY_BEGIN
     hipStream_t stream = (hipStream_t)stream_;
@@ -999,6 +1049,7 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
     if (H % 128 || I % 128) throw std::runtime_error("moe layer: hidden and intermediate sizes must be multiples of 128");
     if (shared && (shared_I < 128 || shared_I % 128))
         throw std::runtime_error("moe layer: shared intermediate size must be a multiple of 128");
+    if (shared_gate && !shared) throw std::runtime_error("moe layer: a shared-expert gate without a shared expert");
     if (!shared) shared_I = 0;
     const bool fold = shared_is_folded(I, shared_I);
     if (fold && E + 1 > kMaxExperts) throw std::runtime_error("moe: at most 1023 routed experts next to a shared expert");
@@ -1153,7 +1204,8 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
     g.out_fp32 = 1;
     // one token: the last expert to finish a column block of the down projection
     // also combines that block, so no combine launch follows
-    const bool fold_combine = T == 1 && L.max_v > 0 && L.max_m == 0 && fold_combine_mode() != 0;
+    // (not with a gate on the always-on expert's row: the combine launch applies it)
+    const bool fold_combine = T == 1 && L.max_v > 0 && L.max_m == 0 && fold_combine_mode() != 0 && !shared_gate;
     if (fold_combine) {
         g.comb_w = (const float*)w;
         g.comb_inv = (const int32_t*)(wsb + L.inv);
@@ -1204,8 +1256,16 @@ extern "C" int berth_moe_layer(const void* x, const void* wr, const float* bias,
     }
 
     if (!fold_combine) {
-        launch_combine((const float*)(wsb + L.slot_out), shared_out, (const float*)w, (const int32_t*)(wsb + L.inv),
-                       (float*)out, T, H, k, stream);
+        const float* scale = nullptr;
+        if (shared_gate) {
+            hipLaunchKernelGGL(moe_shared_gate_kernel, dim3(T), dim3(64), 0, stream, (const _Float16*)x, shared_gate,
+                               (float*)(wsb + L.gate_scale), H);
+            hip_ok(hipGetLastError(), "moe_shared_gate_kernel launch");
+            scale = (const float*)(wsb + L.gate_scale);
+            desc += " + moe_shared_gate_kernel";
+        }
+        launch_combine((const float*)(wsb + L.slot_out), shared_out, scale, (const float*)w,
+                       (const int32_t*)(wsb + L.inv), (float*)out, T, H, k, stream);
         desc += " + moe_combine_kernel";
     }
     if (idx_out) hip_ok(hipMemcpyAsync(idx_out, idx, (size_t)P * 4, hipMemcpyDeviceToDevice, stream), "idx copy");

@@ -86,6 +86,8 @@ def load() -> C.CDLL:
         L.berth_moe_permute_scratch_bytes.restype = C.c_size_t
         L.berth_moe_layer.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t,
                                       ci, ci, ci, ci, ci, ci, ci, ci, ci, vp]
+        L.berth_moe_layer_gated.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, C.c_size_t,
+                                            ci, ci, ci, ci, ci, ci, ci, ci, ci, vp]
         L.berth_moe_workspace_bytes.argtypes = [ci] * 6
         L.berth_moe_workspace_bytes.restype = C.c_size_t
         L.berth_moe_workspace_offsets.argtypes = [ci] * 6 + [C.POINTER(C.c_size_t)]
@@ -405,10 +407,11 @@ class moe:
 
     @staticmethod
     def layer(x, wr, bias, experts_dev, shared_host, out, idx_out, w_out, workspace, workspace_bytes,
-              T, H, E, k, I, shared_I, k_bits, codebook: Codebook, renorm=True, stream=None) -> None:
-        rc = load().berth_moe_layer(x, wr, bias, experts_dev, shared_host, out, idx_out, w_out, workspace,
-                                    workspace_bytes, T, H, E, k, I, shared_I, k_bits, int(codebook),
-                                    int(renorm), stream)
+              T, H, E, k, I, shared_I, k_bits, codebook: Codebook, renorm=True, stream=None, shared_gate=None) -> None:
+        """berth_moe_layer; with `shared_gate` (device fp32 [H]) berth_moe_layer_gated."""
+        rc = load().berth_moe_layer_gated(x, wr, bias, experts_dev, shared_host, shared_gate, out, idx_out, w_out,
+                                          workspace, workspace_bytes, T, H, E, k, I, shared_I, k_bits, int(codebook),
+                                          int(renorm), stream)
         if rc != 0:
             raise LaunchError(moe.last_error() or f"moe layer launch failed ({rc})")
 

@@ -61,9 +61,10 @@ class StackedLinear:
 class MoeLayer:
     def __init__(self, gpu: Gpu, router: np.ndarray, experts, top_k: int, shared=None,
                  bias: np.ndarray | None = None, renorm: bool = True,
-                 codebook: Codebook = Codebook.MUL1):
+                 codebook: Codebook = Codebook.MUL1, shared_gate: np.ndarray | None = None):
         """router fp16 [H][E]; experts: list of (gate, up, down) Exl3Linear; shared:
-        optional (gate, up, down)."""
+        optional (gate, up, down); shared_gate: optional [H] weights of the per-token scale
+        sigmoid(x . shared_gate) on the shared expert's row (kept in fp32)."""
         self.hidden, self.num_experts = router.shape
         if len(experts) != self.num_experts:
             raise InputError("moe: router width and expert count differ")
@@ -95,6 +96,14 @@ class MoeLayer:
             for i, lin in enumerate(shared):
                 arr[i] = ExpertLinStruct(lin.trellis.data_ptr(), lin.suh.data_ptr(), lin.svh.data_ptr())
             self._shared_host = arr
+        self.shared_gate = None
+        if shared_gate is not None:
+            if not shared:
+                raise InputError("moe: a shared-expert gate without a shared expert")
+            sg = np.ascontiguousarray(shared_gate, dtype=np.float32).ravel()
+            if sg.size != self.hidden:
+                raise InputError(f"moe: shared-expert gate has {sg.size} weights for hidden size {self.hidden}")
+            self.shared_gate = torch.from_numpy(sg).to(gpu.device)
         self._ws = None
         self._ws_tokens = 0
 
@@ -109,10 +118,12 @@ class MoeLayer:
           {mlp}.experts.<e>.{gate,up,down}_proj   one EXL3 linear per routed expert and projection, or
           {mlp}.experts.{gate_up,down}_proj       the stacked pair (StackedLinear; gate columns, then up)
           {mlp}.shared_expert.{gate,up,down}_proj the always-on expert
+          {mlp}.shared_expert_gate.weight         optional [1][hidden] (or [hidden]) in F16 / BF16 / F32:
+                                                  the always-on expert's row of token t is scaled by
+                                                  sigmoid(x[t] . weight); the reference never opens this
+                                                  tensor, so the formula is this loader's assumption
         Refused: a plan layer that is not MoE, sizes that differ from the plan's, a quantized
-        router, a bias on an expert linear (the grouped launches have no place for it) and
-        {mlp}.shared_expert_gate.weight (a per-token scale of the shared expert that no launch
-        here applies)."""
+        router and a bias on an expert linear (the grouped launches have no place for it)."""
         if not ffn.is_moe:
             raise InputError(f"moe: layer {layer} is planned with a dense MLP")
         mlp = f"model.language_model.layers.{layer}.mlp"
@@ -126,8 +137,12 @@ class MoeLayer:
             raise WeightsError(f"{gate.name}: expected [{E}][hidden]")
         H = int(gate.shape[1])
         router = np.ascontiguousarray(read_float_tensor(gate).reshape(E, H).T.astype(np.float16))
-        if ckpt.tensors.get(f"{mlp}.shared_expert_gate.weight") is not None:
-            raise WeightsError(f"{mlp}.shared_expert_gate.weight is present and is not applied")
+        shared_gate = None
+        sgt = ckpt.tensors.get(f"{mlp}.shared_expert_gate.weight")
+        if sgt is not None:
+            if int(np.prod(sgt.shape)) != H or len(sgt.shape) > 2:
+                raise WeightsError(f"{sgt.name}: expected [1][{H}]")
+            shared_gate = read_float_tensor(sgt).ravel()
 
         def checked(prefix, k, n):
             lin = Exl3Linear.load(gpu, ckpt, prefix)
@@ -158,7 +173,7 @@ class MoeLayer:
         if any(lin.k_bits != g0.k_bits or lin.codebook != g0.codebook for lin in shared):
             raise InputError("moe: the shared expert must use the routed experts' bit rate and codebook")
         return cls(gpu, router, experts, ffn.router.experts_per_tok, shared=shared, renorm=renorm,
-                   codebook=g0.codebook)
+                   codebook=g0.codebook, shared_gate=shared_gate)
 
     def trellis_bytes(self) -> int:
         n = sum(lin.trellis_bytes() for trio in self.experts for lin in trio)
@@ -186,4 +201,5 @@ class MoeLayer:
                     out.data_ptr(), None if idx_out is None else idx_out.data_ptr(),
                     None if w_out is None else w_out.data_ptr(), ws.data_ptr(), ws.numel(),
                     T, self.hidden, self.num_experts, self.top_k, self.intermediate, self.shared_I,
-                    self.k_bits, self.codebook, self.renorm, gpu.raw_stream())
+                    self.k_bits, self.codebook, self.renorm, gpu.raw_stream(),
+                    None if self.shared_gate is None else self.shared_gate.data_ptr())

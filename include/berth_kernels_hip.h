@@ -331,6 +331,16 @@ int berth_moe_layer(const void* x, const void* wr, const float* bias, const void
                     const berth_exl3_lin* shared, void* out, int32_t* idx_out, float* w_out,
                     void* workspace, size_t workspace_bytes, int T, int H, int E, int k, int I,
                     int shared_I, int k_bits, int codebook, int renorm, void* stream);
+/* The same layer with a gate on the always-on expert: shared_gate fp32 [H] on the device (the
+ * shared_expert_gate.weight of Qwen-MoE checkpoints) scales that expert's row of token t by
+ * sigmoid(x[t] . shared_gate) before the routed experts are added; the dot product is an fp32 fma
+ * chain in row order per 64-row segment, segments added in order.  NULL: berth_moe_layer.  The
+ * reference has no MoE arithmetic (crates/berth-engine/src/model.rs:404-409); the shape of the
+ * layer follows crates/berth-plan/src/plan.rs:24-59. */
+int berth_moe_layer_gated(const void* x, const void* wr, const float* bias, const void* experts,
+                          const berth_exl3_lin* shared, const float* shared_gate, void* out, int32_t* idx_out,
+                          float* w_out, void* workspace, size_t workspace_bytes, int T, int H, int E, int k,
+                          int I, int shared_I, int k_bits, int codebook, int renorm, void* stream);
 size_t berth_moe_workspace_bytes(int T, int H, int E, int k, int I, int shared_I);
 /* byte offsets inside that workspace of {idx, w, offsets, perm, inv, gate_out
  * fp16 [T*k][I], up_out fp16 [T*k][I], slot_out fp32 [T*k][H] (rows in expert-

@@ -578,10 +578,36 @@ int bo_expert_ffn(const uint16_t* x, int m, int H, int I, int bits, int cb,
     return rc;
 }
 
+/* scale[t] = 1 / (1 + exp(-z)), z = x[t] . wg: an fp32 fma chain in row order over every
+ * 64-row segment, the segment sums added in segment order (the routing's arithmetic). */
+int bo_moe_shared_gate(const uint16_t* x, const float* wg, int T, int H, float* scale)
+{
+    if (T < 1 || H < 1) return 1;
+    for (int t = 0; t < T; ++t) {
+        float z = 0.0f;
+        for (int h0 = 0; h0 < H; h0 += 64) {
+            float part = 0.0f;
+            for (int h = h0; h < H && h < h0 + 64; ++h) part = fmaf(bo_f16_to_f32(x[(size_t)t * H + h]), wg[h], part);
+            z += part;
+        }
+        scale[t] = 1.0f / (1.0f + expf(-z));
+    }
+    return 0;
+}
+
 int bo_moe_layer(const uint16_t* x, int T, int H, int E, int k, int I, int bits,
                  int cb, const uint16_t* wr, const float* bias, int renorm,
                  const bo_lin_t* experts, const bo_lin_t* shared, int shared_I,
                  float* out, int32_t* idx_out, float* w_out)
+{
+    return bo_moe_layer_gated(x, T, H, E, k, I, bits, cb, wr, bias, renorm, experts, shared, shared_I, NULL, out,
+                              idx_out, w_out);
+}
+
+int bo_moe_layer_gated(const uint16_t* x, int T, int H, int E, int k, int I, int bits,
+                       int cb, const uint16_t* wr, const float* bias, int renorm,
+                       const bo_lin_t* experts, const bo_lin_t* shared, int shared_I,
+                       const float* shared_gate, float* out, int32_t* idx_out, float* w_out)
 {
     int32_t* idx = (int32_t*)malloc((size_t)T * k * sizeof(int32_t));
     float* w = (float*)malloc((size_t)T * k * sizeof(float));
@@ -610,6 +636,13 @@ int bo_moe_layer(const uint16_t* x, int T, int H, int E, int k, int I, int bits,
         if (shared) rc = bo_expert_ffn(x, T, H, shared_I, bits, cb, &shared[0], &shared[1],
                                        &shared[2], out);
         else memset(out, 0, (size_t)T * H * sizeof(float));
+        if (!rc && shared && shared_gate) {
+            float* scale = (float*)malloc((size_t)T * sizeof(float));
+            rc = bo_moe_shared_gate(x, shared_gate, T, H, scale);
+            for (int t = 0; t < T && !rc; ++t)
+                for (int h = 0; h < H; ++h) out[(size_t)t * H + h] *= scale[t];
+            free(scale);
+        }
     }
     if (!rc) {
         for (int t = 0; t < T; ++t)

@@ -152,6 +152,17 @@ int bo_moe_layer(const uint16_t* x, int T, int H, int E, int k, int I, int bits,
                  const bo_lin_t* experts, const bo_lin_t* shared, int shared_I,
                  float* out, int32_t* idx_out, float* w_out);
 
+/* scale[t] = sigmoid(x[t] . wg) (wg fp32 [H]); the dot product as in bo_moe_route: fp32 fma
+ * chain in row order per 64-row segment, segments added in order.  [D] defined by this build
+ * (the reference never opens shared_expert_gate.weight).  Checked against float64 numpy. */
+int bo_moe_shared_gate(const uint16_t* x, const float* wg, int T, int H, float* scale);
+/* bo_moe_layer with the always-on expert's row of token t multiplied by scale[t] (one fp32
+ * product) before the routed experts are added; shared_gate NULL: bo_moe_layer. */
+int bo_moe_layer_gated(const uint16_t* x, int T, int H, int E, int k, int I, int bits,
+                       int cb, const uint16_t* wr, const float* bias, int renorm,
+                       const bo_lin_t* experts, const bo_lin_t* shared, int shared_I,
+                       const float* shared_gate, float* out, int32_t* idx_out, float* w_out);
+
 /* RMS norm with an optional fused residual, crates/berth-kernels/src/ops.rs:398-500:
  * residual (may be NULL) += x in fp32, then y = fp16((v * rmf) * (w + constant_bias) *
  * constant_scale) with rmf = fp32(1/sqrt(mean(v^2) + epsilon)); weight bf16 or fp16 bits.

@@ -262,9 +262,21 @@ def expert_ffn(x, gate, up, down, I: int, bits: int, cb: int) -> np.ndarray:
     return out
 
 
+def moe_shared_gate(x, wg):
+    """scale[t] = sigmoid(x[t] . wg), the dot product in the routing's arithmetic."""
+    x16 = _u16(x)
+    T, H = x16.shape
+    g = np.ascontiguousarray(wg, dtype=np.float32).ravel()
+    out = np.empty(T, dtype=np.float32)
+    if g.size != H or lib().bo_moe_shared_gate(_p(x16), _p(g), T, H, _p(out)):
+        raise ValueError("bo_moe_shared_gate: bad shape")
+    return out
+
+
 def moe_layer(x, wr, experts, k: int, I: int, bits: int, cb: int, bias=None, renorm=True,
-              shared=None, shared_I: int = 0):
-    """experts: list of E (gate, up, down) with each a (trellis, suh, svh) triple.
+              shared=None, shared_I: int = 0, shared_gate=None):
+    """experts: list of E (gate, up, down) with each a (trellis, suh, svh) triple; shared_gate:
+    optional fp32 [H] weights of the per-token scale on the shared expert's row.
     Returns (out fp32 [T][H], idx, w)."""
     x16, w16 = _u16(x), _u16(wr)
     T, H = x16.shape
@@ -278,8 +290,9 @@ def moe_layer(x, wr, experts, k: int, I: int, bits: int, cb: int, bias=None, ren
     idx = np.empty((T, k), dtype=np.int32)
     w = np.empty((T, k), dtype=np.float32)
     b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
-    rc = lib().bo_moe_layer(_p(x16), T, H, E, k, I, bits, cb, _p(w16), _p(b), int(renorm),
-                            arr, sh_arr, int(shared_I), _p(out), _p(idx), _p(w))
+    sg = None if shared_gate is None else np.ascontiguousarray(shared_gate, dtype=np.float32).ravel()
+    rc = lib().bo_moe_layer_gated(_p(x16), T, H, E, k, I, bits, cb, _p(w16), _p(b), int(renorm),
+                                  arr, sh_arr, int(shared_I), _p(sg), _p(out), _p(idx), _p(w))
     del keep, sh_keep
     if rc:
         raise ValueError("bo_moe_layer failed")

@@ -192,12 +192,13 @@ def moe_ckpt_per_expert(tmp_path_factory):
     tensors.append(("model.language_model.norm.weight", "BF16", (MOE_H,), bytes(2 * MOE_H)))
     tensors.append(("model.visual.pos_embed.weight", "BF16", (64,), bytes(128)))
     U.write_checkpoint(d, tensors, _moe_config(MOE_I))
-    return d, experts, shared, stored.astype(np.float16), MOE_I
+    return d, experts, shared, stored.astype(np.float16), MOE_I, None
 
 
 @pytest.fixture(scope="module")
 def moe_ckpt_stacked(tmp_path_factory):
-    """`experts.gate_up_proj` / `experts.down_proj` stacked along K, an F32 router, a wider shared expert."""
+    """`experts.gate_up_proj` / `experts.down_proj` stacked along K, an F32 router, a wider shared expert
+    with a BF16 `shared_expert_gate.weight` on it."""
     d = tmp_path_factory.mktemp("moe_ckpt_b")
     shared_i = 256
     experts, shared, wf = _moe_parts(9300, shared_i)
@@ -213,8 +214,10 @@ def moe_ckpt_stacked(tmp_path_factory):
                                 np.concatenate([dn[2] for _, _, dn in experts]))
     for name, lin in zip(("gate_proj", "up_proj", "down_proj"), shared):
         tensors += U.linear_tensors(f"{MOE_MLP}.shared_expert.{name}", *lin)
+    gate_bits = _bf16_bits((np.random.default_rng(9301).standard_normal(MOE_H) * 1.5).astype(np.float32))
+    tensors.append((f"{MOE_MLP}.shared_expert_gate.weight", "BF16", (1, MOE_H), gate_bits.tobytes()))
     U.write_checkpoint(d, tensors, _moe_config(shared_i))
-    return d, experts, shared, wf.astype(np.float16), shared_i
+    return d, experts, shared, wf.astype(np.float16), shared_i, (gate_bits.astype(np.uint32) << 16).view(np.float32)
 
 
 def _moe_tokens(T):
@@ -222,8 +225,8 @@ def _moe_tokens(T):
 
 
 def _moe_want(case, x):
-    _, experts, shared, wr, shared_i = case
-    return O.moe_layer(x, wr, experts, MOE_K, MOE_I, 4, 2, shared=shared, shared_I=shared_i)
+    _, experts, shared, wr, shared_i, shared_gate = case
+    return O.moe_layer(x, wr, experts, MOE_K, MOE_I, 4, 2, shared=shared, shared_I=shared_i, shared_gate=shared_gate)
 
 
 @pytest.mark.parametrize("which", ["per_expert", "stacked"])
@@ -238,6 +241,9 @@ def test_python_moe_loader_follows_the_plan(request, which, T):
     layer = MoeLayer.load(gpu, ckpt, 1, ffn)
     assert (layer.hidden, layer.num_experts, layer.top_k, layer.intermediate, layer.shared_I) == \
         (MOE_H, MOE_E, MOE_K, MOE_I, case[4])
+    assert (layer.shared_gate is not None) == (case[5] is not None)
+    if case[5] is not None:
+        assert np.array_equal(layer.shared_gate.cpu().numpy(), case[5])
     x = _moe_tokens(T)
     out = torch.zeros((T, MOE_H), dtype=torch.float32, device=gpu.device)
     idx = torch.zeros((T, MOE_K), dtype=torch.int32, device=gpu.device)
@@ -267,12 +273,12 @@ def test_python_moe_loader_refusals(moe_ckpt_per_expert, ckpt_dir, tmp_path):
         MoeLayer.load(gpu, ckpt, 1, P.Ffn(P.Router(16, MOE_K), P.SharedExpert(MOE_I), P.RoutedExperts(16, MOE_K, MOE_I)))
     with pytest.raises(WeightsError, match="experts.0.gate_proj: 256x128 where the plan has 256x256"):
         MoeLayer.load(gpu, ckpt, 1, P.Ffn(P.Router(MOE_E, MOE_K), P.SharedExpert(MOE_I), P.RoutedExperts(MOE_E, MOE_K, 256)))
-    # a scale on the shared expert's output and a bias on an expert are both refused
+    # a gate of the wrong size on the shared expert and a bias on an expert are both refused
     experts, shared, wf = _moe_parts(9700, MOE_I, bits=2)
     tensors = [(f"{MOE_MLP}.gate.weight", "F32", (MOE_E, MOE_H), np.ascontiguousarray(wf.T).tobytes()),
-               (f"{MOE_MLP}.shared_expert_gate.weight", "F32", (1, MOE_H), bytes(4 * MOE_H))]
+               (f"{MOE_MLP}.shared_expert_gate.weight", "F32", (2, MOE_H), bytes(8 * MOE_H))]
     U.write_checkpoint(tmp_path, tensors, _moe_config(MOE_I))
-    with pytest.raises(WeightsError, match="shared_expert_gate.weight is present and is not applied"):
+    with pytest.raises(WeightsError, match=rf"shared_expert_gate.weight: expected \[1\]\[{MOE_H}\]"):
         MoeLayer.load(gpu, exl3.Checkpoint.open(tmp_path), 1, good)
 
 
@@ -290,6 +296,7 @@ def test_cpp_moe_loader_follows_the_plan(request, tmp_path, which):
     # the stacking order of a pooled expert tensor is this loader's assumption: said once, on stderr
     assert ("convention not fixed by the reference" in r.stderr and "stacked expert tensors" in r.stderr) == \
         (which == "stacked"), r.stderr
+    assert ("shared_expert_gate scales the shared expert's row" in r.stderr) == (which == "stacked"), r.stderr
     want, oi, _ = _moe_want(case, x)
     assert np.array_equal(np.fromfile(tmp_path / "idx.bin", dtype=np.int32).reshape(T, MOE_K), oi)
     y = np.fromfile(tmp_path / "y.bin", dtype=np.float32).reshape(T, MOE_H)

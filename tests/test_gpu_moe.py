@@ -8,6 +8,7 @@ import torch
 from berth_amd import kernels as K
 from berth_amd import synth
 from berth_amd.device import Exl3Linear, Gpu
+from berth_amd.device import InputError
 from berth_amd.moe import MoeLayer
 from oracle import oracle as O
 from tests.gpu_util import DEV, close, dev, knobs
@@ -344,6 +345,41 @@ def test_moe_128_row_problems_give_the_bits_of_32_row_problems():
                 res[big_min] = out.cpu().numpy().view(np.uint32).copy()
         for big_min in (33, 65, 128):
             assert np.array_equal(res[big_min], res[0]), big_min
+
+
+@pytest.mark.parametrize("T,H,E,k,I,bits,shared_I", [
+    (1, 256, 8, 2, 128, 4, 128),         # one token, the shared expert inside the grouped launches
+    (1, 384, 8, 3, 128, 4, 256),         # one token, the shared expert as dense launches
+    (5, 256, 8, 2, 128, 3, 128),
+    (40, 256, 4, 2, 128, 4, 256),        # the MFMA path
+])
+def test_moe_layer_with_a_gate_on_the_shared_expert(T, H, E, k, I, bits, shared_I):
+    """berth_moe_layer_gated: the always-on expert's row is scaled by sigmoid(x . w) before the
+    routed experts are added; routing and every stage ahead of the combine are untouched."""
+    gpu = Gpu(0)
+    wr, experts_np, experts, shared_np, shared = _make_layer(gpu, 6600 + T, H, E, I, bits, shared_I)
+    wg = (np.random.default_rng(6700 + T).standard_normal(H) * 2.0).astype(np.float32)
+    x = (synth.activations(6800 + T, T, H).astype(np.float32) / np.sqrt(H)).astype(np.float16)
+    d_x = dev(x.view(np.uint16))
+    outs = {}
+    for name, gate in (("plain", None), ("gated", wg)):
+        layer = MoeLayer(gpu, wr, experts, k, shared=shared, shared_gate=gate)
+        out = torch.zeros((T, H), dtype=torch.float32, device=DEV)
+        idx = torch.zeros((T, k), dtype=torch.int32, device=DEV)
+        layer.forward(gpu, d_x, out, T, idx)
+        torch.cuda.synchronize()
+        assert ("moe_shared_gate_kernel" in K.moe.last_launch()) == (gate is not None), K.moe.last_launch()
+        want, oi, _ = O.moe_layer(x, wr, experts_np, k, I, bits, 2, shared=shared_np, shared_I=shared_I, shared_gate=gate)
+        assert np.array_equal(idx.cpu().numpy(), oi)
+        outs[name] = out.cpu().numpy()
+        assert np.abs(outs[name] - want).max() <= 2e-3 * np.abs(want).max(), name
+    scale = O.moe_shared_gate(x, wg)
+    assert np.ptp(scale) > 0.05 or T == 1
+    assert np.abs(outs["gated"] - outs["plain"]).max() > 1e-3 * np.abs(outs["plain"]).max()   # the gate does something
+    with pytest.raises(InputError, match="without a shared expert"):
+        MoeLayer(gpu, wr, experts, k, shared_gate=wg)
+    with pytest.raises(K.LaunchError, match="gate without a shared expert"):
+        K.moe.layer(1, 1, None, 1, None, 1, None, None, 1, 1 << 30, 1, 128, 8, 2, 128, 0, 4, K.Codebook.MUL1, shared_gate=1)
 
 
 def test_moe_validation_errors():

@@ -285,6 +285,31 @@ def test_moe_layer_is_weighted_sum_of_expert_ffns():
     assert np.allclose(out, want, rtol=1e-5, atol=1e-4)
 
 
+def test_shared_gate_is_a_sigmoid_of_the_dot_product_and_scales_only_the_shared_row():
+    T, H, E, k, I, bits = 4, 384, 4, 2, 128, 4
+    x = (synth.activations(64, T, H).astype(np.float32) / 8).astype(np.float16)
+    wg = (np.random.default_rng(65).standard_normal(H) * 0.7).astype(np.float32)
+    scale = O.moe_shared_gate(x, wg)
+    z = x.astype(np.float64) @ wg.astype(np.float64)
+    assert np.allclose(scale, 1.0 / (1.0 + np.exp(-z)), rtol=2e-6, atol=1e-7)
+    assert 0.02 < scale.min() and scale.max() < 0.98 and np.ptp(scale) > 0.1       # the case is not saturated
+    # a dropped sign or a missing 1 + would show: sigmoid(-z) = 1 - sigmoid(z), sigmoid(0) = 1/2
+    assert np.allclose(O.moe_shared_gate(x, -wg), 1.0 - scale, atol=1e-6)
+    assert np.array_equal(O.moe_shared_gate(x, np.zeros(H, np.float32)), np.full(T, 0.5, np.float32))
+    wr = (synth.router_weight(66, H, E).astype(np.float32) * 20).astype(np.float16)
+    experts = _experts(67, E, H, I, bits)
+    shared = _experts(68, 1, H, I, bits)[0]
+    routed, idx, w = O.moe_layer(x, wr, experts, k, I, bits, 2)
+    plain, _, _ = O.moe_layer(x, wr, experts, k, I, bits, 2, shared=shared, shared_I=I)
+    gated, gi, gw = O.moe_layer(x, wr, experts, k, I, bits, 2, shared=shared, shared_I=I, shared_gate=wg)
+    assert np.array_equal(gi, idx) and np.array_equal(gw, w)
+    sh = O.expert_ffn(x, *shared, I=I, bits=bits, cb=2).astype(np.float64)
+    assert np.allclose(plain - routed, sh, rtol=1e-4, atol=1e-4 * np.abs(sh).max())
+    assert np.allclose(gated - routed, scale[:, None] * sh, rtol=1e-4, atol=1e-4 * np.abs(sh).max())
+    with pytest.raises(ValueError):
+        O.moe_shared_gate(x, wg[:-1])
+
+
 def test_moe_layer_k_equals_E_dense_mixture_identical_tokens():
     T, H, E, I, bits = 2, 128, 2, 128, 3
     x1 = synth.activations(70, 1, H)
