@@ -42,8 +42,8 @@ PROFILE = {
                      "exl3_gemv_stream_kernel<4,2,table=0x0>",
                      "sliced x2 by value exl3_gemv_stream_kernel<4,2,table=0x0>",
                      "exl3_gemv_stream_kernel<4,2,table=0x0>"],
-        "traffic_bytes_per_launch": int((42378 + 258) * 1024),
-        "valu_instr_per_weight": 4.9},
+        "traffic_bytes_per_launch": int((42265 + 892) * 1024),
+        "valu_instr_per_weight": 5.0},
 }
 ORDER = ["q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"]
 OUT_FP32 = {"q_proj": False, "k_proj": False, "v_proj": False, "o_proj": True,

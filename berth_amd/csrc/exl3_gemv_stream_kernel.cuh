@@ -371,6 +371,19 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
         rot_s[t] = sin[kb * 64 + lane];
         if (SILU) rot_u[t] = uin[kb * 64 + lane];
     }
+    // NORM: this thread's strided share of the whole row, for the sum of squares, asked for now
+    // so that it arrives behind the split arithmetic instead of being waited for later
+    constexpr int kNormAhead = 4;                           // covers K <= 8192; a longer row is read in the loop below
+    float2_t row_x[NORM ? kNormAhead : 1], row_r[NORM ? kNormAhead : 1];
+    if constexpr (NORM) {
+#pragma unroll
+        for (int j = 0; j < kNormAhead; ++j) {
+            const unsigned e = threadIdx.x + (unsigned)j * (kStreamWaves * 64);
+            const unsigned ec = e < (unsigned)p.K / 2 ? e : 0u;         // past the end: any valid element, unused
+            row_x[j] = ((global_ptr<const float2_t>)as_global(p.norm_x))[ec];
+            row_r[j] = ((global_ptr<const float2_t>)as_global(p.norm_res))[ec];
+        }
+    }
 
     // ---- this wave's units [uw0, uw1) and its first tile row
     const unsigned Ww = W0 + (unsigned)wave;
@@ -438,7 +451,18 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
     // fp16, as rms_norm_kernel forms it
     if constexpr (NORM) {
         double ss = 0.0;
-        for (unsigned e = threadIdx.x; e < (unsigned)p.K / 2; e += kStreamWaves * 64) {
+#pragma unroll
+        for (int j = 0; j < kNormAhead; ++j) {
+            const unsigned e = threadIdx.x + (unsigned)j * (kStreamWaves * 64);
+            if (e < (unsigned)p.K / 2) {
+                const float2_t v = {row_r[j].x + row_x[j].x, row_r[j].y + row_x[j].y};
+                ss += (double)v.x * (double)v.x;
+                ss += (double)v.y * (double)v.y;
+                // the first workgroup of the first problem writes the updated residual stream
+                if (prob == 0 && gl == 0) ((global_ptr<float2_t>)as_global(p.norm_res_out))[e] = v;
+            }
+        }
+        for (unsigned e = threadIdx.x + kNormAhead * kStreamWaves * 64; e < (unsigned)p.K / 2; e += kStreamWaves * 64) {
             const float2_t xv = ((global_ptr<const float2_t>)as_global(p.norm_x))[e];
             const float2_t rv = ((global_ptr<const float2_t>)as_global(p.norm_res))[e];
             const float2_t v = {rv.x + xv.x, rv.y + xv.y};
@@ -447,8 +471,21 @@ __global__ __launch_bounds__(1024, 1) void exl3_gemv_stream_kernel(StreamParams 
             // the first workgroup of the first problem writes the updated residual stream
             if (prob == 0 && gl == 0) ((global_ptr<float2_t>)as_global(p.norm_res_out))[e] = v;
         }
-#pragma unroll
-        for (int d = 32; d >= 1; d >>= 1) ss += __shfl_xor(ss, d, 64);
+        // butterflies over lane distances 32 .. 1 (the order of the separate norm kernel's wave sum),
+        // the partner's two dwords fetched with DPP moves and the row swaps instead of LDS permutes
+        auto partner = [](double v, auto move) {
+            const uint64_t b = __builtin_bit_cast(uint64_t, v);
+            const float lo = move(__builtin_bit_cast(float, (uint32_t)b));
+            const float hi = move(__builtin_bit_cast(float, (uint32_t)(b >> 32)));
+            return __builtin_bit_cast(double, (uint64_t)__builtin_bit_cast(uint32_t, lo) |
+                                                  ((uint64_t)__builtin_bit_cast(uint32_t, hi) << 32));
+        };
+        ss += partner(ss, [](float f) { return lane_xor_swap32(f); });
+        ss += partner(ss, [](float f) { return lane_xor_swap16(f); });
+        ss += partner(ss, [](float f) { return lane_xor_dpp<8>(f); });
+        ss += partner(ss, [](float f) { return lane_xor_dpp<4>(f); });
+        ss += partner(ss, [](float f) { return lane_xor_dpp<2>(f); });
+        ss += partner(ss, [](float f) { return lane_xor_dpp<1>(f); });
         if (lane == 0) norm_part[wave] = ss;
         __syncthreads();
         double total = 0.0;
