@@ -163,6 +163,7 @@ Knobs read_knobs()
     k.gemm_rows256 = env_int("BERTH_GEMM_ROWS256", 1);
     k.counter_stride = clamp(env_int("BERTH_COUNTER_STRIDE", 32), 1, 32);
     k.moe_big_min = env_int("BERTH_MOE_BIG_MIN", 33);
+    k.moe_route_slab = env_int("BERTH_MOE_ROUTE_SLAB", 1);
     k.moe_fold_combine = env_int("BERTH_MOE_FOLD_COMBINE", 2);
     k.moe_inline_route = env_int("BERTH_MOE_INLINE_ROUTE", 1);
     k.moe_resolved = env_int("BERTH_MOE_RESOLVED", 1);

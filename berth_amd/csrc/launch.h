@@ -75,6 +75,7 @@ struct Knobs {
     int gemm_rows256;           // BERTH_GEMM_ROWS256
     int counter_stride;         // BERTH_COUNTER_STRIDE         cap on the words between arrival counters (1..32)
     int moe_big_min;            // BERTH_MOE_BIG_MIN
+    int moe_route_slab;         // BERTH_MOE_ROUTE_SLAB: 0 keeps the two-launch routing of many tokens
     int moe_fold_combine;       // BERTH_MOE_FOLD_COMBINE
     int moe_inline_route;       // BERTH_MOE_INLINE_ROUTE
     int moe_resolved;           // BERTH_MOE_RESOLVED

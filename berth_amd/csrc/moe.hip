@@ -370,6 +370,155 @@ __global__ __launch_bounds__(256) void moe_route_finish_kernel(RouteParams p)
     route_topk(lg, tid, p, t);
 }
 
+// Many tokens, an even number of experts: the whole routing of TT tokens x a slab of 128 experts
+// in one workgroup of sixteen waves, so that the segment sums never travel through memory (two
+// launches of the form above write and read 4 * nseg bytes per (token, expert): 16.8 MB each way
+// for 256 tokens x 512 experts).  Wave w takes segments w, w + 16, ...; a lane holds two
+// neighbouring experts (one 4-byte load per router row) and TT tokens, whose activations are
+// wave-uniform and come through the scalar cache.  The segment sums meet in LDS
+// ([segment][token][expert]); after the barrier thread (token, expert) adds them in segment order
+// and adds the bias.  With one slab the workgroup selects right away (wave tt: token tt); with
+// several the logits go to memory and the last slab of a token group to arrive selects.  Same
+// arithmetic as every other routing kernel here: fma chains in row order per 64-row segment,
+// segments added in order.
+constexpr int kSlabExperts = 128;
+// LDS of a workgroup: segment sums [nseg][tt][128] fp32, then the tokens' rows [tt][H] as fp32 (H = 64 nseg)
+inline __host__ __device__ int route_slab_lds_bytes(int nseg, int tt) { return nseg * tt * kSlabExperts * 4 + tt * nseg * kRouteSeg * 4; }
+
+template <int TT>
+__global__ __launch_bounds__(1024) void moe_route_slab_kernel(RouteParams p)
+{
+    extern __shared__ __align__(16) float s_parts[];               // [nseg][TT][128]
+    __shared__ unsigned s_last;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // uniform: the token loads stay scalar
+    // token group fastest: consecutive workgroups go to different dies, so every die works on all
+    // slabs (one slab's rows alone fall on a quarter of an L2's channels)
+    const int grp = blockIdx.x, slab = blockIdx.y, nslab = gridDim.y;
+    const int t0 = grp * TT;
+    const int e0 = slab * kSlabExperts + 2 * lane;
+    const int e_ld = e0 < p.E ? e0 : p.E - 2;                       // lanes past the end redo the last pair, unused
+    const global_ptr<const half2_t> wcol = (global_ptr<const half2_t>)as_global(p.wr + e_ld);
+    const size_t wstride = (size_t)p.E / 2;                         // half2 elements per router row
+    // the tokens' rows go to LDS once, widened to fp32 (tokens past the end: the last token,
+    // unused); a step then reads its sixteen rows of every token with wave-uniform addresses
+    // (broadcast reads).
+    float* const s_x = s_parts + (size_t)p.nseg * TT * kSlabExperts;
+    {
+        const int per_row = p.H / 2;                                        // dwords
+        for (int i = threadIdx.x; i < TT * per_row; i += 1024) {
+            const int tt = i / per_row, d = i - tt * per_row;
+            const uint32_t v = ((global_ptr<const uint32_t>)as_global((const uint32_t*)(p.x + (size_t)min(t0 + tt, p.T - 1) * p.H)))[d];
+            const half2_t h = __builtin_bit_cast(half2_t, v);
+            *(float2_t*)&s_x[2 * i] = float2_t{(float)h.x, (float)h.y};
+        }
+    }
+    __syncthreads();
+
+    // The wave's segments as one run of sixteen-row steps (four per segment; H is a multiple of
+    // 64 here), software-pipelined: the router rows of the next step are requested before the
+    // fma chains of the current one start, across segment boundaries.
+    const int nsteps = wave < p.nseg ? 4 * ((p.nseg - wave + 15) / 16) : 0;
+    auto load_rows = [&](int step, half2_t (&dst)[16]) {
+        const int sc = step < nsteps ? step : nsteps - 1;                  // past the end: reread, unused
+        const int row0 = (wave + 16 * (sc >> 2)) * kRouteSeg + (sc & 3) * 16;
+        const global_ptr<const half2_t> src = wcol + (size_t)row0 * wstride;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dst[i] = src[(size_t)i * wstride];
+    };
+    float part[TT][2];
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) part[tt][0] = part[tt][1] = 0.0f;
+    auto run_step = [&](int step, const half2_t (&wv)[16]) {
+        const int seg = wave + 16 * (step >> 2);
+        const int row0 = seg * kRouteSeg + (step & 3) * 16;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {                                       // four rows at a time
+            float4_t xd[TT];
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt) xd[tt] = *(const float4_t*)(s_x + (size_t)tt * p.H + row0 + 4 * q);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float w0 = (float)wv[4 * q + r].x, w1 = (float)wv[4 * q + r].y;
+#pragma unroll
+                for (int tt = 0; tt < TT; ++tt) {
+                    part[tt][0] = __builtin_fmaf(xd[tt][r], w0, part[tt][0]);
+                    part[tt][1] = __builtin_fmaf(xd[tt][r], w1, part[tt][1]);
+                }
+            }
+        }
+        if ((step & 3) == 3) {                                              // the segment is complete
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt) {
+                *(float2_t*)&s_parts[((size_t)seg * TT + tt) * kSlabExperts + 2 * lane] = float2_t{part[tt][0], part[tt][1]};
+                part[tt][0] = part[tt][1] = 0.0f;
+            }
+        }
+    };
+    if (nsteps > 0) {
+        half2_t wa[16], wb[16];
+        load_rows(0, wa);
+#pragma unroll 1
+        for (int step = 0; step < nsteps; step += 2) {
+            load_rows(step + 1, wb);
+            run_step(step, wa);
+            load_rows(step + 2, wa);
+            run_step(step + 1, wb);
+        }
+    }
+    __syncthreads();
+
+    // ---- thread (token, expert of the slab): segments added in order, bias
+    float v = 0.0f;
+    const int tt_mine = threadIdx.x >> 7, c = threadIdx.x & 127;
+    const int e_mine = slab * kSlabExperts + c, t_mine = t0 + tt_mine;
+    const bool mine = tt_mine < TT && e_mine < p.E;
+    if (mine) {
+        for (int seg = 0; seg < p.nseg; ++seg) v += s_parts[((size_t)seg * TT + tt_mine) * kSlabExperts + c];
+        if (p.bias) v += p.bias[e_mine];
+        if (p.logits && t_mine < p.T) p.logits[(size_t)t_mine * p.E + e_mine] = v;
+    }
+    float lg[kRoutePer];
+#pragma unroll
+    for (int i = 0; i < kRoutePer; ++i) lg[i] = -INFINITY;
+    if (nslab == 1) {
+        __syncthreads();                                            // every sum is formed: the segment sums can go
+        if (mine) s_parts[tt_mine * kSlabExperts + c] = v;
+        __syncthreads();
+        if (wave >= TT || t0 + wave >= p.T) return;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            if (lane + 64 * i < p.E) lg[i] = s_parts[wave * kSlabExperts + lane + 64 * i];
+        route_topk_n<2>(lg, lane, p, t0 + wave);
+        return;
+    }
+    // ---- several slabs: logits to memory ([T][E], the head of the segment-sum scratch), the last
+    // slab of the token group to arrive selects
+    float* const all = p.parts;
+    if (mine && t_mine < p.T)
+        __hip_atomic_store(all + (size_t)t_mine * p.E + e_mine, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    wait_own_stores();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned* counter = p.counters + (size_t)grp * kRouteCounterStride;
+        const unsigned old = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (old == (unsigned)(nslab - 1)) ? 1u : 0u;
+        if (s_last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    if (wave >= TT || t0 + wave >= p.T) return;
+    const int t = t0 + wave;
+#pragma unroll
+    for (int i = 0; i < kRoutePer; ++i) {
+        const int e = lane + 64 * i;
+        if (e < p.E) lg[i] = __hip_atomic_load(all + (size_t)t * p.E + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    route_topk(lg, lane, p, t);
+}
+
 // ---------------------------------------------------------------- permute
 
 
@@ -789,6 +938,33 @@ std::string run_route(const void* x, const void* wr, const float* bias, int32_t*
     p.nseg = (H + kRouteSeg - 1) / kRouteSeg;
     if (sort && T == 1) p.sort = *sort;
     const int groups = (T + kRouteTT - 1) / kRouteTT;
+    if (T >= kRouteBigT && E % 2 == 0 && H % kRouteSeg == 0 && p.nseg <= 128 && knobs().moe_route_slab) {
+        // one launch: tokens per workgroup as many as the segment sums leave room for in 64 KiB
+        // of LDS, fewer while that leaves compute units without a workgroup
+        const int nslab = (E + kSlabExperts - 1) / kSlabExperts;
+        int tt = 4;
+        constexpr int kSlabLdsMax = 144 * 1024;
+        while (tt > 1 && (route_slab_lds_bytes(p.nseg, tt) > kSlabLdsMax || (long)nslab * ((T + tt - 1) / tt) < ws.cu_count / 2)) tt /= 2;
+        const int tgroups = (T + tt - 1) / tt;
+        if (route_slab_lds_bytes(p.nseg, tt) <= kSlabLdsMax && (long)tgroups * kRouteCounterStride <= kCounters) {
+            dim3 grid(tgroups, nslab);
+            const size_t lds = (size_t)route_slab_lds_bytes(p.nseg, tt);
+            static bool raised[3][64] = {};
+            if (tt == 4) {
+                raise_dynamic_lds_limit((const void*)moe_route_slab_kernel<4>, kSlabLdsMax, raised[0], "moe_route_slab_kernel shared-memory attribute");
+                hipLaunchKernelGGL(moe_route_slab_kernel<4>, grid, dim3(1024), lds, stream, p);
+            } else if (tt == 2) {
+                raise_dynamic_lds_limit((const void*)moe_route_slab_kernel<2>, kSlabLdsMax, raised[1], "moe_route_slab_kernel shared-memory attribute");
+                hipLaunchKernelGGL(moe_route_slab_kernel<2>, grid, dim3(1024), lds, stream, p);
+            } else {
+                raise_dynamic_lds_limit((const void*)moe_route_slab_kernel<1>, kSlabLdsMax, raised[2], "moe_route_slab_kernel shared-memory attribute");
+                hipLaunchKernelGGL(moe_route_slab_kernel<1>, grid, dim3(1024), lds, stream, p);
+            }
+            hip_ok(hipGetLastError(), "moe_route_slab_kernel launch");
+            return "moe_route_slab_kernel<" + std::to_string(tt) + "> grid=" + std::to_string(nslab) + "x" +
+                   std::to_string(tgroups);
+        }
+    }
     if (T >= kRouteBigT) {
         const int group = route_big_group(E);
         dim3 grid(p.nseg, (T + group - 1) / group);

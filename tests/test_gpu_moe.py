@@ -382,6 +382,36 @@ def test_moe_layer_with_a_gate_on_the_shared_expert(T, H, E, k, I, bits, shared_
         K.moe.layer(1, 1, None, 1, None, 1, None, None, 1, 1 << 30, 1, 128, 8, 2, 128, 0, 4, K.Codebook.MUL1, shared_gate=1)
 
 
+@pytest.mark.parametrize("T,H,E,k", [(64, 2048, 128, 8), (256, 2048, 512, 10), (33, 256, 6, 2), (40, 1024, 258, 5)])
+def test_many_token_routing_in_one_launch_equals_the_two_launch_form(T, H, E, k):
+    """From 32 tokens on (even expert count, hidden a multiple of 64) the routing is one launch in
+    which the segment sums of a token group x a slab of 128 experts meet in LDS;
+    BERTH_MOE_ROUTE_SLAB=0 keeps the partial-sum launch and the finish launch.  Same arithmetic in
+    the same order: the same logits, experts and weights, bit for bit, and the oracle's."""
+    wr = synth.router_weight(5100 + E, H, E)
+    bias = synth.zipf_bias(5101, E)
+    x = (synth.activations(5102 + T, T, H).astype(np.float32) / np.sqrt(H)).astype(np.float16)
+    d_x, d_wr = dev(x.view(np.uint16)), dev(wr.view(np.uint16))
+    d_bias = torch.from_numpy(bias).to(DEV)
+    res = {}
+    for slab in (1, 0):
+        with knobs(BERTH_MOE_ROUTE_SLAB=slab):
+            idx = torch.zeros((T, k), dtype=torch.int32, device=DEV)
+            w = torch.zeros((T, k), dtype=torch.float32, device=DEV)
+            logits = torch.zeros((T, E), dtype=torch.float32, device=DEV)
+            parts = torch.zeros(T * (H // 64) * E, dtype=torch.float32, device=DEV)
+            K.moe.route(d_x.data_ptr(), d_wr.data_ptr(), d_bias.data_ptr(), idx.data_ptr(), w.data_ptr(),
+                        logits.data_ptr(), parts.data_ptr(), T, H, E, k, True)
+            torch.cuda.synchronize()
+            assert ("moe_route_slab_kernel" in K.moe.last_launch()) == bool(slab), K.moe.last_launch()
+            res[slab] = (idx.cpu().numpy(), w.cpu().numpy().view(np.uint32), logits.cpu().numpy().view(np.uint32))
+    for a, b in zip(res[1], res[0]):
+        assert np.array_equal(a, b)
+    oi, ow, ol = O.moe_route(x, wr, k, bias=bias, want_logits=True)
+    assert np.array_equal(res[1][0], oi)
+    assert np.array_equal(res[1][2], ol.view(np.uint32))
+
+
 def test_moe_validation_errors():
     with pytest.raises(K.LaunchError, match="null"):
         K.moe.layer(None, None, None, None, None, None, None, None, None, 0, 1, 128, 8, 2, 128, 0, 4, K.Codebook.MUL1)
