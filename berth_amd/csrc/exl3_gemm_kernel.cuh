@@ -477,8 +477,9 @@ __global__ __launch_bounds__(256, 2) void exl3_gemm_kernel(GemmParams p)
 // rows.  Both kinds sit in one launch, the long tiles first, so the short ones fill in around
 // them (as two launches the 128-row tiles would run alone on a fraction of the compute units).
 // blockIdx.x = column block (whole K per workgroup: no hand-over), blockIdx.y the linear.
-// Measured and dropped: cutting K in two with the split-K hand-over (the shorter units pack
-// better, the hand-over costs more than that gains), and resident workgroups that take units
+// Measured and dropped: cutting K in two with the split-K hand-over, for every tile or for the
+// 128-row tiles only (the shorter units pack better, the hand-over of 128 KB of partial sums per
+// tile costs far more than that gains: 150 -> 183 us per layer), and resident workgroups that take units
 // from a counter (the same schedule as the hardware's, with slower code).
 template <int BITS, int CB>
 __global__ __launch_bounds__(256, 2) void exl3_gemm_mixed_kernel(GemmParams p)
