@@ -400,6 +400,11 @@ __global__ __launch_bounds__(1024) void moe_route_slab_kernel(RouteParams p)
     const int e_ld = e0 < p.E ? e0 : p.E - 2;                       // lanes past the end redo the last pair, unused
     const global_ptr<const half2_t> wcol = (global_ptr<const half2_t>)as_global(p.wr + e_ld);
     const size_t wstride = (size_t)p.E / 2;                         // half2 elements per router row
+    // thread (token, expert of the slab) of the ordered sum further down; its bias is asked for now
+    const int tt_mine = threadIdx.x >> 7, c = threadIdx.x & 127;
+    const int e_mine = slab * kSlabExperts + c, t_mine = t0 + tt_mine;
+    const bool mine = tt_mine < TT && e_mine < p.E;
+    const float bias_mine = mine && p.bias ? p.bias[e_mine] : 0.0f;
     // the tokens' rows go to LDS once, widened to fp32 (tokens past the end: the last token,
     // unused); a step then reads its sixteen rows of every token with wave-uniform addresses
     // (broadcast reads).
@@ -415,25 +420,28 @@ __global__ __launch_bounds__(1024) void moe_route_slab_kernel(RouteParams p)
     }
     __syncthreads();
 
-    // The wave's segments as one run of sixteen-row steps (four per segment; H is a multiple of
-    // 64 here), software-pipelined: the router rows of the next step are requested before the
-    // fma chains of the current one start, across segment boundaries.
-    const int nsteps = wave < p.nseg ? 4 * ((p.nseg - wave + 15) / 16) : 0;
-    auto load_rows = [&](int step, half2_t (&dst)[16]) {
+    // The wave's segments as one run of steps of kStep rows (H is a multiple of 64 here),
+    // software-pipelined: the router rows of the next step are requested before the fma chains
+    // of the current one start, across segment boundaries.  With few tokens a step holds few
+    // fmas, so it takes more rows: the loop is then paced by the loads in flight.
+    constexpr int kStep = TT >= 4 ? 16 : 32;
+    constexpr int kPerSeg = kRouteSeg / kStep;
+    const int nsteps = wave < p.nseg ? kPerSeg * ((p.nseg - wave + 15) / 16) : 0;
+    auto load_rows = [&](int step, half2_t (&dst)[kStep]) {
         const int sc = step < nsteps ? step : nsteps - 1;                  // past the end: reread, unused
-        const int row0 = (wave + 16 * (sc >> 2)) * kRouteSeg + (sc & 3) * 16;
+        const int row0 = (wave + 16 * (sc / kPerSeg)) * kRouteSeg + (sc % kPerSeg) * kStep;
         const global_ptr<const half2_t> src = wcol + (size_t)row0 * wstride;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[i] = src[(size_t)i * wstride];
+        for (int i = 0; i < kStep; ++i) dst[i] = src[(size_t)i * wstride];
     };
     float part[TT][2];
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) part[tt][0] = part[tt][1] = 0.0f;
-    auto run_step = [&](int step, const half2_t (&wv)[16]) {
-        const int seg = wave + 16 * (step >> 2);
-        const int row0 = seg * kRouteSeg + (step & 3) * 16;
+    auto run_step = [&](int step, const half2_t (&wv)[kStep]) {
+        const int seg = wave + 16 * (step / kPerSeg);
+        const int row0 = seg * kRouteSeg + (step % kPerSeg) * kStep;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {                                       // four rows at a time
+        for (int q = 0; q < kStep / 4; ++q) {                               // four rows at a time
             float4_t xd[TT];
 #pragma unroll
             for (int tt = 0; tt < TT; ++tt) xd[tt] = *(const float4_t*)(s_x + (size_t)tt * p.H + row0 + 4 * q);
@@ -447,7 +455,7 @@ __global__ __launch_bounds__(1024) void moe_route_slab_kernel(RouteParams p)
                 }
             }
         }
-        if ((step & 3) == 3) {                                              // the segment is complete
+        if (step % kPerSeg == kPerSeg - 1) {                                // the segment is complete
 #pragma unroll
             for (int tt = 0; tt < TT; ++tt) {
                 *(float2_t*)&s_parts[((size_t)seg * TT + tt) * kSlabExperts + 2 * lane] = float2_t{part[tt][0], part[tt][1]};
@@ -456,7 +464,7 @@ __global__ __launch_bounds__(1024) void moe_route_slab_kernel(RouteParams p)
         }
     };
     if (nsteps > 0) {
-        half2_t wa[16], wb[16];
+        half2_t wa[kStep], wb[kStep];
         load_rows(0, wa);
 #pragma unroll 1
         for (int step = 0; step < nsteps; step += 2) {
@@ -470,12 +478,9 @@ __global__ __launch_bounds__(1024) void moe_route_slab_kernel(RouteParams p)
 
     // ---- thread (token, expert of the slab): segments added in order, bias
     float v = 0.0f;
-    const int tt_mine = threadIdx.x >> 7, c = threadIdx.x & 127;
-    const int e_mine = slab * kSlabExperts + c, t_mine = t0 + tt_mine;
-    const bool mine = tt_mine < TT && e_mine < p.E;
     if (mine) {
         for (int seg = 0; seg < p.nseg; ++seg) v += s_parts[((size_t)seg * TT + tt_mine) * kSlabExperts + c];
-        if (p.bias) v += p.bias[e_mine];
+        if (p.bias) v += bias_mine;
         if (p.logits && t_mine < p.T) p.logits[(size_t)t_mine * p.E + e_mine] = v;
     }
     float lg[kRoutePer];
