@@ -479,7 +479,10 @@ __global__ __launch_bounds__(256, 2) void exl3_gemm_kernel(GemmParams p)
 // blockIdx.x = column block (whole K per workgroup: no hand-over), blockIdx.y the linear.
 // Measured and dropped: cutting K in two with the split-K hand-over, for every tile or for the
 // 128-row tiles only (the shorter units pack better, the hand-over of 128 KB of partial sums per
-// tile costs far more than that gains: 150 -> 183 us per layer), and resident workgroups that take units
+// tile costs far more than that gains: 150 -> 183 us per layer), 128-column units whose four waves
+// cut K in two and add through LDS (gate + up of 256 tokens x 512 experts 61.3 -> 54.9 us, but its
+// down projection 32.0 -> 39.6 and both launches of 64 tokens x 128 experts 5 - 6 us slower: twice
+// the units pay twice the problem -> expert -> pointer chain), and resident workgroups that take units
 // from a counter (the same schedule as the hardware's, with slower code).
 template <int BITS, int CB>
 __global__ __launch_bounds__(256, 2) void exl3_gemm_mixed_kernel(GemmParams p)
