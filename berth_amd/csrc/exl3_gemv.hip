@@ -124,9 +124,7 @@ static std::string run_stream(const Workspace& ws, const StreamPlan& pl, StreamP
 {
     throw_pending_device_fault(ws);
     int mask = stream_lut_mask(bits, (unsigned long long)pl.q * kStreamWaves * 256 * bits);
-#ifndef BERTH_STREAM_EXTRA_MASKS
     if (mask != 0) mask = 0xA;          // the one hybrid mask that is instantiated
-#endif
     p.accum = ws.accum;
     p.fault = ws.fault_dev;
     p.spin_limit = spin_limit();

@@ -28,12 +28,6 @@ static void launch_stream_bits(const StreamParams& p, int lutmask, dim3 grid, hi
     };
     switch (lutmask) {
     case 0x0: by_input(std::integral_constant<int, 0x0>{}); break;
-#ifdef BERTH_STREAM_EXTRA_MASKS
-    case 0x2: launch_stream_one<BITS, CB, kInPlain, 0x2>(p, grid, stream); break;
-    case 0x8: launch_stream_one<BITS, CB, kInPlain, 0x8>(p, grid, stream); break;
-    case 0xE: launch_stream_one<BITS, CB, kInPlain, 0xE>(p, grid, stream); break;
-    case 0xF: launch_stream_one<BITS, CB, kInPlain, 0xF>(p, grid, stream); break;
-#endif
     default: by_input(std::integral_constant<int, 0xA>{}); break;
     }
 }

@@ -246,11 +246,8 @@ __device__ __forceinline__ void nested_tail(unsigned count, F&& f)
 // memory's latency takes at the rate the decode consumes them; deeper rings only lengthen the
 // queues that everything else (the first loads of the launch, the hand-over at its end) waits in
 // (27B layer set at 4 bits per weight, four launches: 67.1 us with four, 65.3 with two).
-#ifndef BERTH_STREAM_RING
-#define BERTH_STREAM_RING 2
-#endif
 template <int BITS> struct StreamRing {
-    static constexpr int depth = BERTH_STREAM_RING;
+    static constexpr int depth = 2;
 };
 
 // a pointer every lane of the wave agrees on, moved to scalar registers
