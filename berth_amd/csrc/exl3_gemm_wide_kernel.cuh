@@ -13,11 +13,14 @@
 //   MFMA     wave w owns rows 128*(w/4) .. +127 and columns 64*(w%4) .. +63 of the tile:
 //            32 MFMAs per macro-step, A and B operands from LDS.
 //
-// A and B tiles are double-buffered; per macro-step one barrier.  Every wave decodes its
-// share of the next macro-step, then issues its MFMAs on the current one (running the two
-// waves of a SIMD in opposite order, so that one's decode faces the other's MFMAs, was
-// measured and is no faster: the two kinds of work do not overlap on a SIMD).  Trellis
-// registers run four macro-steps ahead of the decode, A registers two.
+// A and B tiles are double-buffered; per macro-step one barrier.  Inside a macro-step a wave
+// issues its 32 MFMAs on the current buffers two at a time and, behind every two, one
+// sixteenth of its decode for the next macro-step (a pair of weights), so the vector pipe
+// works while the matrix pipe is busy: the order is given to the scheduler as groups
+// (operand reads one chunk ahead, two MFMAs, eight vector instructions).  As two blocks
+// (all of the decode, then all of the MFMAs) the 27B gate projection at 512 rows took 141 us,
+// interleaved it takes 124.  Trellis registers run four macro-steps ahead of the decode, A
+// registers two.
 //
 // Handoff between workgroups that share a tile and the epilogue are those of the
 // 128-row kernel (partial sums in register layout, summed in k order by the last
@@ -130,24 +133,49 @@ __device__ __forceinline__ void gemm_tile_wide(const GemmParams& p, const int ti
 #pragma unroll
             for (int i = 0; i < 4; ++i) *(u32x4_t*)(ad + i * 16) = ar[i];
         };
-        auto mfma_step = [&](int buf) {
+        // One macro-step: the 32 MFMAs on buffer `buf`, and behind every two of them one
+        // sixteenth of the decode of the next macro-step (a pair of weights: two windows, two
+        // hashes, one packed fma).  Written in that order here; the scheduler groups after the
+        // call keep the compiler from collecting the MFMAs and the decode back into two blocks.
+        // Operands of the next two MFMAs are read one chunk ahead; the A rows of the next
+        // macro-step go to LDS in the first four chunks, the decoded weights at the end.  Row
+        // blocks past the end of the rows are multiplied too (their A rows repeat the last row)
+        // and never stored: the loop has no branch.
+        auto fused_step = [&](int buf, const uint32_t (&tr)[BITS], const u32x4_t (&ar)[4]) {
             const unsigned char* ao = a_op + (size_t)buf * kWideABytes;
             const unsigned char* bo = b_op + (size_t)buf * kWideBBytes;
+            unsigned char* ad = a_dst + (size_t)(buf ^ 1) * kWideABytes;
+            unsigned char* bd = b_dst + (size_t)(buf ^ 1) * kWideBBytes;
+            const uint32_t prev = fetch_prev(lane, tr[BITS - 1]);
+            const LaneWindows<BITS> win(tr, prev);
+            uint32_t w2[16];
+            half8_t b0 = *(const half8_t*)(bo);
+            half8_t b1 = *(const half8_t*)(bo + 32 * 16);
+            half8_t an = *(const half8_t*)(ao);
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
-                const half8_t b0 = *(const half8_t*)(bo + (size_t)(2 * kk) * 256 * 16);
-                const half8_t b1 = *(const half8_t*)(bo + (size_t)(2 * kk) * 256 * 16 + 32 * 16);
-                half8_t an[2];
-                an[0] = *(const half8_t*)(ao + kk * 32);
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb) {
-                    if (mb + 1 < MB) an[(mb + 1) & 1] = *(const half8_t*)(ao + (size_t)(mb + 1) * 32 * (kWideAStride * 2) + kk * 32);
-                    if (mb * 32 < rows_here) {                      // uniform in the wave
-                        acc[mb][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(an[mb & 1], b0, acc[mb][0], 0, 0, 0);
-                        acc[mb][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(an[mb & 1], b1, acc[mb][1], 0, 0, 0);
+            for (int g = 0; g < 16; ++g) {
+                const int kk = g >> 2, mb = g & 3;
+                const half8_t a_now = an, b0_now = b0, b1_now = b1;
+                if (g < 15) {
+                    const int kn = (g + 1) >> 2, mn = (g + 1) & 3;
+                    an = *(const half8_t*)(ao + (size_t)mn * 32 * (kWideAStride * 2) + kn * 32);
+                    if (mn == 0) {
+                        b0 = *(const half8_t*)(bo + (size_t)(2 * kn) * 256 * 16);
+                        b1 = *(const half8_t*)(bo + (size_t)(2 * kn) * 256 * 16 + 32 * 16);
                     }
                 }
+                acc[mb][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_now, b0_now, acc[mb][0], 0, 0, 0);
+                acc[mb][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_now, b1_now, acc[mb][1], 0, 0, 0);
+                w2[g] = decode_pair<CB>(win.state(2 * g), win.state(2 * g + 1));
+                if (g < 4) *(u32x4_t*)(ad + g * 16) = ar[g];
             }
+#pragma unroll
+            for (int f = 0; f < 2; ++f)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const u32x4_t q = {w2[2 * f + h], w2[4 + 2 * f + h], w2[8 + 2 * f + h], w2[12 + 2 * f + h]};
+                    *(u32x4_t*)(bd + ((size_t)h * 256 + 8 * f) * 16) = q;
+                }
         };
 
         // prologue: macro-step 0 decoded into buffer 0; the rings hold trellis 1..4 and A 1..2
@@ -168,10 +196,29 @@ __device__ __forceinline__ void gemm_tile_wide(const GemmParams& p, const int ti
             for (int u = 0; u < 4; ++u) {
                 if (s + u >= nsteps) break;                         // workgroup-uniform
                 const int buf = u & 1;
-                decode_and_fill(buf ^ 1, tr_ring[(u + 1) & 3], a_ring[(u + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                fused_step(buf, tr_ring[(u + 1) & 3], a_ring[(u + 1) & 1]);
                 issue_tr(s + u + 5, tr_ring[(u + 1) & 3]);
                 issue_a(s + u + 3, a_ring[(u + 1) & 1]);
-                mfma_step(buf);
+                // the order the scheduler has to keep: operand reads one chunk ahead, two MFMAs,
+                // a sixteenth of the decode
+                __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+#define BERTH_WIDE_CHUNK(reads)                                                    \
+    __builtin_amdgcn_sched_group_barrier(0x100, reads, 0);                         \
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                             \
+    __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+#define BERTH_WIDE_CHUNK_A(reads)                                                  \
+    BERTH_WIDE_CHUNK(reads)                                                        \
+    __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                BERTH_WIDE_CHUNK_A(1) BERTH_WIDE_CHUNK_A(1) BERTH_WIDE_CHUNK_A(1) BERTH_WIDE_CHUNK_A(3)
+                BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(3)
+                BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(3)
+                BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(1)
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+#undef BERTH_WIDE_CHUNK_A
+#undef BERTH_WIDE_CHUNK
+                __builtin_amdgcn_sched_group_barrier(0x200, 4, 0);
                 __syncthreads();
             }
         }
