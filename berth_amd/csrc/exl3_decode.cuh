@@ -165,6 +165,7 @@ struct LaneWindows {
     uint32_t c[BITS + 1];   // big-endian 32-bit chunks: c[0] = prev, c[1..] = own
     uint32_t m[BITS + 1];   // m[j] = low 16 of c[j-1] : high 16 of c[j]  (j >= 1)
 
+    LaneWindows() = default;
     __device__ __forceinline__ LaneWindows(const uint32_t (&own)[BITS], uint32_t prev)
     {
         c[0] = __builtin_amdgcn_alignbit(prev, prev, 16);

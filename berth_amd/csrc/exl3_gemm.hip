@@ -84,16 +84,17 @@ std::string launch_gemm(const LinearArgs& a)
     const int rows256 = knobs().gemm_rows256;
     // 128-row tiles rarely divide over the compute units (272 tiles on 256 units leave most of
     // the chip idle for the second half of the launch): deal the (tile, k-block) units out evenly.
-    // 128-row tiles: one workgroup per compute unit, two when a workgroup still gets 16 k-blocks
-    // or more (measured on the 27B shapes at 512 rows: gate/up and down are fastest with two, q
-    // and o with one, where fewer workgroups share a tile).  256-row tiles (more than 128 rows,
+    // 128-row tiles: one workgroup per compute unit (a wave interleaves its own decode with its
+    // MFMAs, so a second workgroup per unit adds nothing and more workgroups share a tile: the 27B
+    // down projection at 512 rows takes 147 us with 256 workgroups, 160 with 512).  256-row tiles
+    // (more than 128 rows,
     // wide outputs): a weight is decoded once per 256 rows; one workgroup of eight waves fills a
     // compute unit.
     auto balanced = [&](int mb) {
         const int mtiles = (a.size_m + mb * 32 - 1) / (mb * 32);
         const long tiles = (long)nblocks * mtiles;
         const long units = tiles * KB;
-        long slots = (mb == 4 && units >= 32L * ws.cu_count) ? 2L * ws.cu_count : ws.cu_count;
+        long slots = ws.cu_count;
         if (balance > 1) slots = balance;
         const long G = units < slots ? units : slots;
         const long per_wg = units / G;                                   // >= 1

@@ -201,12 +201,21 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
         const uint32_t* tbase = lin.trellis + (size_t)half_id * row_dw +
                                 (size_t)((nw >> 4) + (slot >> 3)) * tile_dw + (slot & 7) * BITS;
 
-        // Both operands run one k-block ahead in registers: the trellis dwords of the
-        // wave's four steps (nxt) and this thread's share of the A tile (a_nxt, 32 bytes
-        // per 256-thread pass).  The A tile is double-buffered in LDS, so a k-block costs
-        // one barrier.
+        // Operands run ahead in registers: this thread's share of the next k-block's A tile
+        // (a_nxt, 32 bytes per 256-thread pass; the tile is double-buffered in LDS, so a
+        // k-block costs one barrier) and the trellis dwords of the wave's four steps (ring),
+        // each reloaded for the next k-block as soon as its step is decoded.
+        //
+        // A step's 32 weights per lane are 16 pairs; the even pairs are the B operands for
+        // k 0..7 of each lane's 16 (A operand a0), the odd pairs those for k 8..15 (a1).  The
+        // loop runs in half-steps: the eight MFMAs of one half are issued two at a time, and
+        // behind every two a quarter of the decode of the NEXT half (the odd pairs of the same
+        // step, or the even pairs of the next step, which across the barrier is step 0 of the
+        // next k-block), so the vector pipe decodes while the matrix pipe multiplies.  Row
+        // blocks past the end of the rows are multiplied too (their A rows are zero): the loop
+        // has no branch.  The order is given to the scheduler as groups after each half-step.
         constexpr int kAPasses = BM * 8 / 256;
-        uint32_t nxt[4][BITS];
+        uint32_t ring[4][BITS];
         uint4 a_nxt[kAPasses][2];
         const int a_row = threadIdx.x >> 3, a_ch = threadIdx.x & 7;       // + 32 rows per pass
         auto load_a = [&](int kb) {
@@ -223,26 +232,34 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
                 a_nxt[ps][1] = v1;
             }
         };
-        auto load_b = [&](int kb) {
-            const uint32_t* nb = tbase + (size_t)(kb * 8) * row_dw;
+        auto load_b_step = [&](int kb, int st) {
+            const uint32_t* nb = tbase + (size_t)(kb * 8 + 2 * st) * row_dw;
     #pragma unroll
-            for (int st = 0; st < 4; ++st)
-    #pragma unroll
-                for (int j = 0; j < BITS; ++j) nxt[st][j] = nb[(size_t)(2 * st) * row_dw + j];
+            for (int j = 0; j < BITS; ++j) ring[st][j] = nb[j];
         };
+        // the eight pairs of one half, numbered j = 4f + q: out[f][q] = pair 4q + 2f + h
+        auto decode_pairs = [&](const LaneWindows<BITS>& w, int h, int j0, int n, uint32_t (&out)[2][4]) {
+    #pragma unroll
+            for (int j = j0; j < j0 + n; ++j) {
+                const int f = j >> 2, q = j & 3;
+                const int pr = 4 * q + 2 * f + h;
+                out[f][q] = decode_pair<CB>(w.state(2 * pr), w.state(2 * pr + 1));
+            }
+        };
+        uint32_t b_half[2][2][4];                       // [which half-step buffer][f][q]
+        LaneWindows<BITS> win;
         if (kr.kb0 < kr.kb1) {
             load_a(kr.kb0);
-            if (active) load_b(kr.kb0);
+            if (active) {
+    #pragma unroll
+                for (int st = 0; st < 4; ++st) load_b_step(kr.kb0, st);
+                win = LaneWindows<BITS>(ring[0], fetch_prev(lane, ring[0][BITS - 1]));
+                decode_pairs(win, 0, 0, 8, b_half[0]);
+            }
         }
 
         int buf = 0;
         for (int kb = kr.kb0; kb < kr.kb1; kb += kr.step, buf ^= 1) {
-            uint32_t cur[4][BITS];
-    #pragma unroll
-            for (int st = 0; st < 4; ++st)
-    #pragma unroll
-                for (int j = 0; j < BITS; ++j) cur[st][j] = nxt[st][j];
-
             // publish this k-block's A tile; the other buffer may still be read by slower waves
             _Float16* a_buf = a_tile + (size_t)buf * BM * kAStride;
     #pragma unroll
@@ -251,38 +268,51 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
                 dst[0] = a_nxt[ps][0];
                 dst[1] = a_nxt[ps][1];
             }
-            if (kb + kr.step < kr.kb1) {
-                load_a(kb + kr.step);
-                if (active) load_b(kb + kr.step);
-            }
+            // the next k-block (on the last one the same again: read and ignored, no branch)
+            const int nkb = kb + kr.step < kr.kb1 ? kb + kr.step : kb;
+            load_a(nkb);
             __syncthreads();
 
             if (active) {
+                const _Float16* a_lane = a_buf + slot * kAStride + 16 * half_id;
+                // A operand of half-step hs = 2 * st + h, row block mb: k = 32 * st + 16 * half_id + 8 * h .. + 7 of the k-block
+                auto a_operand = [&](int hs, int mb) {
+                    return *(const half8_t*)(a_lane + mb * 32 * kAStride + 32 * (hs >> 1) + 8 * (hs & 1));
+                };
+                half8_t a_op = a_operand(0, 0);
     #pragma unroll
-                for (int st = 0; st < 4; ++st) {
-                    uint32_t prev = fetch_prev(lane, cur[st][BITS - 1]);
-                    uint32_t w2[16];
-                    decode_lane<BITS, CB>(cur[st], prev, w2);
-                    half8_t b[2][2];
-    #pragma unroll
-                    for (int f = 0; f < 2; ++f)
-    #pragma unroll
-                        for (int h = 0; h < 2; ++h) {
-                            const uint4 q = {w2[2 * f + h], w2[4 + 2 * f + h], w2[8 + 2 * f + h], w2[12 + 2 * f + h]};
-                            b[f][h] = __builtin_bit_cast(half8_t, q);
-                        }
-                    // A operand: row = mb*32 + slot, k = 32*st + 16*half_id + 8h .. +7 inside the k-block
+                for (int hs = 0; hs < 8; ++hs) {
+                    const int st = hs >> 1, h = hs & 1;
+                    __builtin_amdgcn_sched_barrier(0);
+                    uint32_t (&b_cur)[2][4] = b_half[h];
+                    uint32_t (&b_nx)[2][4] = b_half[h ^ 1];
+                    const half8_t b0 = __builtin_bit_cast(half8_t, uint4{b_cur[0][0], b_cur[0][1], b_cur[0][2], b_cur[0][3]});
+                    const half8_t b1 = __builtin_bit_cast(half8_t, uint4{b_cur[1][0], b_cur[1][1], b_cur[1][2], b_cur[1][3]});
+                    if (h == 1) {
+                        // the step after this one: its windows, then (below) its even pairs
+                        const int ns = (st + 1) & 3;
+                        win = LaneWindows<BITS>(ring[ns], fetch_prev(lane, ring[ns][BITS - 1]));
+                    }
     #pragma unroll
                     for (int mb = 0; mb < MB; ++mb) {
-                        if (MB > 1 && mb * 32 >= rows_here) break;          // workgroup-uniform
-                        const _Float16* arow = a_buf + (mb * 32 + slot) * kAStride + 32 * st + 16 * half_id;
-                        const half8_t a0 = *(const half8_t*)(arow);
-                        const half8_t a1 = *(const half8_t*)(arow + 8);
-                        acc[mb][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b[0][0], acc[mb][0], 0, 0, 0);
-                        acc[mb][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, b[1][0], acc[mb][1], 0, 0, 0);
-                        acc[mb][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b[0][1], acc[mb][0], 0, 0, 0);
-                        acc[mb][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b[1][1], acc[mb][1], 0, 0, 0);
+                        const half8_t a_now = a_op;
+                        if (mb + 1 < MB) a_op = a_operand(hs, mb + 1);
+                        else if (hs < 7) a_op = a_operand(hs + 1, 0);
+                        acc[mb][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_now, b0, acc[mb][0], 0, 0, 0);
+                        acc[mb][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_now, b1, acc[mb][1], 0, 0, 0);
+                        decode_pairs(win, h ^ 1, mb * (8 / MB), 8 / MB, b_nx);
                     }
+                    // the step's dwords are decoded once its odd pairs exist: request the next k-block's
+                    if (h == 0) load_b_step(nkb, st);
+    #define BERTH_GEMM_CHUNK(valu0, valu1)                                              \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                              \
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                              \
+        __builtin_amdgcn_sched_group_barrier(0x002, valu0, 0);                          \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                              \
+        __builtin_amdgcn_sched_group_barrier(0x002, valu1, 0);
+                    static_assert(MB == 4, "the groups below describe eight MFMAs per half-step");
+                    BERTH_GEMM_CHUNK(9, 9) BERTH_GEMM_CHUNK(9, 9) BERTH_GEMM_CHUNK(9, 9) BERTH_GEMM_CHUNK(9, 9)
+    #undef BERTH_GEMM_CHUNK
                 }
             }
         }
