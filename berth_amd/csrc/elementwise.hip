@@ -52,6 +52,62 @@ __global__ __launch_bounds__(256) void had_r_128_kernel(const T* __restrict__ in
     }
 }
 
+// The rotated inputs of a bundle in one launch: blockIdx.y is the slab, whose sign scales come
+// from a device list of pointers or from the pointers passed by value.
+struct SuhTable {
+    const _Float16* suh[kBundleMaxSlices];
+};
+__global__ __launch_bounds__(256) void had_r_128_slabs_kernel(const _Float16* __restrict__ in, size_t in_stride,
+                                                              _Float16* __restrict__ out, size_t out_stride,
+                                                              const uint64_t* __restrict__ suh_list, SuhTable tab,
+                                                              long blocks, int col_blocks)
+{
+    const int slab = blockIdx.y;
+    const _Float16* scale = suh_list ? (const _Float16*)suh_list[slab] : tab.suh[slab];
+    in += (size_t)slab * in_stride;
+    out += (size_t)slab * out_stride;
+    const int lane = threadIdx.x & 63;
+    const int l16 = lane & 15;
+    const long waves = (long)gridDim.x * 4;
+    const long groups = (blocks + 3) / 4;
+    for (long g = (long)blockIdx.x * 4 + (threadIdx.x >> 6); g < groups; g += waves) {
+        const long blk = g * 4 + (lane >> 4);
+        const bool live = blk < blocks;
+        const long b = live ? blk : blocks - 1;             // lanes past the end redo the last block and store nothing
+        const int cb = (int)(b % col_blocks);
+        const size_t at = (size_t)b * 128 + 8 * l16;
+        const half8_t x = *(const half8_t*)(in + at);
+        const half8_t s8 = *(const half8_t*)(scale + cb * 128 + 8 * l16);
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (float)x[i] * (float)s8[i];
+        had128_row16(v, lane);
+        half8_t o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = (_Float16)(v[i] * kRsqrt128);
+        if (live) *(half8_t*)(out + at) = o;
+    }
+}
+
+std::string launch_had_r_128_slabs(const void* in, size_t in_stride, void* out, size_t out_stride, const void* suh_list,
+                                   const void* const* suh_host, int slabs, int rows, int cols, hipStream_t stream)
+{
+    if (slabs < 1 || slabs > 65535) throw std::runtime_error("had_r_128 slabs: between 1 and 65535 slabs");
+    SuhTable tab{};
+    if (!suh_list) {
+        if (slabs > kBundleMaxSlices) throw std::runtime_error("had_r_128 slabs: too many slabs for the by-value table");
+        for (int i = 0; i < slabs; ++i) tab.suh[i] = (const _Float16*)suh_host[i];
+    }
+    const int col_blocks = cols / 128;
+    const long blocks = (long)rows * col_blocks;
+    const long wgs = (blocks + 15) / 16;
+    const dim3 grid((unsigned)(wgs < 4096 ? wgs : 4096), (unsigned)slabs);
+    hipLaunchKernelGGL(had_r_128_slabs_kernel, grid, dim3(256), 0, stream, (const _Float16*)in, in_stride, (_Float16*)out,
+                       out_stride, (const uint64_t*)suh_list, tab, blocks, col_blocks);
+    hip_ok(hipGetLastError(), "had_r_128 slabs launch");
+    return "had_r_128_slabs_kernel grid=" + std::to_string(grid.x) + "x" + std::to_string(grid.y) + " block=256";
+}
+
 std::string launch_had_r_128(const void* in, void* out, const void* scale, int pre_scale,
                              int rows, int cols, int fp32, hipStream_t stream)
 {

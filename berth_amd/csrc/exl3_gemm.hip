@@ -10,6 +10,7 @@
 namespace berth {
 
 static_assert(kGemmWrittenBase * 2 == kCounters, "the GEMM keeps two counters per tile");
+static_assert(kGemmMaxSlices == kBundleMaxSlices, "one limit for the by-value slices of a bundle");
 
 // one translation unit per codebook (exl3_gemm_cb{0,1,2}.hip) keeps the build parallel
 void launch_gemm_cb0(const GemmParams& p, int bits, int mb, hipStream_t stream, std::string& desc, dim3 grid);
@@ -50,6 +51,70 @@ static int gemm_counter_stride(long tiles)
     return stride;
 }
 
+// Tile shape and work split of a dense launch: `nblocks` column blocks of 256 (all slices of
+// a bundle together), size_m rows.  Fills the split fields of p and launches.
+static void dispatch_dense(const Workspace& ws, GemmParams& p, int k_bits, int codebook, int size_m, int size_k,
+                           int nblocks, hipStream_t stream, std::string& desc)
+{
+    // 128-row tiles decode a weight once per 128 rows, but need enough tiles to spread
+    // over the chip; narrow outputs (few column tiles) run as 32-row tiles instead
+    p.cstride = gemm_counter_stride((long)nblocks * ((size_m + 31) / 32));
+    const long tiles128 = (long)nblocks * ((size_m + 127) / 128);
+    const int mb_plain = (size_m <= 32 || tiles128 * 4 < ws.cu_count) ? 1 : 4;
+    const int KB = size_k / 128;
+    p.tile0 = 0;
+    const int balance = knobs().gemm_balanced;
+    // 0: never 256-row tiles; 1 (default): where they are faster; 2: wherever they are possible
+    const int rows256 = knobs().gemm_rows256;
+    // 128-row tiles rarely divide over the compute units (272 tiles on 256 units leave most of
+    // the chip idle for the second half of the launch): deal the (tile, k-block) units out evenly.
+    // 128-row tiles: one workgroup per compute unit (a wave interleaves its own decode with its
+    // MFMAs, so a second workgroup per unit adds nothing and more workgroups share a tile: the 27B
+    // down projection at 512 rows takes 147 us with 256 workgroups, 160 with 512).  256-row tiles
+    // (more than 128 rows, wide outputs): a weight is decoded once per 256 rows; one workgroup of
+    // eight waves fills a compute unit.
+    auto balanced = [&](int mb) {
+        const int mtiles = (size_m + mb * 32 - 1) / (mb * 32);
+        const long tiles = (long)nblocks * mtiles;
+        const long units = tiles * KB;
+        long slots = ws.cu_count;
+        if (balance > 1) slots = balance;
+        const long G = units < slots ? units : slots;
+        const long per_wg = units / G;                                   // >= 1
+        const long parts = (KB + per_wg - 1) / per_wg + 1;               // workgroups that can share a tile
+        const size_t part_bytes = (size_t)4 * mb * 2 * 16 * 64 * sizeof(float);
+        if (!(tiles <= kCounters / 2 && per_wg < KB && units < (1L << 30) &&
+              (size_t)tiles * parts * part_bytes <= kPartialBytes))
+            return false;
+        p.tiles_y = mtiles;
+        p.S = 1;
+        p.units = (int)units;
+        p.unit_q = (int)(units / G);
+        p.unit_r = (int)(units % G);
+        p.max_parts = (int)parts;
+        gemm_bits(p, k_bits, codebook, mb, stream, desc, dim3((unsigned)G, 1, 1));
+        return true;
+    };
+    bool done = false;
+    if (balance && mb_plain == 4) {
+        // 256-row tiles pay when there are enough of them that few workgroups share a tile
+        // (measured at 512 rows: gate/up 5120x17408, 136 tiles, 148 -> 139 us; q, o and down
+        // with 40..48 tiles are 5 % slower than with 128-row tiles)
+        const long tiles256 = (long)nblocks * ((size_m + 255) / 256);
+        if (size_m > 128 && (rows256 >= 2 || (rows256 == 1 && tiles256 * 2 >= ws.cu_count))) done = balanced(8);
+        if (!done) done = balanced(4);
+    }
+    if (!done) {
+        const int mtiles = (size_m + mb_plain * 32 - 1) / (mb_plain * 32);
+        const long tiles = (long)nblocks * mtiles;
+        p.tiles_y = mtiles;
+        p.units = 0;
+        p.S = gemm_split(ws, tiles, KB, mb_plain);
+        gemm_bits(p, k_bits, codebook, mb_plain, stream, desc, dim3((unsigned)(tiles * p.S), 1, 1));
+    }
+    hip_ok(hipGetLastError(), "exl3_gemm_kernel launch");
+}
+
 std::string launch_gemm(const LinearArgs& a)
 {
     if (a.size_k % 128 != 0) throw std::runtime_error("exl3 linear: size_k must be a multiple of 128");
@@ -70,67 +135,83 @@ std::string launch_gemm(const LinearArgs& a)
     p.out_fp32 = a.out_fp32;
     p.partials = ws.partials;
     p.counters = ws.counters;
-    // 128-row tiles decode a weight once per 128 rows, but need enough tiles to spread
-    // over the chip; narrow outputs (few column tiles) run as 32-row tiles instead
-    const int nblocks = (a.size_n + 255) / 256;
-    p.cstride = gemm_counter_stride((long)nblocks * ((a.size_m + 31) / 32));
-    const long tiles128 = (long)nblocks * ((a.size_m + 127) / 128);
-    const int mb_plain = (a.size_m <= 32 || tiles128 * 4 < ws.cu_count) ? 1 : 4;
-    const int KB = a.size_k / 128;
     std::string desc;
-    p.tile0 = 0;
-    const int balance = knobs().gemm_balanced;
-    // 0: never 256-row tiles; 1 (default): where they are faster; 2: wherever they are possible
-    const int rows256 = knobs().gemm_rows256;
-    // 128-row tiles rarely divide over the compute units (272 tiles on 256 units leave most of
-    // the chip idle for the second half of the launch): deal the (tile, k-block) units out evenly.
-    // 128-row tiles: one workgroup per compute unit (a wave interleaves its own decode with its
-    // MFMAs, so a second workgroup per unit adds nothing and more workgroups share a tile: the 27B
-    // down projection at 512 rows takes 147 us with 256 workgroups, 160 with 512).  256-row tiles
-    // (more than 128 rows,
-    // wide outputs): a weight is decoded once per 256 rows; one workgroup of eight waves fills a
-    // compute unit.
-    auto balanced = [&](int mb) {
-        const int mtiles = (a.size_m + mb * 32 - 1) / (mb * 32);
-        const long tiles = (long)nblocks * mtiles;
-        const long units = tiles * KB;
-        long slots = ws.cu_count;
-        if (balance > 1) slots = balance;
-        const long G = units < slots ? units : slots;
-        const long per_wg = units / G;                                   // >= 1
-        const long parts = (KB + per_wg - 1) / per_wg + 1;               // workgroups that can share a tile
-        const size_t part_bytes = (size_t)4 * mb * 2 * 16 * 64 * sizeof(float);
-        if (!(tiles <= kCounters / 2 && per_wg < KB && units < (1L << 30) &&
-              (size_t)tiles * parts * part_bytes <= kPartialBytes))
-            return false;
-        p.tiles_y = mtiles;
-        p.S = 1;
-        p.units = (int)units;
-        p.unit_q = (int)(units / G);
-        p.unit_r = (int)(units % G);
-        p.max_parts = (int)parts;
-        gemm_bits(p, a.k_bits, a.codebook, mb, a.stream, desc, dim3((unsigned)G, 1, 1));
-        return true;
-    };
-    bool done = false;
-    if (balance && mb_plain == 4) {
-        // 256-row tiles pay when there are enough of them that few workgroups share a tile
-        // (measured at 512 rows: gate/up 5120x17408, 136 tiles, 148 -> 139 us; q, o and down
-        // with 40..48 tiles are 5 % slower than with 128-row tiles)
-        const long tiles256 = (long)nblocks * ((a.size_m + 255) / 256);
-        if (a.size_m > 128 && (rows256 >= 2 || (rows256 == 1 && tiles256 * 2 >= ws.cu_count))) done = balanced(8);
-        if (!done) done = balanced(4);
-    }
-    if (!done) {
-        const int mtiles = (a.size_m + mb_plain * 32 - 1) / (mb_plain * 32);
-        const long tiles = (long)nblocks * mtiles;
-        p.tiles_y = mtiles;
-        p.units = 0;
-        p.S = gemm_split(ws, tiles, KB, mb_plain);
-        gemm_bits(p, a.k_bits, a.codebook, mb_plain, a.stream, desc, dim3((unsigned)(tiles * p.S), 1, 1));
-    }
-    hip_ok(hipGetLastError(), "exl3_gemm_kernel launch");
+    dispatch_dense(ws, p, a.k_bits, a.codebook, a.size_m, a.size_k, (a.size_n + 255) / 256, a.stream, desc);
     return d0 + " + " + desc + (a.out_fp32 ? " out=f32" : " out=f16");
+}
+
+// berth_ops_mgemm with more than 8 rows: the bundle's linears as one dense MFMA launch behind
+// one launch that rotates every distinct input (slab s of a_had = Hh(input(s) * suh[s])).
+std::string launch_gemm_bundle(const MgemmArgs& m)
+{
+    if (m.size_k % 128 != 0) throw std::runtime_error("exl3_mgemm: size_k must be a multiple of 128");
+    const bool sliced = m.had_src_list != nullptr;
+    if (m.host_lists && m.bszm_out > kGemmMaxSlices)
+        throw std::runtime_error("exl3_mgemm (host lists): at most " + std::to_string(kGemmMaxSlices) + " slices");
+    LaunchScope scope(m.stream);
+    Workspace& ws = scope.ws;
+    throw_pending_device_fault(ws);
+    const int slabs = sliced ? m.num_had_src : m.bszm_out;
+    const size_t slab_stride = (size_t)m.size_m * m.size_k;
+    GemmParams p{};
+    p.fault = ws.fault_dev;
+    p.spin_limit = spin_limit();
+    p.a_had[0] = (const _Float16*)m.a_had;
+    p.c[0] = m.c;
+    p.M = m.size_m;
+    p.K = m.size_k;
+    p.N = m.size_n;
+    p.out_fp32 = m.c_fp32;
+    p.partials = ws.partials;
+    p.counters = ws.counters;
+    p.num_slices = m.bszm_out;
+    p.slab_stride = slab_stride;
+    const void* suh_host[kGemmMaxSlices] = {};
+    if (m.host_lists) {
+        const uint64_t* b = (const uint64_t*)m.b_list;
+        const uint64_t* su = (const uint64_t*)m.suh_list;
+        const uint64_t* sv = (const uint64_t*)m.svh_list;
+        if (slabs > kGemmMaxSlices) throw std::runtime_error("exl3_mgemm (host lists): too many input rotations");
+        for (int i = 0; i < slabs; ++i) suh_host[i] = (const void*)su[i];
+        for (int i = 0; i < m.bszm_out; ++i) {
+            GemmSlice& g = p.slice[i];
+            g.trellis = (const uint32_t*)b[i];
+            g.svh = (const _Float16*)sv[i];
+            if (sliced) {
+                const int src = m.had_src_list[i];
+                if (src < 0 || src >= m.num_had_src) throw std::runtime_error("exl3_mgemm (host lists): had_src_list entry out of range");
+                if (m.size_n_list[i] < 0 || m.size_n_list[i] > m.size_n || m.size_n_list[i] % 128 != 0)
+                    throw std::runtime_error("exl3_mgemm (host lists): size_n_list entry must be a multiple of 128 within size_n");
+                g.c = (void*)((const uint64_t*)m.c_ptrs)[i];
+                g.width = m.size_n_list[i];
+                g.n_stride = m.n_stride_list[i];
+                g.had_slab = src;
+            } else {
+                g.c = (char*)m.c + (size_t)i * m.size_m * m.size_n * (m.c_fp32 ? 4 : 2);
+                g.width = m.size_n;
+                g.n_stride = m.size_n;
+                g.had_slab = i;
+            }
+        }
+    } else {
+        p.b_list = (const uint64_t*)m.b_list;
+        p.svh_list = (const uint64_t*)m.svh_list;
+        if (sliced) {
+            p.c_ptrs = (const uint64_t*)m.c_ptrs;
+            p.size_n_list = m.size_n_list;
+            p.n_stride_list = m.n_stride_list;
+            p.had_src_list = m.had_src_list;
+        }
+    }
+    const size_t in_stride = (!sliced && m.bszm_in > 1) ? slab_stride : 0;
+    std::string d0 = launch_had_r_128_slabs(m.a, in_stride, m.a_had, slab_stride, m.host_lists ? nullptr : m.suh_list,
+                                            suh_host, slabs, m.size_m, m.size_k, m.stream);
+    const long nblocks = (long)m.bszm_out * ((m.size_n + 255) / 256);
+    if (nblocks * ((m.size_m + 31) / 32) > kCounters / 2) throw std::runtime_error("exl3_mgemm: too many output tiles");
+    std::string desc;
+    dispatch_dense(ws, p, m.k_bits, m.codebook, m.size_m, m.size_k, (int)nblocks, m.stream, desc);
+    return std::string(sliced ? "sliced x" : "uniform x") + std::to_string(m.bszm_out) + (m.host_lists ? " by value " : " ") + d0 +
+           " + " + desc + (m.c_fp32 ? " out=f32" : " out=f16");
 }
 
 // grouped: problems of at most 32 * g.mb rows each; a_had rows are in problem order

@@ -30,6 +30,18 @@
 
 namespace berth {
 
+// one linear of a bundle whose lists the host knows
+struct GemmSlice {
+    const uint32_t* trellis;
+    const _Float16* svh;
+    void* c;
+    int width;                  // columns of this linear (a multiple of 128, at most N)
+    int n_stride;               // columns of the whole weight the slice is cut from: elements between
+                                // output rows and, in tiles of 16, between the tile rows of its trellis
+    int had_slab;               // which rotated copy of the input it multiplies
+};
+constexpr int kGemmMaxSlices = 16;
+
 struct GemmParams {
     const _Float16* a_had[2];   // [rows][K], already rotated (one per linear of the launch)
     ExpertLin lin;              // dense mode
@@ -65,7 +77,74 @@ struct GemmParams {
     // index to *fault (host-visible memory; may be null) and leaves the tile unwritten.
     unsigned* fault;
     unsigned spin_limit;
+    // Bundles (crates/berth-kernels/src/ops.rs:264-293 with more than 8 rows): num_slices
+    // linears that share K and the row count run as one dense launch.  Every slice owns
+    // ceil(N / 256) column blocks of the launch (N = the widest slice); a block past the end of
+    // a narrower slice is empty.  The slice's tensors come from the device lists when b_list is
+    // set (uniform mode: c_ptrs null, outputs [slice][M][N] behind c[0], rotated input = slab
+    // `slice`; sliced mode: all seven lists), else from `slice` by value.  a_had[0] holds the
+    // rotated inputs, slab_stride elements apart.
+    int num_slices;             // 0: one linear (lin, c[0], a_had[0])
+    size_t slab_stride;
+    const uint64_t* b_list;
+    const uint64_t* svh_list;
+    const uint64_t* c_ptrs;
+    const int* size_n_list;
+    const int* n_stride_list;
+    const int* had_src_list;
+    GemmSlice slice[kGemmMaxSlices];
 };
+
+// the tensors of the column block `nblk` of a dense launch
+struct TileView {
+    ExpertLin lin;
+    const _Float16* a_had;
+    void* cout;
+    int N;                      // columns of the linear
+    int ldc;                    // elements between output rows
+    int nblk;                   // column block inside the linear
+    bool empty;                 // the block lies past the end of its (narrower) slice
+};
+__device__ __forceinline__ TileView dense_tile_view(const GemmParams& p, const int nblk)
+{
+    TileView v;
+    v.lin = p.lin;
+    v.a_had = p.a_had[0];
+    v.cout = p.c[0];
+    v.N = p.N;
+    v.ldc = p.N;
+    v.nblk = nblk;
+    v.empty = false;
+    if (p.num_slices > 0) {
+        const int per = (p.N + 255) >> 8;
+        const int sl = nblk / per;
+        v.nblk = nblk - sl * per;
+        int slab = sl;
+        if (p.b_list) {
+            v.lin.trellis = (const uint32_t*)p.b_list[sl];
+            v.lin.svh = (const _Float16*)p.svh_list[sl];
+            if (p.c_ptrs) {
+                v.N = p.size_n_list[sl];
+                v.ldc = p.n_stride_list[sl];
+                slab = p.had_src_list[sl];
+                v.cout = (void*)p.c_ptrs[sl];
+            } else {
+                v.cout = (char*)p.c[0] + (size_t)sl * p.M * p.N * (p.out_fp32 ? 4 : 2);
+            }
+        } else {
+            const GemmSlice& g = p.slice[sl];
+            v.lin.trellis = g.trellis;
+            v.lin.svh = g.svh;
+            v.cout = g.c;
+            v.N = g.width;
+            v.ldc = g.n_stride;
+            slab = g.had_slab;
+        }
+        v.a_had = p.a_had[0] + (size_t)slab * p.slab_stride;
+        v.empty = v.nblk * 256 >= v.N;
+    }
+    return v;
+}
 
 // The finisher's wait for `counter` to reach `want`, bounded.  Called by one thread.  A
 // workgroup that has arrived is running and depends on nothing, so the counter gets there
@@ -108,12 +187,23 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
     const int wave = threadIdx.x >> 6;
     const int half_id = lane >> 5;                      // which of the two tile rows
     const int slot = lane & 31;                         // MFMA row / column slot
-    const int n0 = nblk * 256;
     int m0 = tile_y * BM;
     int m_end = p.M;
     ExpertLin lin = p.lin;
     const _Float16* a_had = p.a_had[0];
     void* cout = p.c[0];
+    int N = p.N, ldc = p.N, nblk_lin = nblk;
+    if constexpr (DENSE) {
+        const TileView v = dense_tile_view(p, nblk);
+        if (v.empty) return;                            // the same for every workgroup that shares the tile
+        lin = v.lin;
+        a_had = v.a_had;
+        cout = v.cout;
+        N = v.N;
+        ldc = v.ldc;
+        nblk_lin = v.nblk;
+    }
+    const int n0 = nblk_lin * 256;
     if constexpr (!DENSE) {
         // (dynamic indexing of the parameter block: kept out of the dense instantiations, where
         // it would force the whole block into private memory)
@@ -127,8 +217,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
     }
     const int rows_here = min(BM, m_end - m0);          // >= 1
     const int nw = n0 + wave * 64;                      // first column of this wave
-    const bool active = nw < p.N;
-    const int tn = p.N >> 4;
+    const bool active = nw < N;
+    const int tn = ldc >> 4;                            // tiles per tile row of the weight (of the whole weight, for a slice)
     constexpr int tile_dw = 8 * BITS;
     const size_t row_dw = (size_t)tn * tile_dw;
     const int KB = p.K >> 7;
@@ -420,7 +510,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk) {
         const int gn = n0 + blk * 128;
-        sv_blk[blk] = gn < p.N ? ((global_ptr<const half8_t>)as_global(lin.svh + gn))[l16] : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        sv_blk[blk] = gn < N ? ((global_ptr<const half8_t>)as_global(lin.svh + gn))[l16] : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
     }
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
@@ -443,7 +533,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
             const int vec = pass * 16 + wave * 4 + (lane >> 4);
             const int row = vec >> 1, blk = vec & 1;
             const int gn = n0 + blk * 128;
-            if (row < rows_blk && gn < p.N) {
+            if (row < rows_blk && gn < N) {
                 float v[8];
                 const float4_t* zp = (const float4_t*)&z_tile[row * kZStride + blk * 128 + 8 * l16];
                 const float4_t z0 = zp[0], z1 = zp[1];
@@ -453,7 +543,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
                 const half8_t sv = blk ? sv_blk[1] : sv_blk[0];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) v[i] = (v[i] * kRsqrt128) * (float)sv[i];
-                const size_t at = (size_t)(m0 + mb * 32 + row) * p.N + gn + 8 * l16;
+                const size_t at = (size_t)(m0 + mb * 32 + row) * ldc + gn + 8 * l16;
                 if (p.out_fp32) {
                     global_ptr<float4_t> dst = (global_ptr<float4_t>)(as_global((float*)cout) + at);
                     dst[0] = float4_t{v[0], v[1], v[2], v[3]};
@@ -480,7 +570,7 @@ __global__ __launch_bounds__(256, 2) void exl3_gemm_kernel(GemmParams p)
     extern __shared__ __align__(16) unsigned char smem[];
     const int unit = blockIdx.x / p.S;
     const int split = blockIdx.x - unit * p.S;
-    const int nblocks = (p.N + 255) >> 8;
+    const int nblocks = ((p.N + 255) >> 8) * (p.num_slices > 0 ? p.num_slices : 1);
     KRange kr;
     kr.kb0 = split;
     kr.kb1 = p.K >> 7;
@@ -567,7 +657,7 @@ template <int BITS, int CB, int MB>
 __device__ __forceinline__ void gemm_segment(const GemmParams& p, const int w, const int u, const int stop,
                                              unsigned char* smem)
 {
-    const int nblocks = (p.N + 255) >> 8;
+    const int nblocks = ((p.N + 255) >> 8) * (p.num_slices > 0 ? p.num_slices : 1);
     const int KB = p.K >> 7;
     const int tile = u / KB;
     const int t0 = tile * KB;                                   // the tile's first unit

@@ -52,17 +52,20 @@ __device__ __forceinline__ void gemm_tile_wide(const GemmParams& p, const int ti
     const int cq = wave8 & 3;                           // column quarter of the MFMA tile
     const int slot = lane & 31;
     const int kh = lane >> 5;
-    const int n0 = nblk * 256;
+    const TileView view = dense_tile_view(p, nblk);
+    if (view.empty) return;                             // the same for every workgroup that shares the tile
+    const int n0 = view.nblk * 256;
     const int m_end = p.M;
     const int m_tile = tile_y * 256;
     const int m0 = m_tile + rh * 128;
     const int rows_here = min(128, m_end - m0);         // <= 0: this row half is empty
     const int rows_first = min(128, m_end - m_tile);    // rows of the first half, >= 1
-    const ExpertLin lin = p.lin;
-    const _Float16* a_had = p.a_had[0];
-    void* cout = p.c[0];
-    const bool active = n0 + cq * 64 < p.N;             // this wave's 64 output columns exist
-    const int tn = p.N >> 4;
+    const ExpertLin lin = view.lin;
+    const _Float16* a_had = view.a_had;
+    void* cout = view.cout;
+    const int N = view.N, ldc = view.ldc;
+    const bool active = n0 + cq * 64 < N;               // this wave's 64 output columns exist
+    const int tn = ldc >> 4;                            // tiles per tile row of the weight (of the whole weight, for a slice)
     constexpr int tile_dw = 8 * BITS;
     const size_t row_dw = (size_t)tn * tile_dw;
 
@@ -84,7 +87,7 @@ __device__ __forceinline__ void gemm_tile_wide(const GemmParams& p, const int ti
         const int du = lane & 7;
         // tile columns past the end of the weight are decoded from the first half of the
         // block instead (never used): no branch around loads
-        const int dtc_ld = (n0 >> 4) + dtc < tn ? dtc : dtc - 8;
+        const int dtc_ld = (n0 >> 4) + dtc < (N >> 4) ? dtc : dtc - 8;
         const global_ptr<const uint32_t> tbase = as_global(lin.trellis) + (size_t)dtr * row_dw +
                                                  (size_t)((n0 >> 4) + dtc_ld) * tile_dw + du * BITS;
         // B tile destinations of this lane: column dtc*16 + du + 8f, k octet 2*dtr + h
@@ -308,7 +311,7 @@ __device__ __forceinline__ void gemm_tile_wide(const GemmParams& p, const int ti
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk) {
         const int gn = n0 + blk * 128;
-        sv_blk[blk] = gn < p.N ? ((global_ptr<const half8_t>)as_global(lin.svh + gn))[l16] : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        sv_blk[blk] = gn < N ? ((global_ptr<const half8_t>)as_global(lin.svh + gn))[l16] : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
     }
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
@@ -330,7 +333,7 @@ __device__ __forceinline__ void gemm_tile_wide(const GemmParams& p, const int ti
             const int vec = pass * 16 + cq * 4 + (lane >> 4);
             const int row = vec >> 1, blk = vec & 1;
             const int gn = n0 + blk * 128;
-            if (row < rows_blk && gn < p.N) {
+            if (row < rows_blk && gn < N) {
                 float v[8];
                 const float4_t* zp = (const float4_t*)&z_tile[row * kZStride + blk * 128 + 8 * l16];
                 const float4_t z0 = zp[0], z1 = zp[1];
@@ -340,7 +343,7 @@ __device__ __forceinline__ void gemm_tile_wide(const GemmParams& p, const int ti
                 const half8_t sv = blk ? sv_blk[1] : sv_blk[0];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) v[i] = (v[i] * kRsqrt128) * (float)sv[i];
-                const size_t at = (size_t)(m0 + mb * 32 + row) * p.N + gn + 8 * l16;
+                const size_t at = (size_t)(m0 + mb * 32 + row) * ldc + gn + 8 * l16;
                 if (p.out_fp32) {
                     global_ptr<float4_t> dst = (global_ptr<float4_t>)(as_global((float*)cout) + at);
                     dst[0] = float4_t{v[0], v[1], v[2], v[3]};
@@ -360,7 +363,7 @@ template <int BITS, int CB>
 __device__ __forceinline__ void gemm_segment_wide(const GemmParams& p, const int w, const int u, const int stop,
                                                   unsigned char* smem)
 {
-    const int nblocks = (p.N + 255) >> 8;
+    const int nblocks = ((p.N + 255) >> 8) * (p.num_slices > 0 ? p.num_slices : 1);
     const int KB = p.K >> 7;
     const int tile = u / KB;
     const int t0 = tile * KB;

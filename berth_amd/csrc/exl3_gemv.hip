@@ -324,7 +324,7 @@ std::string launch_gemv_pair(const PairArgs& a)
 std::string launch_mgemm(const MgemmArgs& m)
 {
     if (m.size_k % 128 != 0) throw std::runtime_error("exl3_mgemm: size_k must be a multiple of 128");
-    if (m.size_m > 8) throw std::runtime_error("exl3_mgemm: more than 8 rows is not built (use one linear per call)");
+    if (m.size_m > 8) return launch_gemm_bundle(m);
     LaunchScope scope(m.stream);
     Workspace& ws = scope.ws;
     throw_pending_device_fault(ws);

@@ -236,6 +236,13 @@ struct MgemmArgs {
     bool host_lists = false;    // the seven lists are host memory (one row, the streaming kernel only)
 };
 std::string launch_mgemm(const MgemmArgs& args);
+// more than 8 rows: the bundle as one dense MFMA launch
+std::string launch_gemm_bundle(const MgemmArgs& args);
+// out slab s = Hh(in(s) * suh(s)) for s < slabs (fp16; in(s) = in + s * in_stride, out slabs
+// out_stride elements apart); suh(s) from the device list, or from the host array when the list is null
+std::string launch_had_r_128_slabs(const void* in, size_t in_stride, void* out, size_t out_stride, const void* suh_list,
+                                   const void* const* suh_host, int slabs, int rows, int cols, hipStream_t stream);
+constexpr int kBundleMaxSlices = 16;    // slices of a bundle whose lists travel by value
 
 // rows 1..8: VALU dot-product kernel.  Returns the launch description.  `scratch`: the
 // split-K scratch to use instead of the device's lazily allocated workspace.

@@ -243,7 +243,9 @@ class Exl3MultiLinear:
     """Several EXL3 linears that share one input, launched as one sliced
     `exl3_mgemm` (the qkv bundles of crates/berth-engine/src/attn.rs:1934-1973 and
     gdn.rs:1102-1130; list layout from crates/berth-kernels/src/ops.rs:264-293):
-    every source is cut into slices of the greatest common width."""
+    every source is cut into slices of the greatest common width.  Any row count: one
+    row runs the streaming kernel, 2..8 the dot-product kernel, more the MFMA kernels
+    (the reference sends 9..32 rows through the same call, prefill.rs:81-85)."""
 
     def __init__(self, gpu: Gpu, sources: list[Exl3Linear]):
         import math
@@ -286,10 +288,12 @@ class Exl3MultiLinear:
         self._h_c = None
         self.host_lists = self.slices <= 16
 
-    def forward(self, gpu: Gpu, a: torch.Tensor, outs: list[torch.Tensor], out: OutDtype, rows: int = 1) -> None:
-        """a fp16 [rows][K]; outs[i] [rows][N_i] of `out` for source i."""
-        if rows < 1 or rows > 8:
-            raise InputError("multi-linear: rows must be in 1..=8")
+    def forward(self, gpu: Gpu, a: torch.Tensor, outs: list[torch.Tensor], out: OutDtype, rows: int = 1,
+                by_value: bool = True) -> None:
+        """a fp16 [rows][K]; outs[i] [rows][N_i] of `out` for source i.  `by_value` False
+        keeps the lists in device memory whatever the row count."""
+        if rows < 1:
+            raise InputError("multi-linear: rows must be positive")
         if rows * self.size_k > self.a_had.numel() // len(self.sources):
             self.a_had = torch.zeros(len(self.sources) * rows * self.size_k, dtype=torch.float16, device=gpu.device)
         esz = 4 if out == OutDtype.F32 else 2
@@ -299,17 +303,19 @@ class Exl3MultiLinear:
             self._c_ptrs = torch.tensor(ptrs, dtype=torch.int64, device=gpu.device)
             self._h_c = np.array(ptrs, dtype=np.uint64)
             self._c_key = key
-        if rows == 1 and self.host_lists:
+        # lists by value: one row through the streaming kernel, more than 8 rows through the MFMA
+        # kernels (2..8 rows read the device lists)
+        if by_value and ((rows == 1 and self.host_lists) or (rows > 8 and self.slices <= 16)):
             h = self._h
             try:
                 K.ops.exl3_mgemm_hostlists(ptr(a), h["b"].ctypes.data, ptr(outs[0]), h["suh"].ctypes.data, ptr(self.a_had),
-                                           h["svh"].ctypes.data, 1, self.size_k, self.width, self.k_bits, self.codebook,
+                                           h["svh"].ctypes.data, rows, self.size_k, self.width, self.k_bits, self.codebook,
                                            out, 1, self.slices, h["size_n"].ctypes.data, self._h_c.ctypes.data,
                                            h["stride"].ctypes.data, h["src"].ctypes.data, len(self.sources),
                                            gpu.raw_stream())
                 return
             except K.LaunchError as err:
-                if "host lists" not in str(err):
+                if rows > 1 or "host lists" not in str(err):
                     raise
                 self.host_lists = False         # too small for the streaming kernel: device lists from now on
         K.ops.exl3_mgemm(ptr(a), ptr(self.b_list), ptr(outs[0]), ptr(self.suh_list), ptr(self.a_had),

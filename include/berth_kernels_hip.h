@@ -205,8 +205,12 @@ int berth_ops_cat_f16_last(const void* embedding, const void* hidden, void* out,
  * size_n_list[s] <= size_n = slice width; had_src_list[s] = source index;
  * a_had holds num_had_src slabs of size_m*size_k.  Uniform mode (lists NULL):
  * bszm_out linears of one shape, inputs a[i] (bszm_in == bszm_out) or a[0]
- * (bszm_in == 1), outputs c[i] contiguous.  size_m <= 8.  Returns 1 on success
- * (the reference returns its kernel-shape tag there), -1 on error. */
+ * (bszm_in == 1), outputs c[i] contiguous.  Any row count: up to 8 rows run the
+ * dot-product kernels (the rotation of the input inside the launch), more rows one
+ * launch that rotates the input once per source / linear and one dense MFMA launch
+ * over all slices (the reference sends 9..32 rows of its fused q/k/v and gate/up
+ * bundles through this call, crates/berth-engine/src/prefill.rs:81-85).  Returns 1
+ * on success (the reference returns its kernel-shape tag there), -1 on error. */
 int berth_ops_mgemm(const void* a, const void* b_list, void* c, const void* suh_list, void* a_had,
                     const void* svh_list, int size_m, int size_k, int size_n, int k_bits,
                     int codebook, int c_fp32, int bszm_in, int bszm_out, const int* size_n_list,
@@ -217,9 +221,10 @@ int berth_ops_mgemm(const void* a, const void* b_list, void* c, const void* suh_
  * ints; a, c and a_had stay device pointers).  For callers that built the lists themselves and
  * still hold them: the problems then travel by value in the kernel arguments, which takes the
  * two dependent device reads (list entry, then the source's scale pointer) out of the head of
- * the launch (1.5 - 2.5 us of a 12 - 30 us launch).  Serves one row, at most 16 slices, and
- * weights large enough for the one-row streaming kernel; anything else returns -1 and the
- * caller passes device lists to berth_ops_mgemm.  Same return values and error slot. */
+ * the launch (1.5 - 2.5 us of a 12 - 30 us launch).  Serves one row (at most 16 slices and
+ * weights large enough for the one-row streaming kernel) and more than 8 rows (at most 16
+ * slices, the MFMA kernels); anything else returns -1 and the caller passes device lists to
+ * berth_ops_mgemm.  Same return values and error slot. */
 int berth_ops_mgemm_hostlists(const void* a, const void* b_list, void* c, const void* suh_list, void* a_had,
                               const void* svh_list, int size_m, int size_k, int size_n, int k_bits,
                               int codebook, int c_fp32, int bszm_in, int bszm_out, const int* size_n_list,
