@@ -653,8 +653,10 @@ def mlp_block_bench(gpu, layers, bits: int, steps: int):
 
 def prefill_bench(gpu, layers, bits: int, rows: int, steps: int):
     """BASELINE.json configs[2]: the same 27B-shaped linears at `rows` = 512 tokens,
-    fp16 activations N(0,1), fp16/fp32 outputs with fp32 accumulation, through
-    berth_prefill_exl3_linear (Hadamard pre-pass + decode-in-GEMM MFMA kernel)."""
+    fp16 activations N(0,1), fp16/fp32 outputs with fp32 accumulation: seven calls of
+    berth_prefill_exl3_linear (Hadamard pre-pass + decode-in-GEMM MFMA kernel), and the same
+    work with q/k/v and gate/up as bundles (berth_ops_mgemm: one rotation launch and one dense
+    MFMA launch per bundle), which is what the decode benchmark's four launches do at one row."""
     import torch
 
     from berth_amd import synth
@@ -667,44 +669,67 @@ def prefill_bench(gpu, layers, bits: int, rows: int, steps: int):
                            device=gpu.device) for n in ORDER}
     flops = sum(2.0 * rows * K * N for K, N in (synth.SHAPES_27B[n] for n in ORDER))
 
-    def step(i):
+    def step_seven(i):
         lin = layers[i % len(layers)]
         for n in ORDER:
             l = lin[n]
             l.forward_rows(gpu, scratch, xin[l.size_k], outs[n], rows, OutDtype.F32 if OUT_FP32[n] else OutDtype.F16)
 
-    for i in range(3):
-        step(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        step(i)
-    torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / steps
-    eager_ms, launch = dt * 1e3, "eager"
-    # one pass over the rotated weight sets recorded into a HIP graph and replayed
-    n = len(layers)
-    graph = torch.cuda.CUDAGraph()
-    side = torch.cuda.Stream(device=gpu.device)
-    side.wait_stream(torch.cuda.current_stream(gpu.device))
-    with torch.cuda.stream(side):
-        for i in range(n):
+    def step_bundles(i):
+        # q/k/v and gate/up share their inputs: each group is one berth_ops_mgemm call (lists by value)
+        lin = layers[i % len(layers)]
+        lin["qkv"].forward(gpu, xin[5120], [outs["q_proj"], outs["k_proj"], outs["v_proj"]], OutDtype.F16, rows)
+        l = lin["o_proj"]
+        l.forward_rows(gpu, scratch, xin[l.size_k], outs["o_proj"], rows, OutDtype.F32 if OUT_FP32["o_proj"] else OutDtype.F16)
+        lin["gate_up"].forward(gpu, xin[5120], [outs["gate_proj"], outs["up_proj"]], OutDtype.F16, rows)
+        l = lin["down_proj"]
+        l.forward_rows(gpu, scratch, xin[l.size_k], outs["down_proj"], rows,
+                       OutDtype.F32 if OUT_FP32["down_proj"] else OutDtype.F16)
+
+    def timed(step):
+        for i in range(3):
             step(i)
         torch.cuda.synchronize()
-        with torch.cuda.graph(graph, stream=side):
+        t0 = time.perf_counter()
+        for i in range(steps):
+            step(i)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        eager_ms, launch = dt * 1e3, "eager"
+        # one pass over the rotated weight sets recorded into a HIP graph and replayed
+        n = len(layers)
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream(device=gpu.device)
+        side.wait_stream(torch.cuda.current_stream(gpu.device))
+        with torch.cuda.stream(side):
             for i in range(n):
                 step(i)
-    torch.cuda.current_stream(gpu.device).wait_stream(side)
-    replays = max(2, steps // n)
-    graph.replay()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(replays):
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(n):
+                    step(i)
+        torch.cuda.current_stream(gpu.device).wait_stream(side)
+        replays = max(2, steps // n)
         graph.replay()
-    torch.cuda.synchronize()
-    graph_dt = (time.perf_counter() - t0) / (replays * n)
-    if graph_dt < dt:
-        dt, launch = graph_dt, f"hip graph of {n} layer sets"
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(replays):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_dt = (time.perf_counter() - t0) / (replays * n)
+        if graph_dt < dt:
+            dt, launch = graph_dt, f"hip graph of {n} layer sets"
+        return dt, eager_ms, launch
+
+    seven_dt, seven_eager_ms, seven_launch = timed(step_seven)
+    bundled = all("qkv" in lin and "gate_up" in lin for lin in layers) and all(
+        not OUT_FP32[n] for n in ("q_proj", "k_proj", "v_proj", "gate_proj", "up_proj"))
+    if bundled:
+        dt, eager_ms, launch = timed(step_bundles)
+        calls = "four calls: q/k/v and gate/up as berth_ops_mgemm bundles, o and down berth_prefill_exl3_linear"
+    else:
+        dt, eager_ms, launch = seven_dt, seven_eager_ms, seven_launch
+        calls = "seven calls of berth_prefill_exl3_linear"
 
     # Beside it: the vendor library's dense fp16 GEMM (torch.matmul) on already
     # decoded fp16 weights of the same seven shapes.  It reads 4x the weight bytes
@@ -730,7 +755,10 @@ def prefill_bench(gpu, layers, bits: int, rows: int, steps: int):
     torch.cuda.empty_cache()
     return {"rows": rows, "ms_per_layer_set": round(dt * 1e3, 3), "tflops": round(flops / dt / 1e12, 1),
             "mfma_peak_tflops": 2500.0, "frac_of_fp16_mfma_peak": round(flops / dt / 2.5e15, 4),
-            "tokens_per_s": round(rows / dt, 0), "launch": launch, "eager_ms_per_layer_set": round(eager_ms, 3),
+            "tokens_per_s": round(rows / dt, 0), "launch": launch, "calls": calls,
+            "eager_ms_per_layer_set": round(eager_ms, 3),
+            "seven_calls": {"ms_per_layer_set": round(seven_dt * 1e3, 3), "tflops": round(flops / seven_dt / 1e12, 1),
+                            "launch": seven_launch},
             "vendor_dense_fp16_gemm": {"what": "torch.matmul on decoded fp16 weights, same shapes and rows",
                                        "ms_per_layer_set": round(dense_us * 1e-3, 3),
                                        "tflops": round(flops / dense_us / 1e6, 1)}}

@@ -83,7 +83,7 @@ static void dispatch_dense(const Workspace& ws, GemmParams& p, int k_bits, int c
         const long per_wg = units / G;                                   // >= 1
         const long parts = (KB + per_wg - 1) / per_wg + 1;               // workgroups that can share a tile
         const size_t part_bytes = (size_t)4 * mb * 2 * 16 * 64 * sizeof(float);
-        if (!(tiles <= kCounters / 2 && per_wg < KB && units < (1L << 30) &&
+        if (!(tiles <= kCounters / 2 && units < (1L << 30) &&
               (size_t)tiles * parts * part_bytes <= kPartialBytes))
             return false;
         p.tiles_y = mtiles;

@@ -675,22 +675,19 @@ __device__ __forceinline__ void gemm_segment(const GemmParams& p, const int w, c
     gemm_tile<BITS, CB, MB, true>(p, t / nblocks, t % nblocks, kr, 0, smem);
 }
 
-// The launcher uses this kernel when a range is at most one tile long, so a range has at
-// most two segments: the end of one tile and the start of the next.
+// A range runs through the end of one tile, any whole tiles after it and the start of another.
 template <int BITS, int CB, int MB>
 __global__ __launch_bounds__(256, 2) void exl3_gemm_balanced_kernel(GemmParams p)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     const int KB = p.K >> 7;
     const int w = die_major_index((int)blockIdx.x, (int)gridDim.x);
-    const int u = range_start(p, w);
     const int u_end = range_start(p, w + 1);
-    const int t1 = (u / KB + 1) * KB;
-    const int stop = min(u_end, t1);
-    gemm_segment<BITS, CB, MB>(p, w, u, stop, smem);
-    if (stop < u_end) {
-        __syncthreads();                                        // the epilogue's LDS tile is the next A tile
-        gemm_segment<BITS, CB, MB>(p, w, stop, u_end, smem);
+    for (int u = range_start(p, w); u < u_end;) {
+        const int stop = min(u_end, (u / KB + 1) * KB);
+        gemm_segment<BITS, CB, MB>(p, w, u, stop, smem);
+        u = stop;
+        if (u < u_end) __syncthreads();                         // the epilogue's LDS tile is the next A tile
     }
 }
 

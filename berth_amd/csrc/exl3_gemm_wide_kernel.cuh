@@ -389,14 +389,12 @@ __global__ __launch_bounds__(512, 1) void exl3_gemm_wide_kernel(GemmParams p)
     extern __shared__ __align__(16) unsigned char smem[];
     const int KB = p.K >> 7;
     const int w = die_major_index((int)blockIdx.x, (int)gridDim.x);
-    const int u = range_start(p, w);
     const int u_end = range_start(p, w + 1);
-    const int t1 = (u / KB + 1) * KB;
-    const int stop = min(u_end, t1);
-    gemm_segment_wide<BITS, CB>(p, w, u, stop, smem);
-    if (stop < u_end) {
-        __syncthreads();                                        // the epilogue's LDS tile is the next A tile
-        gemm_segment_wide<BITS, CB>(p, w, stop, u_end, smem);
+    for (int u = range_start(p, w); u < u_end;) {
+        const int stop = min(u_end, (u / KB + 1) * KB);
+        gemm_segment_wide<BITS, CB>(p, w, u, stop, smem);
+        u = stop;
+        if (u < u_end) __syncthreads();                         // the epilogue's LDS tile is the next A tile
     }
 }
 
