@@ -412,6 +412,102 @@ private:
     DeviceBuffer<float> bias_;
 };
 
+// Several EXL3 linears that share one input, as one sliced berth_ops_mgemm (the q/k/v bundle
+// of crates/berth-engine/src/attn.rs:1934-1973 and gdn.rs:1102-1130; list layout
+// crates/berth-kernels/src/ops.rs:264-293): every source is cut into slices of the greatest
+// common width.  Any row count: one row and more than 8 rows pass the lists by value when
+// there are at most 16 slices, 2..8 rows read them from device memory.
+class MultiLinear {
+public:
+    MultiLinear(const Gpu& gpu, std::vector<const Exl3Linear*> sources) : sources_(std::move(sources))
+    {
+        if (sources_.empty()) throw InputError("multi-linear: no sources");
+        size_k_ = sources_[0]->size_k();
+        k_bits_ = sources_[0]->k_bits();
+        codebook_ = sources_[0]->codebook();
+        int width = 0;
+        for (const Exl3Linear* s : sources_) {
+            if (s->size_k() != size_k_ || s->k_bits() != k_bits_ || s->codebook() != codebook_)
+                throw InputError("multi-linear: sources must share in-features, bit rate and codebook");
+            if (s->has_bias()) throw InputError("multi-linear: a source with a bias runs as its own linear");
+            int a = width, b = s->size_n();
+            while (b) { const int t = a % b; a = b; b = t; }
+            width = a;
+        }
+        if (width % 128) throw InputError("multi-linear: slice width must be a multiple of 128");
+        width_ = width;
+        const uint64_t tile_bytes = (uint64_t)16 * k_bits_ * 2;
+        for (size_t si = 0; si < sources_.size(); ++si) {
+            const berth_exl3_lin e = sources_[si]->table_entry();
+            suh_.push_back((uint64_t)(uintptr_t)e.suh);
+            for (int n0 = 0; n0 < sources_[si]->size_n(); n0 += width) {
+                b_.push_back((uint64_t)(uintptr_t)e.trellis + (uint64_t)(n0 / 16) * tile_bytes);
+                svh_.push_back((uint64_t)(uintptr_t)e.svh + (uint64_t)n0 * 2);
+                stride_.push_back(sources_[si]->size_n());
+                src_.push_back((int)si);
+                n0_.push_back(n0);
+                size_n_.push_back(width);
+            }
+        }
+        d_b_ = DeviceBuffer<uint64_t>::from_host(gpu, b_);
+        d_svh_ = DeviceBuffer<uint64_t>::from_host(gpu, svh_);
+        d_suh_ = DeviceBuffer<uint64_t>::from_host(gpu, suh_);
+        d_stride_ = DeviceBuffer<int>::from_host(gpu, stride_);
+        d_src_ = DeviceBuffer<int>::from_host(gpu, src_);
+        d_size_n_ = DeviceBuffer<int>::from_host(gpu, size_n_);
+        gpu.synchronize();                                      // the host vectors may move from here on
+    }
+
+    int slices() const { return (int)b_.size(); }
+    int width() const { return width_; }
+
+    // a fp16 [rows][K]; outs[i] = device address of source i's output [rows][N_i] in `out`
+    void forward(const Gpu& gpu, const DeviceBuffer<Half>& a, const std::vector<uint64_t>& outs, int rows, OutDtype out)
+    {
+        if (rows < 1) throw InputError("multi-linear: rows must be positive");
+        if (outs.size() != sources_.size()) throw InputError("multi-linear: one output per source");
+        if (a.len() < (size_t)rows * size_k_) throw InputError("multi-linear: input too small");
+        const size_t need = sources_.size() * (size_t)rows * size_k_;
+        if (a_had_.len() < need) a_had_ = DeviceBuffer<Half>::zeroed(gpu, need);
+        const size_t esz = out_bytes(out);
+        std::vector<uint64_t> c(b_.size());
+        for (size_t i = 0; i < c.size(); ++i) c[i] = outs[(size_t)src_[i]] + (uint64_t)n0_[i] * esz;
+        const bool by_value = slices() <= 16 && ((rows == 1 && host_lists_) || rows > 8);
+        if (by_value) {
+            const int rc = berth_ops_mgemm_hostlists(a.raw(), b_.data(), (void*)(uintptr_t)outs[0], suh_.data(), a_had_.raw(),
+                                                     svh_.data(), rows, size_k_, width_, k_bits_, (int)codebook_, (int)out, 1,
+                                                     slices(), size_n_.data(), c.data(), stride_.data(), src_.data(),
+                                                     (int)sources_.size(), gpu.raw_stream());
+            if (rc > 0) return;
+            const std::string err = berth_ops_last_error();
+            if (rows > 1 || err.find("host lists") == std::string::npos) throw KernelError(err);
+            host_lists_ = false;                                // too small for the streaming kernel: device lists from now on
+        }
+        if (c != c_host_) {
+            gpu.synchronize();                                  // a launch in flight may still read the old list
+            d_c_ = DeviceBuffer<uint64_t>::from_host(gpu, c);
+            gpu.synchronize();
+            c_host_ = c;
+        }
+        if (berth_ops_mgemm(a.raw(), d_b_.raw(), (void*)(uintptr_t)outs[0], d_suh_.raw(), a_had_.raw(), d_svh_.raw(), rows,
+                            size_k_, width_, k_bits_, (int)codebook_, (int)out, 1, slices(), (const int*)d_size_n_.raw(),
+                            d_c_.raw(), (const int*)d_stride_.raw(), (const int*)d_src_.raw(), (int)sources_.size(),
+                            gpu.raw_stream()) <= 0)
+            throw KernelError(berth_ops_last_error());
+    }
+
+private:
+    std::vector<const Exl3Linear*> sources_;
+    int size_k_ = 0, k_bits_ = 0, width_ = 0;
+    Codebook codebook_ = Codebook::Mul1;
+    std::vector<uint64_t> b_, svh_, suh_, c_host_;
+    std::vector<int> stride_, src_, n0_, size_n_;
+    DeviceBuffer<uint64_t> d_b_, d_svh_, d_suh_, d_c_;
+    DeviceBuffer<int> d_stride_, d_src_, d_size_n_;
+    DeviceBuffer<Half> a_had_;
+    bool host_lists_ = true;
+};
+
 // gate -> up -> silu_mul -> down (mlp.rs:118-150 decode, :219-303 prefill)
 class MlpLayer {
 public:

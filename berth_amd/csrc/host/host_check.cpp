@@ -101,6 +101,39 @@ static int run_linear(const Gpu& gpu, const std::string& dir)
     return 0;
 }
 
+// meta: K rows fp32 N_0 N_1 ...; sources src0, src1, ...; outputs y0.bin, y1.bin, ...
+static int run_bundle(const Gpu& gpu, const std::string& dir)
+{
+    const auto m = read_meta(dir);
+    const int K = (int)m.at(0), rows = (int)m.at(1);
+    const OutDtype out = m.at(2) ? OutDtype::F32 : OutDtype::F16;
+    std::vector<Exl3Linear> lins;
+    for (size_t i = 3; i < m.size(); ++i) lins.push_back(load_linear(gpu, dir, "src" + std::to_string(i - 3), K, (int)m[i]));
+    std::vector<const Exl3Linear*> sources;
+    for (const Exl3Linear& l : lins) sources.push_back(&l);
+    MultiLinear multi(gpu, sources);
+    const auto x = DeviceBuffer<Half>::from_host(gpu, read_file<Half>(dir + "/x.bin"));
+    std::vector<DeviceBuffer<uint8_t>> ys;
+    std::vector<uint64_t> outs;
+    for (const Exl3Linear& l : lins) {
+        ys.push_back(DeviceBuffer<uint8_t>::zeroed(gpu, (size_t)rows * l.size_n() * out_bytes(out)));
+        outs.push_back(ys.back().ptr());
+    }
+    bool refused = false;
+    try {
+        multi.forward(gpu, x, {outs[0]}, rows, out);            // one output for several sources
+    } catch (const InputError&) {
+        refused = true;
+    }
+    if (!refused && lins.size() > 1) throw std::runtime_error("a short output list was not refused");
+    multi.forward(gpu, x, outs, rows, out);
+    multi.forward(gpu, x, outs, rows, out);                     // the second call finds its lists in place
+    gpu.synchronize();
+    for (size_t i = 0; i < ys.size(); ++i) write_file(dir + "/y" + std::to_string(i) + ".bin", ys[i].copy_to_host());
+    std::printf("bundle ok rows=%d slices=%d width=%d launch=%s\n", rows, multi.slices(), multi.width(), berth_ops_last_launch());
+    return 0;
+}
+
 static int run_mlp(const Gpu& gpu, const std::string& dir)
 {
     const auto m = read_meta(dir);
@@ -264,6 +297,7 @@ int main(int argc, char** argv)
         if (what == "ckpt-mlp" && argc >= 5) return run_ckpt_mlp(gpu, dir, (uint32_t)std::stoul(argv[3]), argv[4]);
         if (what == "ckpt-moe" && argc >= 5) return run_ckpt_moe(gpu, dir, (uint32_t)std::stoul(argv[3]), argv[4]);
         if (what == "linear") return run_linear(gpu, dir);
+        if (what == "bundle") return run_bundle(gpu, dir);
         if (what == "mlp") return run_mlp(gpu, dir);
         if (what == "moe") return run_moe(gpu, dir);
         std::fprintf(stderr, "unknown case %s\n", what.c_str());

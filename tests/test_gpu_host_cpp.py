@@ -1,5 +1,5 @@
 """The C++ host layer (berth_amd/csrc/host/engine.hpp: Gpu, DeviceBuffer, Exl3Linear,
-RowScratch, MlpLayer, MoeLayer over the two C ABIs) driven through its check
+RowScratch, MultiLinear, MlpLayer, MoeLayer over the two C ABIs) driven through its check
 program on case files, results compared with the CPU oracle.  This is also the
 functional test of the device-runtime library (contexts, streams, events,
 buffers, copies)."""
@@ -46,6 +46,25 @@ def test_cpp_linear(tmp_path, rows, fp32, use_rows):
     y = np.fromfile(tmp_path / "y.bin", dtype=np.float32 if fp32 else np.float16).reshape(rows, N)
     want, _ = O.linear(x, *lin, Kk, N, bits, 2, out_fp32=bool(fp32))
     assert close(y, want.reshape(rows, N))[0] == 0
+
+
+@pytest.mark.parametrize("rows,fp32", [(1, 0), (4, 1), (20, 0), (150, 1)])
+def test_cpp_bundle(tmp_path, rows, fp32):
+    """MultiLinear: three linears on one input as one sliced berth_ops_mgemm, every row-count
+    route (one row, 2..8 rows from the device lists, more than 8 rows on the MFMA kernels)."""
+    Kk, Ns, bits = 256, (768, 256, 512), 4
+    lins = [synth.linear(4500 + rows + i, Kk, n, bits) for i, n in enumerate(Ns)]
+    x = synth.activations(4600 + rows, rows, Kk)
+    for i, lin in enumerate(lins):
+        _write_linear(tmp_path, f"src{i}", lin)
+    x.view(np.uint16).tofile(tmp_path / "x.bin")
+    (tmp_path / "meta.txt").write_text(f"{Kk} {rows} {fp32} " + " ".join(str(n) for n in Ns) + "\n")
+    out = _run("bundle", tmp_path)
+    assert "bundle ok" in out and "slices=6 width=256" in out and "sliced x6" in out, out
+    for i, lin in enumerate(lins):
+        y = np.fromfile(tmp_path / f"y{i}.bin", dtype=np.float32 if fp32 else np.float16).reshape(rows, Ns[i])
+        want, _ = O.linear(x, *lin, Kk, Ns[i], bits, 2, out_fp32=bool(fp32))
+        assert close(y, want.reshape(rows, Ns[i]))[0] == 0, i
 
 
 @pytest.mark.parametrize("rows", [1, 24])
