@@ -595,13 +595,23 @@ extern "C" int berth_exl3_mlp(const void* x, const berth_exl3_lin* lins, void* g
             g_exl3_launch = desc + " ; " + launch_gemv(down);
             return 0;
         }
-        LinearArgs up = gate;
-        up.trellis = lins[1].trellis;
-        up.suh = lins[1].suh;
-        up.svh = lins[1].svh;
-        up.c = up_out;
-        std::string desc = launch_gemm(gate);
-        desc += " ; " + launch_gemm(up);
+        std::string desc;
+        if (intermediate >= hidden) {
+            // gate and up as one bundle: one launch rotates the input with either linear's scales (the
+            // up projection's copy waits in act_had, which the down projection fills only afterwards),
+            // one dense launch runs both
+            PairArgs pair{x, {lins[0].trellis, lins[1].trellis}, {lins[0].suh, lins[1].suh}, {lins[0].svh, lins[1].svh},
+                          {gate_out, up_out}, a_had, size_m, hidden, intermediate, k_bits, codebook, st};
+            desc = launch_gemm_pair(pair, act_had);
+        } else {
+            LinearArgs up = gate;
+            up.trellis = lins[1].trellis;
+            up.suh = lins[1].suh;
+            up.svh = lins[1].svh;
+            up.c = up_out;
+            desc = launch_gemm(gate);
+            desc += " ; " + launch_gemm(up);
+        }
         desc += " ; " + launch_silu_mul(gate_out, up_out, up_out, (int64_t)size_m * intermediate, 0.0f, st);
         g_exl3_launch = desc + " ; " + launch_gemm(down);
         return 0;

@@ -56,6 +56,7 @@ __global__ __launch_bounds__(256) void had_r_128_kernel(const T* __restrict__ in
 // from a device list of pointers or from the pointers passed by value.
 struct SuhTable {
     const _Float16* suh[kBundleMaxSlices];
+    _Float16* out[kBundleMaxSlices];        // null: slab s goes to out + s * out_stride
 };
 __global__ __launch_bounds__(256) void had_r_128_slabs_kernel(const _Float16* __restrict__ in, size_t in_stride,
                                                               _Float16* __restrict__ out, size_t out_stride,
@@ -65,7 +66,7 @@ __global__ __launch_bounds__(256) void had_r_128_slabs_kernel(const _Float16* __
     const int slab = blockIdx.y;
     const _Float16* scale = suh_list ? (const _Float16*)suh_list[slab] : tab.suh[slab];
     in += (size_t)slab * in_stride;
-    out += (size_t)slab * out_stride;
+    out = (!suh_list && tab.out[slab]) ? tab.out[slab] : out + (size_t)slab * out_stride;
     const int lane = threadIdx.x & 63;
     const int l16 = lane & 15;
     const long waves = (long)gridDim.x * 4;
@@ -90,13 +91,17 @@ __global__ __launch_bounds__(256) void had_r_128_slabs_kernel(const _Float16* __
 }
 
 std::string launch_had_r_128_slabs(const void* in, size_t in_stride, void* out, size_t out_stride, const void* suh_list,
-                                   const void* const* suh_host, int slabs, int rows, int cols, hipStream_t stream)
+                                   const void* const* suh_host, int slabs, int rows, int cols, hipStream_t stream,
+                                   void* const* out_host)
 {
     if (slabs < 1 || slabs > 65535) throw std::runtime_error("had_r_128 slabs: between 1 and 65535 slabs");
     SuhTable tab{};
     if (!suh_list) {
         if (slabs > kBundleMaxSlices) throw std::runtime_error("had_r_128 slabs: too many slabs for the by-value table");
-        for (int i = 0; i < slabs; ++i) tab.suh[i] = (const _Float16*)suh_host[i];
+        for (int i = 0; i < slabs; ++i) {
+            tab.suh[i] = (const _Float16*)suh_host[i];
+            tab.out[i] = out_host ? (_Float16*)out_host[i] : nullptr;
+        }
     }
     const int col_blocks = cols / 128;
     const long blocks = (long)rows * col_blocks;

@@ -185,12 +185,12 @@ std::string launch_gemm_bundle(const MgemmArgs& m)
                 g.c = (void*)((const uint64_t*)m.c_ptrs)[i];
                 g.width = m.size_n_list[i];
                 g.n_stride = m.n_stride_list[i];
-                g.had_slab = src;
+                g.a_had = (const _Float16*)m.a_had + (size_t)src * slab_stride;
             } else {
                 g.c = (char*)m.c + (size_t)i * m.size_m * m.size_n * (m.c_fp32 ? 4 : 2);
                 g.width = m.size_n;
                 g.n_stride = m.size_n;
-                g.had_slab = i;
+                g.a_had = (const _Float16*)m.a_had + (size_t)i * slab_stride;
             }
         }
     } else {
@@ -212,6 +212,42 @@ std::string launch_gemm_bundle(const MgemmArgs& m)
     dispatch_dense(ws, p, m.k_bits, m.codebook, m.size_m, m.size_k, (int)nblocks, m.stream, desc);
     return std::string(sliced ? "sliced x" : "uniform x") + std::to_string(m.bszm_out) + (m.host_lists ? " by value " : " ") + d0 +
            " + " + desc + (m.c_fp32 ? " out=f32" : " out=f16");
+}
+
+std::string launch_gemm_pair(const PairArgs& a, void* a_had_second)
+{
+    if (a.size_k % 128 != 0) throw std::runtime_error("exl3 linear: size_k must be a multiple of 128");
+    LaunchScope scope(a.stream);
+    Workspace& ws = scope.ws;
+    throw_pending_device_fault(ws);
+    GemmParams p{};
+    p.fault = ws.fault_dev;
+    p.spin_limit = spin_limit();
+    p.a_had[0] = (const _Float16*)a.a_had;
+    p.c[0] = a.c[0];
+    p.M = a.size_m;
+    p.K = a.size_k;
+    p.N = a.size_n;
+    p.out_fp32 = 0;
+    p.partials = ws.partials;
+    p.counters = ws.counters;
+    p.num_slices = 2;
+    void* const slabs[2] = {a.a_had, a_had_second};
+    for (int i = 0; i < 2; ++i) {
+        GemmSlice& g = p.slice[i];
+        g.trellis = (const uint32_t*)a.trellis[i];
+        g.svh = (const _Float16*)a.svh[i];
+        g.c = a.c[i];
+        g.width = a.size_n;
+        g.n_stride = a.size_n;
+        g.a_had = (const _Float16*)slabs[i];
+    }
+    std::string d0 = launch_had_r_128_slabs(a.a, 0, a.a_had, 0, nullptr, a.suh, 2, a.size_m, a.size_k, a.stream, slabs);
+    const long nblocks = 2L * ((a.size_n + 255) / 256);
+    if (nblocks * ((a.size_m + 31) / 32) > kCounters / 2) throw std::runtime_error("exl3 linear pair: too many output tiles");
+    std::string desc;
+    dispatch_dense(ws, p, a.k_bits, a.codebook, a.size_m, a.size_k, (int)nblocks, a.stream, desc);
+    return "pair " + d0 + " + " + desc + " out=f16";
 }
 
 // grouped: problems of at most 32 * g.mb rows each; a_had rows are in problem order

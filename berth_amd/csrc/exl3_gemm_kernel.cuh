@@ -38,7 +38,7 @@ struct GemmSlice {
     int width;                  // columns of this linear (a multiple of 128, at most N)
     int n_stride;               // columns of the whole weight the slice is cut from: elements between
                                 // output rows and, in tiles of 16, between the tile rows of its trellis
-    int had_slab;               // which rotated copy of the input it multiplies
+    const _Float16* a_had;      // the rotated copy of the input it multiplies, [M][K]
 };
 constexpr int kGemmMaxSlices = 16;
 
@@ -82,8 +82,8 @@ struct GemmParams {
     // ceil(N / 256) column blocks of the launch (N = the widest slice); a block past the end of
     // a narrower slice is empty.  The slice's tensors come from the device lists when b_list is
     // set (uniform mode: c_ptrs null, outputs [slice][M][N] behind c[0], rotated input = slab
-    // `slice`; sliced mode: all seven lists), else from `slice` by value.  a_had[0] holds the
-    // rotated inputs, slab_stride elements apart.
+    // `slice`; sliced mode: all seven lists; a_had[0] holds the rotated inputs, slab_stride
+    // elements apart), else from `slice` by value.
     int num_slices;             // 0: one linear (lin, c[0], a_had[0])
     size_t slab_stride;
     const uint64_t* b_list;
@@ -119,8 +119,8 @@ __device__ __forceinline__ TileView dense_tile_view(const GemmParams& p, const i
         const int per = (p.N + 255) >> 8;
         const int sl = nblk / per;
         v.nblk = nblk - sl * per;
-        int slab = sl;
         if (p.b_list) {
+            int slab = sl;
             v.lin.trellis = (const uint32_t*)p.b_list[sl];
             v.lin.svh = (const _Float16*)p.svh_list[sl];
             if (p.c_ptrs) {
@@ -131,6 +131,7 @@ __device__ __forceinline__ TileView dense_tile_view(const GemmParams& p, const i
             } else {
                 v.cout = (char*)p.c[0] + (size_t)sl * p.M * p.N * (p.out_fp32 ? 4 : 2);
             }
+            v.a_had = p.a_had[0] + (size_t)slab * p.slab_stride;
         } else {
             const GemmSlice& g = p.slice[sl];
             v.lin.trellis = g.trellis;
@@ -138,9 +139,8 @@ __device__ __forceinline__ TileView dense_tile_view(const GemmParams& p, const i
             v.cout = g.c;
             v.N = g.width;
             v.ldc = g.n_stride;
-            slab = g.had_slab;
+            v.a_had = g.a_had;
         }
-        v.a_had = p.a_had[0] + (size_t)slab * p.slab_stride;
         v.empty = v.nblk * 256 >= v.N;
     }
     return v;

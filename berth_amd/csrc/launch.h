@@ -239,9 +239,14 @@ std::string launch_mgemm(const MgemmArgs& args);
 // more than 8 rows: the bundle as one dense MFMA launch
 std::string launch_gemm_bundle(const MgemmArgs& args);
 // out slab s = Hh(in(s) * suh(s)) for s < slabs (fp16; in(s) = in + s * in_stride, out slabs
-// out_stride elements apart); suh(s) from the device list, or from the host array when the list is null
+// out_stride elements apart, or at out_host[s] when that is given with a null list); suh(s) from
+// the device list, or from the host array when the list is null
 std::string launch_had_r_128_slabs(const void* in, size_t in_stride, void* out, size_t out_stride, const void* suh_list,
-                                   const void* const* suh_host, int slabs, int rows, int cols, hipStream_t stream);
+                                   const void* const* suh_host, int slabs, int rows, int cols, hipStream_t stream,
+                                   void* const* out_host = nullptr);
+// gate and up of an MLP above 8 rows as one bundle: two linears of one shape on one input, each
+// with its own output and its own buffer for the rotated input
+std::string launch_gemm_pair(const PairArgs& pair, void* a_had_second);
 constexpr int kBundleMaxSlices = 16;    // slices of a bundle whose lists travel by value
 
 // rows 1..8: VALU dot-product kernel.  Returns the launch description.  `scratch`: the

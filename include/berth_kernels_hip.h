@@ -261,8 +261,11 @@ typedef struct {
  * output) in one entry.  Up to 8 rows run as two launches: gate and up share one
  * launch and the rotated input, and the down projection evaluates silu(g) * u
  * while it rotates its input (same fp16 steps as berth_ops_silu_mul, so the
- * activation is bit-identical to the unfused sequence).  More rows run the
- * unfused sequence on the MFMA kernel.
+ * activation is bit-identical to the unfused sequence).  More rows run on the MFMA
+ * kernels: gate and up as one bundle (one launch rotates the input with either
+ * linear's scales, one dense launch runs both; the up projection's rotated copy
+ * waits in act_had, so this form needs intermediate >= hidden, else gate and up run
+ * one after the other), berth_ops_silu_mul, the down projection.
  * lins: HOST array {gate, up, down} of device pointers.  x fp16 [m][hidden];
  * gate_out, up_out fp16 [m][intermediate] (written; above 8 rows up_out ends up
  * holding the activation); a_had fp16 [m][hidden] and act_had fp16

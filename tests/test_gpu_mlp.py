@@ -32,6 +32,9 @@ def test_fused_mlp_stage_by_stage(rows, H, I, bits):
     launch = run_mlp_block(rows, H, I, bits)
     if rows <= 8:
         assert launch.count("exl3_gemv_kernel") == 2 and "pair" in launch and ",silu>" in launch
+    elif I >= H:
+        # gate and up as one bundle (one rotation launch, one dense launch), then the down projection
+        assert launch.count("exl3_gemm_kernel") == 2 and "had_r_128_slabs_kernel" in launch and "silu_mul" in launch
     else:
         assert launch.count("exl3_gemm_kernel") == 3 and "silu_mul" in launch
 
@@ -50,9 +53,11 @@ def run_mlp_block(rows, H, I, bits):
     u_want, _ = O.linear(x, *up, H, I, bits, 2)
     g_got = host_f16(mlp.g)[:rows * I].reshape(rows, I)
     assert close(g_got, g_want.reshape(rows, I))[0] == 0
-    if rows <= 8:
-        # the rotated input is the gate's (its suh); above 8 rows the up projection rewrites it with its own
+    if rows <= 8 or I >= H:
+        # the rotated input is the gate's (its suh); above 8 rows with intermediate < hidden the up
+        # projection, a launch of its own then, rewrites it with its own
         assert np.array_equal(host_u16(mlp.x_had)[:rows * H], xh_want.view(np.uint16).ravel())
+    if rows <= 8:
         u_got = host_f16(mlp.u)[:rows * I].reshape(rows, I)
         assert close(u_got, u_want.reshape(rows, I))[0] == 0
         act = O.silu_mul(g_got, u_got).reshape(rows, I)            # from the GPU's own gate / up outputs
