@@ -295,14 +295,14 @@ def test_gemm_split_k(m, Kk, N):
     assert np.array_equal(got.view(np.uint32), got2.view(np.uint32))
 
 
-def _check_balanced(m, Kk, N, fp32, tile, bits=4):
-    got, want, ah, want_ah, launch = _run_linear(m, Kk, N, bits, 2, fp32, 700 + m, prefill=True)
+def _check_balanced(m, Kk, N, fp32, tile, bits=4, cb=2):
+    got, want, ah, want_ah, launch = _run_linear(m, Kk, N, bits, cb, fp32, 700 + m, prefill=True)
     name = "exl3_gemm_wide_kernel" if tile == 256 else "exl3_gemm_balanced_kernel"
-    assert f"{name}<{bits},2,{tile}x256>" in launch, launch
+    assert f"{name}<{bits},{cb},{tile}x256>" in launch, launch
     assert np.array_equal(ah, want_ah)
     bad, worst = close(got, want)
     assert bad == 0, (bad, worst, launch)
-    got2, _, _, _, _ = _run_linear(m, Kk, N, bits, 2, fp32, 700 + m, prefill=True)
+    got2, _, _, _, _ = _run_linear(m, Kk, N, bits, cb, fp32, 700 + m, prefill=True)
     assert np.array_equal(got.view(np.uint16), got2.view(np.uint16))
 
 
@@ -320,6 +320,28 @@ def test_gemm_256_row_tiles_dealt_out_evenly(m, Kk, N, fp32, bits):
     of eight waves; every weight is decoded once per tile and reaches the MFMA waves through
     LDS.  Dealt out the same way.  The last row tile may be short (44 or 128 rows)."""
     _check_balanced(m, Kk, N, fp32, 256, bits)
+
+
+@pytest.mark.parametrize("m,Kk,N,tile,bits,cb", [(128, 512, 16384, 128, 2, 2), (96, 384, 16640, 128, 3, 2),
+                                                 (128, 256, 16384, 128, 5, 2), (70, 256, 16384, 128, 6, 2),
+                                                 (128, 384, 16384, 128, 4, 0), (100, 256, 16640, 128, 4, 1),
+                                                 (128, 256, 16384, 128, 8, 2), (512, 384, 16384, 256, 2, 2),
+                                                 (300, 256, 16640, 256, 5, 2), (512, 256, 16384, 256, 4, 1),
+                                                 (260, 256, 16384, 256, 6, 0)])
+def test_gemm_pipelined_tiles_other_rates_and_codebooks(m, Kk, N, tile, bits, cb):
+    """The 128- and 256-row loops issue the decode of the next half-step (128 rows) or macro-step
+    (256 rows) behind the MFMAs of the current one; the scheduling groups that hold that order
+    are sized for 4 bpw with the mul1 codebook.  Every other bit rate and both other codebooks
+    through the same loops: same results as the oracle, same bits on a second run."""
+    _check_balanced(m, Kk, N, bool(bits & 1), tile, bits, cb)
+
+
+@pytest.mark.parametrize("m,Kk,N,tile", [(1280, 384, 16640, 256), (1024, 256, 16384, 256), (2048, 128, 16384, 256)])
+def test_gemm_ranges_that_run_through_whole_tiles(m, Kk, N, tile):
+    """More (tile, k-block) units per workgroup than a tile has k-blocks: a workgroup's range
+    covers the end of one tile, whole tiles (finished without any hand-over) and the start of
+    another; with exactly one tile per workgroup nothing is shared at all."""
+    _check_balanced(m, Kk, N, False, tile)
 
 
 def test_gemm_256_row_tiles_on_narrow_outputs():
