@@ -1051,6 +1051,18 @@ extern "C" int berth_moe_workspace_offsets(int T, int H, int E, int k, int I, in
     return 0;
 }
 
+// the always-on expert's own intermediates when its width differs from the routed experts'
+// (it is then no row of the grouped launches): {gate fp16 [T][shared_I], up fp16 [T][shared_I]};
+// above 8 rows the second one ends up holding silu(gate) * up
+extern "C" int berth_moe_workspace_shared_offsets(int T, int H, int E, int k, int I, int shared_I, size_t out[2])
+{
+    if (T < 1 || H < 1 || E < 1 || k < 1 || I < 1 || shared_I < 1 || shared_I == I || !out) return -1;
+    const MoeLayout L = moe_layout(T, H, E, k, I, shared_I);
+    out[0] = L.sg;
+    out[1] = L.su;
+    return 0;
+}
+
 extern "C" int berth_moe_route(const void* x, const void* wr, const float* bias, int32_t* idx, float* w,
                                float* logits, void* parts_scratch, int T, int H, int E, int k,
                                int renorm, void* stream)

@@ -91,6 +91,7 @@ def load() -> C.CDLL:
         L.berth_moe_workspace_bytes.argtypes = [ci] * 6
         L.berth_moe_workspace_bytes.restype = C.c_size_t
         L.berth_moe_workspace_offsets.argtypes = [ci] * 6 + [C.POINTER(C.c_size_t)]
+        L.berth_moe_workspace_shared_offsets.argtypes = [ci] * 6 + [C.POINTER(C.c_size_t)]
         L.berth_moe_last_error.restype = C.c_char_p
         L.berth_moe_last_launch.restype = C.c_char_p
         L.berth_kernels_workspace.argtypes = [C.POINTER(vp), C.POINTER(C.c_size_t), C.POINTER(vp), C.POINTER(ci)]
@@ -404,6 +405,14 @@ class moe:
             raise LaunchError("moe: sizes must be positive")
         names = ("idx", "w", "offsets", "perm", "inv", "gate_out", "up_out", "slot_out", "shared_out")
         return dict(zip(names, (int(v) for v in out)))
+
+    @staticmethod
+    def workspace_shared_offsets(T, H, E, k, I, shared_I) -> dict:
+        """The always-on expert's own gate / up outputs when shared_I != I."""
+        out = (C.c_size_t * 2)()
+        if load().berth_moe_workspace_shared_offsets(T, H, E, k, I, shared_I, out) != 0:
+            raise LaunchError("moe: no separate buffers for the shared expert at these sizes")
+        return {"shared_gate_out": int(out[0]), "shared_up_out": int(out[1])}
 
     @staticmethod
     def layer(x, wr, bias, experts_dev, shared_host, out, idx_out, w_out, workspace, workspace_bytes,

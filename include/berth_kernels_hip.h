@@ -354,6 +354,10 @@ size_t berth_moe_workspace_bytes(int T, int H, int E, int k, int I, int shared_I
  * fp16 [T*k][I], up_out fp16 [T*k][I], slot_out fp32 [T*k][H] (rows in expert-
  * sorted order), shared_out fp32 [T][H]}, valid after berth_moe_layer returns */
 int berth_moe_workspace_offsets(int T, int H, int E, int k, int I, int shared_I, size_t out[9]);
+/* the always-on expert's own gate and up outputs, fp16 [T][shared_I] each, when shared_I != I
+ * (with shared_I == I they are rows T*k .. of gate_out / up_out); above 8 rows the second one
+ * ends up holding silu(gate) * up.  -1 when there is no such buffer. */
+int berth_moe_workspace_shared_offsets(int T, int H, int E, int k, int I, int shared_I, size_t out[2]);
 const char* berth_moe_last_error(void);
 const char* berth_moe_last_launch(void);
 
