@@ -27,11 +27,16 @@ static void gemm_bits(const GemmParams& p, int bits, int cb, int mb, hipStream_t
 }
 
 // split-K factor for `tiles` output tiles of MB*32 x 256: one workgroup per compute unit
-// (a second resident workgroup adds nothing once the whole chip is busy, and fewer
-// workgroups share a tile), at least two k-blocks per workgroup, inside the workspace
-static int gemm_split(const Workspace& ws, long tiles, int KB, int mb)
+// (fewer workgroups share a tile); two for a dense launch of at most 32 rows with at least a
+// quarter as many tiles as compute units (a workgroup of four waves leaves a compute unit's
+// vector pipes half idle, and each workgroup still keeps several k-blocks: the 27B gate + up
+// bundle at 16 rows 63 -> 54 us; with few tiles the extra hand-overs cost more than that, q/k/v
+// 24 -> 30 us, and with several row tiles nothing is gained: k at 512 rows 34.9 -> 36.0 us),
+// at least two k-blocks per workgroup, inside the workspace
+static int gemm_split(const Workspace& ws, long tiles, int KB, int mb, bool one_row_tile = false)
 {
-    const int per_cu = knobs().gemm_wg_per_cu > 0 ? knobs().gemm_wg_per_cu : 1;
+    const int per_cu = knobs().gemm_wg_per_cu > 0 ? knobs().gemm_wg_per_cu
+                                                  : (mb == 1 && one_row_tile && tiles * 4 >= ws.cu_count ? 2 : 1);
     long S = ((long)ws.cu_count * per_cu + tiles - 1) / tiles;
     if (S > KB / 2) S = KB / 2;
     if (S < 1) S = 1;
@@ -109,7 +114,7 @@ static void dispatch_dense(const Workspace& ws, GemmParams& p, int k_bits, int c
         const long tiles = (long)nblocks * mtiles;
         p.tiles_y = mtiles;
         p.units = 0;
-        p.S = gemm_split(ws, tiles, KB, mb_plain);
+        p.S = gemm_split(ws, tiles, KB, mb_plain, size_m <= 32);
         gemm_bits(p, k_bits, codebook, mb_plain, stream, desc, dim3((unsigned)(tiles * p.S), 1, 1));
     }
     hip_ok(hipGetLastError(), "exl3_gemm_kernel launch");
