@@ -30,6 +30,8 @@
 
 namespace berth {
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
 // one linear of a bundle whose lists the host knows
 struct GemmSlice {
     const uint32_t* trellis;
@@ -306,15 +308,16 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
         // has no branch.  The order is given to the scheduler as groups after each half-step.
         constexpr int kAPasses = BM * 8 / 256;
         uint32_t ring[4][BITS];
-        uint4 a_nxt[kAPasses][2];
+        u32x4_t a_nxt[kAPasses][2];
         const int a_row = threadIdx.x >> 3, a_ch = threadIdx.x & 7;       // + 32 rows per pass
         auto load_a = [&](int kb) {
     #pragma unroll
             for (int ps = 0; ps < kAPasses; ++ps) {
                 const int r = a_row + 32 * ps;
-                uint4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
+                u32x4_t v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
                 if (m0 + r < m_end) {
-                    const uint4* src = (const uint4*)(a_had + (size_t)(m0 + r) * p.K + kb * 128 + a_ch * 16);
+                    const global_ptr<const u32x4_t> src =
+                        (global_ptr<const u32x4_t>)(as_global(a_had) + (size_t)(m0 + r) * p.K + kb * 128 + a_ch * 16);
                     v0 = src[0];
                     v1 = src[1];
                 }
@@ -323,7 +326,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
             }
         };
         auto load_b_step = [&](int kb, int st) {
-            const uint32_t* nb = tbase + (size_t)(kb * 8 + 2 * st) * row_dw;
+            const global_ptr<const uint32_t> nb = as_global(tbase) + (size_t)(kb * 8 + 2 * st) * row_dw;
     #pragma unroll
             for (int j = 0; j < BITS; ++j) ring[st][j] = nb[j];
         };
@@ -354,7 +357,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int tile_y,
             _Float16* a_buf = a_tile + (size_t)buf * BM * kAStride;
     #pragma unroll
             for (int ps = 0; ps < kAPasses; ++ps) {
-                uint4* dst = (uint4*)(a_buf + (a_row + 32 * ps) * kAStride + a_ch * 16);
+                u32x4_t* dst = (u32x4_t*)(a_buf + (a_row + 32 * ps) * kAStride + a_ch * 16);
                 dst[0] = a_nxt[ps][0];
                 dst[1] = a_nxt[ps][1];
             }
@@ -683,11 +686,25 @@ __global__ __launch_bounds__(256, 2) void exl3_gemm_balanced_kernel(GemmParams p
     const int KB = p.K >> 7;
     const int w = die_major_index((int)blockIdx.x, (int)gridDim.x);
     const int u_end = range_start(p, w + 1);
-    for (int u = range_start(p, w); u < u_end;) {
+    int u = range_start(p, w);
+    // the first two segments are written out (as the body of a loop the compiler's scheduler does
+    // not reliably keep the interleaved order of the main loop); the loop takes the rest
+    {
         const int stop = min(u_end, (u / KB + 1) * KB);
         gemm_segment<BITS, CB, MB>(p, w, u, stop, smem);
         u = stop;
-        if (u < u_end) __syncthreads();                         // the epilogue's LDS tile is the next A tile
+    }
+    if (u < u_end) {
+        __syncthreads();                                        // the epilogue's LDS tile is the next A tile
+        const int stop = min(u_end, (u / KB + 1) * KB);
+        gemm_segment<BITS, CB, MB>(p, w, u, stop, smem);
+        u = stop;
+    }
+    while (u < u_end) {
+        __syncthreads();
+        const int stop = min(u_end, (u / KB + 1) * KB);
+        gemm_segment<BITS, CB, MB>(p, w, u, stop, smem);
+        u = stop;
     }
 }
 

@@ -14,13 +14,13 @@
 //            32 MFMAs per macro-step, A and B operands from LDS.
 //
 // A and B tiles are double-buffered; per macro-step one barrier.  Inside a macro-step a wave
-// issues its 32 MFMAs on the current buffers two at a time and, behind every two, one
-// sixteenth of its decode for the next macro-step (a pair of weights), so the vector pipe
-// works while the matrix pipe is busy: the order is given to the scheduler as groups
-// (operand reads one chunk ahead, two MFMAs, eight vector instructions).  As two blocks
-// (all of the decode, then all of the MFMAs) the 27B gate projection at 512 rows took 141 us,
-// interleaved it takes 124.  Trellis registers run four macro-steps ahead of the decode, A
-// registers two.
+// issues its 32 MFMAs on the current buffers, every operand read one pair of MFMAs ahead, and
+// decodes its share of the next macro-step; the loop has no branch (row blocks past the end of
+// the rows are multiplied too and never stored).  Whether the decode is issued in sixteenths
+// between the MFMAs or as one block behind them makes no difference here (the other wave of
+// the SIMD fills either gap): the 27B gate projection at 512 rows takes 124-130 us both ways,
+// 141 with a branch around every row block's MFMAs and the decode ahead of them.  Trellis
+// registers run four macro-steps ahead of the decode, A registers two.
 //
 // Handoff between workgroups that share a tile and the epilogue are those of the
 // 128-row kernel (partial sums in register layout, summed in k order by the last
@@ -30,8 +30,6 @@
 #include "exl3_gemm_kernel.cuh"
 
 namespace berth {
-
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kWideAStride = 64 + 8;                    // halves per LDS row of the A tile (144 B)
 constexpr int kWideABytes = 256 * kWideAStride * 2;     // one A buffer: 36864
@@ -136,14 +134,11 @@ __device__ __forceinline__ void gemm_tile_wide(const GemmParams& p, const int ti
 #pragma unroll
             for (int i = 0; i < 4; ++i) *(u32x4_t*)(ad + i * 16) = ar[i];
         };
-        // One macro-step: the 32 MFMAs on buffer `buf`, and behind every two of them one
-        // sixteenth of the decode of the next macro-step (a pair of weights: two windows, two
-        // hashes, one packed fma).  Written in that order here; the scheduler groups after the
-        // call keep the compiler from collecting the MFMAs and the decode back into two blocks.
-        // Operands of the next two MFMAs are read one chunk ahead; the A rows of the next
-        // macro-step go to LDS in the first four chunks, the decoded weights at the end.  Row
-        // blocks past the end of the rows are multiplied too (their A rows repeat the last row)
-        // and never stored: the loop has no branch.
+        // One macro-step: the 32 MFMAs on buffer `buf` (operands of the next two MFMAs read one
+        // pair ahead) and the decode of the next macro-step into the other buffers; the A rows of
+        // the next macro-step go to LDS with the first four pairs, the decoded weights at the end.
+        // Row blocks past the end of the rows are multiplied too (their A rows repeat the last
+        // row) and never stored: the loop has no branch.
         auto fused_step = [&](int buf, const uint32_t (&tr)[BITS], const u32x4_t (&ar)[4]) {
             const unsigned char* ao = a_op + (size_t)buf * kWideABytes;
             const unsigned char* bo = b_op + (size_t)buf * kWideBBytes;
@@ -199,29 +194,9 @@ __device__ __forceinline__ void gemm_tile_wide(const GemmParams& p, const int ti
             for (int u = 0; u < 4; ++u) {
                 if (s + u >= nsteps) break;                         // workgroup-uniform
                 const int buf = u & 1;
-                __builtin_amdgcn_sched_barrier(0);
                 fused_step(buf, tr_ring[(u + 1) & 3], a_ring[(u + 1) & 1]);
                 issue_tr(s + u + 5, tr_ring[(u + 1) & 3]);
                 issue_a(s + u + 3, a_ring[(u + 1) & 1]);
-                // the order the scheduler has to keep: operand reads one chunk ahead, two MFMAs,
-                // a sixteenth of the decode
-                __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
-#define BERTH_WIDE_CHUNK(reads)                                                    \
-    __builtin_amdgcn_sched_group_barrier(0x100, reads, 0);                         \
-    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                             \
-    __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
-#define BERTH_WIDE_CHUNK_A(reads)                                                  \
-    BERTH_WIDE_CHUNK(reads)                                                        \
-    __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-                BERTH_WIDE_CHUNK_A(1) BERTH_WIDE_CHUNK_A(1) BERTH_WIDE_CHUNK_A(1) BERTH_WIDE_CHUNK_A(3)
-                BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(3)
-                BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(3)
-                BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(1) BERTH_WIDE_CHUNK(1)
-                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-                __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
-#undef BERTH_WIDE_CHUNK_A
-#undef BERTH_WIDE_CHUNK
-                __builtin_amdgcn_sched_group_barrier(0x200, 4, 0);
                 __syncthreads();
             }
         }
@@ -390,6 +365,7 @@ __global__ __launch_bounds__(512, 1) void exl3_gemm_wide_kernel(GemmParams p)
     const int KB = p.K >> 7;
     const int w = die_major_index((int)blockIdx.x, (int)gridDim.x);
     const int u_end = range_start(p, w + 1);
+    // a range is the end of one tile, any whole tiles and the start of another
     for (int u = range_start(p, w); u < u_end;) {
         const int stop = min(u_end, (u / KB + 1) * KB);
         gemm_segment_wide<BITS, CB>(p, w, u, stop, smem);
